@@ -1,0 +1,154 @@
+"""ctypes front end of the C oracle (oracle/libomega_oracle.so).
+
+Test infrastructure only: imported by tests/, by the smoke check and by the benchmark's
+cpu_baseline leg; never by the shipped package.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libomega_oracle.so")
+
+
+def build(force=False):
+    """Compile the oracle with gcc (seconds)."""
+    if force or not os.path.exists(_SO):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"], stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+_f = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_i = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(_SO)
+        L.orc_stream_key.restype = C.c_uint64
+        L.orc_stream_key.argtypes = [C.c_uint64, C.c_uint64]
+        L.orc_fill_normal.argtypes = [_f, C.c_uint64, C.c_uint64, C.c_uint64, C.c_double, C.c_uint64]
+        L.orc_round_bf16.argtypes = [_f, C.c_uint64]
+        L.orc_gate.argtypes = [_f, _f, C.c_void_p, C.c_int, C.c_int, C.c_int, _f]
+        L.orc_softmax.argtypes = [_f, C.c_int, C.c_int, _f]
+        L.orc_topk.argtypes = [_f, C.c_int, C.c_int, C.c_int, C.c_int, _i, _f]
+        L.orc_dispatch.argtypes = [_i, C.c_int, C.c_int, C.c_int, _i, _i, _i, _i]
+        L.orc_gather.argtypes = [_f, _i, C.c_int, C.c_int, _f]
+        L.orc_swiglu_rows.argtypes = [_f, C.c_int, _f, _f, _f, C.c_int, C.c_int, C.c_int, _f, _f]
+        L.orc_combine.argtypes = [_f, _i, _f, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _f]
+        L.orc_moe_tokens.argtypes = [_f, _i, _f, _f, _f, _f] + [C.c_int] * 6 + [_i, C.c_int, _f]
+        L.orc_moe_forward.argtypes = [_f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8 + [_f, _f, _i, _f, _i, _i, _i, _i, _f]
+        L.orc_cpu_baseline_forward.restype = C.c_double
+        L.orc_cpu_baseline_forward.argtypes = [_f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8 + [_f]
+        L.orc_cpu_sgemm_tn.argtypes = [C.c_int, C.c_int, C.c_int, _f, C.c_int, _f, C.c_int, _f, C.c_int, C.c_int]
+        _lib = L
+    return _lib
+
+
+def _opt(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def fill_normal(n, seed, stream, std, first=0):
+    out = np.empty(int(n), np.float32)
+    lib().orc_fill_normal(out, int(n), int(seed), int(stream), float(std), int(first))
+    return out
+
+
+def round_bf16(a):
+    out = np.ascontiguousarray(a, np.float32).copy()
+    lib().orc_round_bf16(out.reshape(-1), out.size)
+    return out
+
+
+def gate(x, Wg, bg=None):
+    T, d = x.shape
+    E = Wg.shape[0]
+    out = np.empty((T, E), np.float32)
+    lib().orc_gate(x, Wg, _opt(bg), T, d, E, out)
+    return out
+
+
+def softmax(logits):
+    T, E = logits.shape
+    out = np.empty((T, E), np.float32)
+    lib().orc_softmax(np.ascontiguousarray(logits), T, E, out)
+    return out
+
+
+def topk(p, K, renorm):
+    T, E = p.shape
+    ids = np.empty((T, K), np.int32)
+    w = np.empty((T, K), np.float32)
+    lib().orc_topk(np.ascontiguousarray(p), T, E, K, int(renorm), ids, w)
+    return ids, w
+
+
+def dispatch(ids, E):
+    T, K = ids.shape
+    counts = np.empty(E, np.int32)
+    offsets = np.empty(E + 1, np.int32)
+    dst = np.empty(T * K, np.int32)
+    src_row = np.empty(T * K, np.int32)
+    lib().orc_dispatch(np.ascontiguousarray(ids), T, K, E, counts, offsets, dst, src_row)
+    return counts, offsets, dst, src_row
+
+
+def swiglu_rows(xg, W1, W3, W2, bf16=False):
+    rows, d = xg.shape
+    H = W1.shape[0]
+    y = np.empty((rows, d), np.float32)
+    lib().orc_swiglu_rows(np.ascontiguousarray(xg), rows, W1, W3, W2, d, H, int(bf16), y, np.empty(H, np.float32))
+    return y
+
+
+def moe_tokens(x, ids, w, W1, W3, W2, E, Es, tokens, bf16=False):
+    """Layer output for the listed tokens only (routing given)."""
+    T, d = x.shape
+    K = ids.shape[1]
+    H = W1.shape[1]
+    tok = np.ascontiguousarray(tokens, np.int32)
+    out = np.empty((len(tok), d), np.float32)
+    lib().orc_moe_tokens(x, np.ascontiguousarray(ids), np.ascontiguousarray(w), W1, W3, W2, d, H, E, K, Es,
+                         int(bf16), tok, len(tok), out)
+    return out
+
+
+def moe_forward(x, Wg, bg, W1, W3, W2, K, renorm, Es=0, bf16=False):
+    """Whole layer; W1,W3: [E+Es,H,d], W2: [E+Es,d,H]. Returns a dict of every intermediate."""
+    T, d = x.shape
+    E = Wg.shape[0]
+    H = W1.shape[1]
+    P = T * K
+    r = dict(logits=np.empty((T, E), np.float32), p=np.empty((T, E), np.float32), ids=np.empty((T, K), np.int32),
+             w=np.empty((T, K), np.float32), counts=np.empty(E, np.int32), offsets=np.empty(E + 1, np.int32),
+             dst=np.empty(P, np.int32), src_row=np.empty(P, np.int32), out=np.empty((T, d), np.float32))
+    lib().orc_moe_forward(x, Wg, _opt(bg), W1, W3, W2, T, d, E, K, H, Es, int(renorm), int(bf16), r["logits"],
+                          r["p"], r["ids"], r["w"], r["counts"], r["offsets"], r["dst"], r["src_row"], r["out"])
+    return r
+
+
+def cpu_baseline_forward(x, Wg, bg, W1, W3, W2, K, renorm, Es, n_threads):
+    """Reference-CPU-style forward (column-major j8->p->i sgemm, one task per expert). Returns (seconds, out)."""
+    T, d = x.shape
+    E = Wg.shape[0]
+    H = W1.shape[1]
+    out = np.empty((T, d), np.float32)
+    s = lib().orc_cpu_baseline_forward(x, Wg, _opt(bg), W1, W3, W2, T, d, E, K, H, Es, int(renorm), int(n_threads), out)
+    return s, out
+
+
+def cpu_sgemm_tn(A, B, n_threads=1):
+    """Column-major C[m,n] = A^T B with A stored [k,m] col-major == row-major [m,k]; B row-major [n,k].
+    Returns row-major [n,m]."""
+    m, k = A.shape
+    n = B.shape[0]
+    Cm = np.zeros((n, m), np.float32)
+    lib().orc_cpu_sgemm_tn(m, n, k, np.ascontiguousarray(A), k, np.ascontiguousarray(B), k, Cm, m, n_threads)
+    return Cm
