@@ -1,0 +1,157 @@
+/*
+ * libomega_hip.so -- C ABI of the MI355X (gfx950) mixture-of-experts forward path.
+ *
+ * Plain C: opaque handles, raw device addresses, sizes and ints.  Every entry point returns an
+ * omega_status (0 = OK) and never throws or aborts across the boundary; a human-readable message
+ * for the last failure on a context is available from omega_hip_last_error().
+ *
+ * Each declaration names the reference interface it stands in for
+ * (J/ = src/main/java/com/omega/ in the reference checkout).
+ */
+#ifndef OMEGA_HIP_H
+#define OMEGA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct omega_ctx omega_ctx; /* one device + one stream; calls on a ctx are serialised */
+typedef struct omega_moe omega_moe; /* one MoE layer: owns its weights and its workspace      */
+
+typedef enum {
+    OMEGA_OK = 0,
+    OMEGA_ERR_INVALID_ARG = 1,
+    OMEGA_ERR_OOM = 2,
+    OMEGA_ERR_HIP = 3,
+    OMEGA_ERR_UNSUPPORTED = 4
+} omega_status;
+
+typedef enum { OMEGA_DTYPE_F32 = 0, OMEGA_DTYPE_BF16 = 1 } omega_dtype;
+
+/* EXACT: gate logits summed sequentially over k with separate multiply and add (the order of the
+ * reference's CPU dot, J/common/utils/MatrixOperation.java:1472-1478), so expert ids are
+ * reproducible bit for bit.  FAST: wave-parallel fp32 FMA reduction, tolerance only. */
+typedef enum { OMEGA_ROUTER_EXACT = 0, OMEGA_ROUTER_FAST = 1 } omega_router_mode;
+
+typedef enum {
+    OMEGA_W_GATE = 0,      /* [E,d]            */
+    OMEGA_W_GATE_BIAS = 1, /* [E] always fp32  */
+    OMEGA_W_W1 = 2,        /* [H,d] per expert */
+    OMEGA_W_W3 = 3,        /* [H,d] per expert */
+    OMEGA_W_W2 = 4         /* [d,H] per expert */
+} omega_weight_kind;
+
+/* Constructor arguments of the layer, in the house style of
+ * LlamaMLPLayer(embedDim, nChannel, multiple_of, bias, network), J/engine/nn/layer/llama/LlamaMLPLayer.java:47-63. */
+typedef struct {
+    int32_t T_max;         /* workspace is sized for this many tokens; grows on demand            */
+    int32_t d;             /* model width (embedDim)                                               */
+    int32_t E;             /* routed experts                                                       */
+    int32_t K;             /* experts per token                                                    */
+    int32_t H;             /* expert hidden width                                                  */
+    int32_t Es;            /* always-on shared experts (same SwiGLU shape), summed into the output */
+    int32_t renorm;        /* 1: top-k weights divided by their sum                                */
+    int32_t has_gate_bias; /* 1: logits += bg[e]                                                   */
+    int32_t dtype;         /* omega_dtype of x, out and all weights                                */
+    int32_t router_mode;   /* omega_router_mode                                                    */
+} omega_moe_config;
+
+/* Library version, major*10000 + minor*100 + patch. */
+int omega_hip_version(void);
+
+/* Per-device context.  Replaces new CUDAManager(rank) -> cuInit/cuCtxCreate
+ * (J/engine/gpu/CUDAManager.java:111-116) and the per-rank pool J/engine/parallel/cuda/CUDAPool.java:12-22.
+ * No module loading is needed: kernels are linked into the library
+ * (replaces CUDAManager.getLocalFunctionByModule, J/engine/gpu/CUDAManager.java:125-159). */
+int omega_hip_ctx_create(int device, omega_ctx **out);
+int omega_hip_ctx_destroy(omega_ctx *ctx);
+/* Message of the last failed call on ctx (or of the last failed ctx_create when ctx is NULL).
+ * Mirrors checkCUDA's "Error code N:msg" RuntimeException, J/engine/gpu/CUDAMemoryManager.java:179-201. */
+const char *omega_hip_last_error(omega_ctx *ctx);
+
+/* Device memory.  Replaces CUDAMemoryManager.getPointer / free
+ * (J/engine/gpu/CUDAMemoryManager.java:115-123,161-165). */
+int omega_hip_malloc(omega_ctx *ctx, size_t bytes, void **dptr);
+int omega_hip_free(omega_ctx *ctx, void *dptr);
+/* Blocking copies, as Tensor.hostToDevice / Tensor.syncHost (J/engine/tensor/Tensor.java:559-579). */
+int omega_hip_memcpy_h2d(omega_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+int omega_hip_memcpy_d2h(omega_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+/* Tensor.clearGPU (J/engine/tensor/Tensor.java:680-685). */
+int omega_hip_memset(omega_ctx *ctx, void *dptr, int value, size_t bytes);
+/* JCuda.cudaDeviceSynchronize() as used around timed regions (J/engine/nn/network/Llama3.java:140-156). */
+int omega_hip_sync(omega_ctx *ctx);
+
+/* Seeded synthetic data on the device: element i of `stream` under `seed`, N(0,std), written as
+ * `dtype`.  Counter-based, so any slice (first, n) of a stream can be produced independently.
+ * Stands in for RandomUtils.normal_ (J/common/utils/RandomUtils.java:697-703) + Tensor upload. */
+int omega_hip_fill_normal(omega_ctx *ctx, void *dptr, uint64_t n, uint64_t seed, uint64_t stream, double std,
+                          uint64_t first, int dtype);
+/* fp32 <-> bf16 conversion of device buffers (round to nearest even). */
+int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src, int src_dtype, uint64_t n);
+
+/* Layer life cycle.  create = the layer constructor + initParam (weights allocated, zeroed);
+ * the workspace plays the role of the lazily (re)allocated activation tensors of init()
+ * (J/engine/nn/layer/llama/LlamaMLPLayer.java:98-104, J/engine/nn/layer/FullyLayer.java:159-175). */
+int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **out);
+int omega_moe_destroy(omega_moe *moe);
+
+/* Load one weight tensor (layout [out,in] row-major, J/engine/nn/layer/FullyLayer.java:181) from host or
+ * device memory, elements of the layer dtype (gate bias: fp32).  expert: 0..E-1 routed, E..E+Es-1
+ * shared; ignored for the gate.  Stands in for FullyLayer.loadModel / weight upload
+ * (J/engine/nn/layer/FullyLayer.java:854-866). */
+int omega_moe_set_weights(omega_moe *moe, int which, int expert, const void *src, int is_device);
+/* Device address of the layer-owned storage of one weight tensor (for in-place initialisation). */
+int omega_moe_weight_ptr(omega_moe *moe, int which, int expert, void **dptr);
+
+/* forward(Tensor): x_dev [T,d] -> out_dev [T,d], both of the layer dtype, caller-owned device
+ * buffers.  Asynchronous on the context's stream; omega_hip_sync / memcpy_d2h make it visible.
+ * The drop-in for the FFN slot, J/engine/nn/layer/llama/LlamaTransformerBlock.java:135 ->
+ * LlamaMLPLayer.forward(Tensor) (J/engine/nn/layer/llama/LlamaMLPLayer.java:200-217). */
+int omega_moe_forward(omega_moe *moe, const void *x_dev, int T, void *out_dev);
+
+/* The four stages of forward, callable one at a time (per-stage timing and tests); they use the
+ * same kernels and workspace as omega_moe_forward and must be called in this order for one T:
+ *   router   x -> ids, weights, per-tile expert histogram      (gate: FullyLayer.output, FullyLayer.java:218-243;
+ *                                                               softmax: J/engine/gpu/SoftmaxKernel.cu:4-24)
+ *   dispatch histogram -> counts, offsets, dst, src_row, tile list; gather x rows into the
+ *            expert-contiguous buffer                           (gather as img_token_drop,
+ *                                                               J/engine/nn/layer/dit/kernel/TokenDropKernel.cu:147-160)
+ *   experts  grouped SwiGLU: a = silu(xg W1^T) * (xg W3^T); y = a W2^T
+ *                                                              (LlamaMLPLayer.output, LlamaMLPLayer.java:117-130)
+ *   combine  out[t] = sum_j w[t,j] * y[dst[t*K+j]] (+ shared)   (weighted sum as add_mul_kernel,
+ *                                                               J/engine/gpu/BaseKernel.cu:228-241) */
+int omega_moe_router(omega_moe *moe, const void *x_dev, int T);
+int omega_moe_dispatch(omega_moe *moe, const void *x_dev, int T);
+int omega_moe_experts(omega_moe *moe, const void *x_dev, int T);
+int omega_moe_combine(omega_moe *moe, int T, void *out_dev);
+/* The two products of the experts stage separately (profiling). */
+int omega_moe_experts_up(omega_moe *moe, const void *x_dev, int T);
+int omega_moe_experts_down(omega_moe *moe, int T);
+
+/* Routing of the last forward/router+dispatch call, copied to host (blocking).  Any pointer may
+ * be NULL.  ids,w: [T,K]; counts: [E]; offsets: [E+1]; dst, src_row: [T*K]
+ * (dst[p] = row of pair p=t*K+j in the expert-contiguous buffer; src_row[r] = token of row r). */
+int omega_moe_get_routing(omega_moe *moe, int T, int32_t *ids, float *w, int32_t *counts, int32_t *offsets,
+                          int32_t *dst, int32_t *src_row);
+/* Router intermediates, for tests: runs the router on x_dev and copies logits and probabilities
+ * [T,E] to host (blocking).  Overwrites the routing state like omega_moe_router. */
+int omega_moe_get_router_probs(omega_moe *moe, const void *x_dev, int T, float *logits, float *probs);
+/* Device addresses of workspace buffers for inspection: which = 0 xg [T*K,d] (layer dtype),
+ * 1 a [T*K+Es*T,H] (layer dtype), 2 y [T*K+Es*T,d] fp32. */
+int omega_moe_workspace_ptr(omega_moe *moe, int which, void **dptr);
+
+/* Average duration in milliseconds of the launches of one stage, measured with events on the
+ * context's stream: runs `iters` back-to-back repetitions of the stage (0 router, 1 dispatch,
+ * 2 experts_up, 3 experts_down, 4 combine, 5 whole forward, 6 dispatch index kernels only, 7 dispatch
+ * row gather only) after `warmup` untimed ones.
+ * x_dev/out_dev as for forward; the stages before `stage` must have been run for this T. */
+int omega_moe_time_stage(omega_moe *moe, int stage, const void *x_dev, int T, void *out_dev, int warmup, int iters,
+                         float *ms_avg);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OMEGA_HIP_H */

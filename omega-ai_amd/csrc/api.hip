@@ -1,0 +1,537 @@
+// C ABI of libomega_hip.so: contexts, device memory, the MoE layer handle and its forward stages.
+#include <stdio.h>
+#include <string.h>
+
+#include <new>
+
+#include "common.h"
+
+#define OMEGA_VERSION 100  // 0.1.0
+
+static thread_local std::string g_create_error;
+
+int omega_set_error(omega_ctx *ctx, int status, const char *what, hipError_t herr, const char *file, int line)
+{
+    char buf[512];
+    const char *base = strrchr(file, '/');
+    if (herr != hipSuccess)
+        snprintf(buf, sizeof buf, "Error code %d:%s (%s at %s:%d)", (int)herr, hipGetErrorString(herr), what,
+                 base ? base + 1 : file, line);
+    else
+        snprintf(buf, sizeof buf, "Error code %d:%s (%s:%d)", status, what, base ? base + 1 : file, line);
+    if (ctx) ctx->last_error = buf; else g_create_error = buf;
+    return status;
+}
+
+extern "C" {
+
+int omega_hip_version(void) { return OMEGA_VERSION; }
+
+const char *omega_hip_last_error(omega_ctx *ctx) { return ctx ? ctx->last_error.c_str() : g_create_error.c_str(); }
+
+int omega_hip_ctx_create(int device, omega_ctx **out)
+{
+    if (!out) OMEGA_FAIL(nullptr, OMEGA_ERR_INVALID_ARG, "ctx_create: out is NULL");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0)
+        return omega_set_error(nullptr, OMEGA_ERR_HIP, "ctx_create: no HIP device available", e, __FILE__, __LINE__);
+    if (device < 0 || device >= n) OMEGA_FAIL(nullptr, OMEGA_ERR_INVALID_ARG, "ctx_create: device index out of range");
+    OMEGA_HIP_CHECK(nullptr, hipSetDevice(device));
+    hipDeviceProp_t prop;
+    OMEGA_HIP_CHECK(nullptr, hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        OMEGA_FAIL(nullptr, OMEGA_ERR_UNSUPPORTED, "ctx_create: device is not gfx950 (MI355X)");
+    omega_ctx *c = new (std::nothrow) omega_ctx();
+    if (!c) OMEGA_FAIL(nullptr, OMEGA_ERR_OOM, "ctx_create: host allocation failed");
+    c->device = device;
+    c->num_cus = prop.multiProcessorCount;
+    e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = experts_bf16_init();
+    if (e != hipSuccess) {
+        delete c;
+        return omega_set_error(nullptr, OMEGA_ERR_HIP, "ctx_create: stream / kernel attribute setup", e, __FILE__, __LINE__);
+    }
+    *out = c;
+    return OMEGA_OK;
+}
+
+int omega_hip_ctx_destroy(omega_ctx *ctx)
+{
+    if (!ctx) return OMEGA_OK;
+    hipSetDevice(ctx->device);
+    hipStreamSynchronize(ctx->stream);
+    hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return OMEGA_OK;
+}
+
+#define CTX_ENTER(ctx)                                                                      \
+    if (!(ctx)) OMEGA_FAIL(nullptr, OMEGA_ERR_INVALID_ARG, "NULL context");                \
+    std::lock_guard<std::mutex> _lk((ctx)->mu);                                             \
+    OMEGA_HIP_CHECK((ctx), hipSetDevice((ctx)->device))
+
+int omega_hip_malloc(omega_ctx *ctx, size_t bytes, void **dptr)
+{
+    CTX_ENTER(ctx);
+    if (!dptr) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "malloc: dptr is NULL");
+    *dptr = nullptr;
+    if (bytes == 0) return OMEGA_OK;
+    OMEGA_HIP_CHECK(ctx, hipMalloc(dptr, bytes));
+    return OMEGA_OK;
+}
+
+int omega_hip_free(omega_ctx *ctx, void *dptr)
+{
+    CTX_ENTER(ctx);
+    if (!dptr) return OMEGA_OK;
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipFree(dptr));
+    return OMEGA_OK;
+}
+
+int omega_hip_memcpy_h2d(omega_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes)
+{
+    CTX_ENTER(ctx);
+    if (bytes == 0) return OMEGA_OK;
+    if (!dst_dev || !src_host) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "memcpy_h2d: NULL pointer");
+    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    return OMEGA_OK;
+}
+
+int omega_hip_memcpy_d2h(omega_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes)
+{
+    CTX_ENTER(ctx);
+    if (bytes == 0) return OMEGA_OK;
+    if (!dst_host || !src_dev) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "memcpy_d2h: NULL pointer");
+    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    return OMEGA_OK;
+}
+
+int omega_hip_memset(omega_ctx *ctx, void *dptr, int value, size_t bytes)
+{
+    CTX_ENTER(ctx);
+    if (bytes == 0) return OMEGA_OK;
+    if (!dptr) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "memset: NULL pointer");
+    OMEGA_HIP_CHECK(ctx, hipMemsetAsync(dptr, value, bytes, ctx->stream));
+    return OMEGA_OK;
+}
+
+int omega_hip_sync(omega_ctx *ctx)
+{
+    CTX_ENTER(ctx);
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    return OMEGA_OK;
+}
+
+static bool dtype_ok(int dt) { return dt == OMEGA_DTYPE_F32 || dt == OMEGA_DTYPE_BF16; }
+
+int omega_hip_fill_normal(omega_ctx *ctx, void *dptr, uint64_t n, uint64_t seed, uint64_t stream, double std,
+                          uint64_t first, int dtype)
+{
+    CTX_ENTER(ctx);
+    if (n == 0) return OMEGA_OK;
+    if (!dptr || !dtype_ok(dtype)) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "fill_normal: bad pointer or dtype");
+    OMEGA_HIP_CHECK(ctx, launch_fill_normal(dptr, n, seed, stream, std, first, dtype, ctx->stream));
+    return OMEGA_OK;
+}
+
+int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src, int src_dtype, uint64_t n)
+{
+    CTX_ENTER(ctx);
+    if (n == 0) return OMEGA_OK;
+    if (!dst || !src || !dtype_ok(dst_dtype) || !dtype_ok(src_dtype))
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "convert: bad pointer or dtype");
+    OMEGA_HIP_CHECK(ctx, launch_convert(dst, dst_dtype, src, src_dtype, n, ctx->stream));
+    return OMEGA_OK;
+}
+
+// ------------------------------------------------------------------------------------------ layer
+
+static void moe_free_workspace(omega_moe *m)
+{
+    void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->src_row, m->tiles, m->xg, m->a, m->y};
+    for (void *p : ptrs)
+        if (p) hipFree(p);
+    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->src_row = nullptr;
+    m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
+    m->T_cap = 0;
+}
+
+static int moe_tile_m(const omega_moe *m, int T)
+{
+    return m->cfg.dtype == OMEGA_DTYPE_BF16 ? experts_bf16_tile_m(m, T) : experts_f32_tile_m();
+}
+
+// Sizes the workspace for T tokens (grow-only, like the named caches of
+// J/engine/gpu/CUDAMemoryManager.java:34-55).
+static int moe_reserve(omega_moe *m, int T)
+{
+    omega_ctx *ctx = m->ctx;
+    if (T <= m->T_cap) return OMEGA_OK;
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    moe_free_workspace(m);
+    const omega_moe_config &c = m->cfg;
+    const size_t P = (size_t)T * c.K, R = P + (size_t)c.Es * T;
+    const int n_tok_tiles = ceil_div(T, ROUTER_TOK_TILE);
+    // smallest row tile any kernel variant uses bounds the tile list
+    const int bm_min = c.dtype == OMEGA_DTYPE_BF16 ? 32 : experts_f32_tile_m();
+    const int max_tiles = (int)(P / bm_min) + c.E + c.Es * ceil_div(T, bm_min);
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->ids, P * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->w, P * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_counts, (size_t)n_tok_tiles * c.E * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_base, (size_t)n_tok_tiles * c.E * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->dst, P * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->src_row, P * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tiles, (size_t)max_tiles * sizeof(omega_tile)));
+    OMEGA_HIP_CHECK(ctx, hipMalloc(&m->xg, P * c.d * m->esize));
+    OMEGA_HIP_CHECK(ctx, hipMalloc(&m->a, R * c.H * m->esize));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->y, R * c.d * 4));
+    m->T_cap = T;
+    return OMEGA_OK;
+}
+
+static int moe_max_m_tiles(const omega_moe *m, int T, int bm)
+{
+    const omega_moe_config &c = m->cfg;
+    return (T * c.K) / bm + c.E + c.Es * ceil_div(T, bm);
+}
+
+int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **out)
+{
+    CTX_ENTER(ctx);
+    if (!cfg || !out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "moe_create: NULL argument");
+    *out = nullptr;
+    const omega_moe_config &c = *cfg;
+    if (c.T_max < 0 || c.d <= 0 || c.E <= 0 || c.K <= 0 || c.H <= 0 || c.Es < 0)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "moe_create: dimensions must be positive");
+    if (c.K > c.E) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "moe_create: K must not exceed E");
+    if (!dtype_ok(c.dtype)) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "moe_create: unknown dtype");
+    if (c.router_mode != OMEGA_ROUTER_EXACT && c.router_mode != OMEGA_ROUTER_FAST)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "moe_create: unknown router mode");
+    if (c.E > 256) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: more than 256 routed experts");
+    if (c.Es > 64) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: more than 64 shared experts");
+    if (c.K > 64 || (c.E <= 8 && c.K > 8)) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: K above 64");
+    if (c.dtype == OMEGA_DTYPE_BF16 && (c.d % 256 != 0 || c.H % 128 != 0))
+        OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: bf16 layers need d % 256 == 0 and H % 128 == 0");
+    if ((double)c.T_max * c.K * (double)(c.d > c.H ? c.d : c.H) > 2.0e9)
+        OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: T_max*K*max(d,H) exceeds 2e9 elements");
+
+    omega_moe *m = new (std::nothrow) omega_moe();
+    if (!m) OMEGA_FAIL(ctx, OMEGA_ERR_OOM, "moe_create: host allocation failed");
+    m->ctx = ctx;
+    m->cfg = c;
+    m->G = c.E + c.Es;
+    m->esize = c.dtype == OMEGA_DTYPE_BF16 ? 2 : 4;
+    const size_t wsz = (size_t)m->G * c.H * c.d * m->esize;
+    hipError_t e = hipSuccess;
+    auto alloc0 = [&](void **p, size_t bytes) {
+        if (e != hipSuccess) return;
+        e = hipMalloc(p, bytes);
+        if (e == hipSuccess) e = hipMemsetAsync(*p, 0, bytes, ctx->stream);
+    };
+    alloc0(&m->Wg, (size_t)c.E * c.d * m->esize);
+    alloc0((void **)&m->bg, (size_t)c.E * 4);
+    alloc0(&m->W1, wsz);
+    alloc0(&m->W3, wsz);
+    alloc0(&m->W2, wsz);
+    alloc0((void **)&m->counts, (size_t)c.E * 4);
+    alloc0((void **)&m->offsets, (size_t)(c.E + 1) * 4);
+    alloc0((void **)&m->tile_meta, (size_t)(m->G + 2) * 4);
+    if (e == hipSuccess) e = hipEventCreate(&m->ev0);
+    if (e == hipSuccess) e = hipEventCreate(&m->ev1);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        omega_set_error(ctx, e == hipErrorOutOfMemory ? OMEGA_ERR_OOM : OMEGA_ERR_HIP, "moe_create: allocation", e,
+                        __FILE__, __LINE__);
+        // release whatever was allocated
+        void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta};
+        for (void *p : ptrs)
+            if (p) hipFree(p);
+        if (m->ev0) hipEventDestroy(m->ev0);
+        if (m->ev1) hipEventDestroy(m->ev1);
+        delete m;
+        return e == hipErrorOutOfMemory ? OMEGA_ERR_OOM : OMEGA_ERR_HIP;
+    }
+    if (c.T_max > 0) {
+        int st = moe_reserve(m, c.T_max);
+        if (st != OMEGA_OK) {
+            moe_free_workspace(m);
+            void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta};
+            for (void *p : ptrs)
+                if (p) hipFree(p);
+            hipEventDestroy(m->ev0);
+            hipEventDestroy(m->ev1);
+            delete m;
+            return st;
+        }
+    }
+    *out = m;
+    return OMEGA_OK;
+}
+
+int omega_moe_destroy(omega_moe *m)
+{
+    if (!m) return OMEGA_OK;
+    omega_ctx *ctx = m->ctx;
+    CTX_ENTER(ctx);
+    hipStreamSynchronize(ctx->stream);
+    moe_free_workspace(m);
+    void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta};
+    for (void *p : ptrs)
+        if (p) hipFree(p);
+    hipEventDestroy(m->ev0);
+    hipEventDestroy(m->ev1);
+    delete m;
+    return OMEGA_OK;
+}
+
+static int weight_slot(omega_moe *m, int which, int expert, void **ptr, size_t *bytes)
+{
+    const omega_moe_config &c = m->cfg;
+    const size_t per = (size_t)c.H * c.d * m->esize;
+    switch (which) {
+        case OMEGA_W_GATE: *ptr = m->Wg; *bytes = (size_t)c.E * c.d * m->esize; return OMEGA_OK;
+        case OMEGA_W_GATE_BIAS: *ptr = m->bg; *bytes = (size_t)c.E * 4; return OMEGA_OK;
+        case OMEGA_W_W1: case OMEGA_W_W3: case OMEGA_W_W2: {
+            if (expert < 0 || expert >= m->G) return OMEGA_ERR_INVALID_ARG;
+            unsigned char *base = (unsigned char *)(which == OMEGA_W_W1 ? m->W1 : which == OMEGA_W_W3 ? m->W3 : m->W2);
+            *ptr = base + per * (size_t)expert;
+            *bytes = per;
+            return OMEGA_OK;
+        }
+        default: return OMEGA_ERR_INVALID_ARG;
+    }
+}
+
+int omega_moe_set_weights(omega_moe *m, int which, int expert, const void *src, int is_device)
+{
+    if (!m) OMEGA_FAIL(nullptr, OMEGA_ERR_INVALID_ARG, "NULL layer");
+    omega_ctx *ctx = m->ctx;
+    CTX_ENTER(ctx);
+    void *p; size_t bytes;
+    if (!src || weight_slot(m, which, expert, &p, &bytes) != OMEGA_OK)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "set_weights: bad kind, expert index or source");
+    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(p, src, bytes, is_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    return OMEGA_OK;
+}
+
+int omega_moe_weight_ptr(omega_moe *m, int which, int expert, void **dptr)
+{
+    if (!m) OMEGA_FAIL(nullptr, OMEGA_ERR_INVALID_ARG, "NULL layer");
+    omega_ctx *ctx = m->ctx;
+    CTX_ENTER(ctx);
+    size_t bytes;
+    if (!dptr || weight_slot(m, which, expert, dptr, &bytes) != OMEGA_OK)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "weight_ptr: bad kind or expert index");
+    return OMEGA_OK;
+}
+
+// ---- stages (caller holds the context lock) ----
+static int check_T(omega_moe *m, const void *x, int T, bool need_x)
+{
+    omega_ctx *ctx = m->ctx;
+    if (T < 0) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "forward: negative token count");
+    if (need_x && T > 0 && !x) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "forward: x is NULL");
+    if ((double)T * m->cfg.K * (double)(m->cfg.d > m->cfg.H ? m->cfg.d : m->cfg.H) > 2.0e9)
+        OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "forward: T*K*max(d,H) exceeds 2e9 elements");
+    return OMEGA_OK;
+}
+
+static int stage_router(omega_moe *m, const void *x, int T)
+{
+    OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, nullptr, m->ctx->stream));
+    return OMEGA_OK;
+}
+static int stage_dispatch(omega_moe *m, const void *x, int T)
+{
+    const int bm = moe_tile_m(m, T);
+    m->bm = bm;
+    m->max_m_tiles = moe_max_m_tiles(m, T, bm);
+    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));
+    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));
+    return OMEGA_OK;
+}
+static int stage_experts(omega_moe *m, const void *x, int T, int which)
+{
+    if (m->bm != moe_tile_m(m, T)) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "experts: dispatch has not run for this T");
+    if (m->cfg.dtype == OMEGA_DTYPE_BF16) OMEGA_HIP_CHECK(m->ctx, launch_experts_bf16(m, x, T, which, m->ctx->stream));
+    else OMEGA_HIP_CHECK(m->ctx, launch_experts_f32(m, x, T, which, m->ctx->stream));
+    return OMEGA_OK;
+}
+static int stage_combine(omega_moe *m, int T, void *out)
+{
+    OMEGA_HIP_CHECK(m->ctx, launch_combine(m, T, out, m->ctx->stream));
+    return OMEGA_OK;
+}
+
+#define MOE_ENTER(m)                                                          \
+    if (!(m)) OMEGA_FAIL(nullptr, OMEGA_ERR_INVALID_ARG, "NULL layer");      \
+    omega_ctx *ctx = (m)->ctx;                                                \
+    CTX_ENTER(ctx)
+
+#define RUN(expr)                         \
+    do {                                  \
+        int _st = (expr);                 \
+        if (_st != OMEGA_OK) return _st;  \
+    } while (0)
+
+int omega_moe_forward(omega_moe *m, const void *x, int T, void *out)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, x, T, true));
+    if (T == 0) return OMEGA_OK;
+    if (!out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "forward: out is NULL");
+    RUN(moe_reserve(m, T));
+    RUN(stage_router(m, x, T));
+    RUN(stage_dispatch(m, x, T));
+    RUN(stage_experts(m, x, T, 0));
+    RUN(stage_experts(m, x, T, 1));
+    RUN(stage_combine(m, T, out));
+    return OMEGA_OK;
+}
+
+int omega_moe_router(omega_moe *m, const void *x, int T)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, x, T, true));
+    if (T == 0) return OMEGA_OK;
+    RUN(moe_reserve(m, T));
+    return stage_router(m, x, T);
+}
+
+int omega_moe_dispatch(omega_moe *m, const void *x, int T)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, x, T, true));
+    if (T == 0) return OMEGA_OK;
+    if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "dispatch: router has not run for this T");
+    return stage_dispatch(m, x, T);
+}
+
+int omega_moe_experts_up(omega_moe *m, const void *x, int T)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, x, T, m->cfg.Es > 0));
+    if (T == 0) return OMEGA_OK;
+    if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "experts: router has not run for this T");
+    return stage_experts(m, x, T, 0);
+}
+
+int omega_moe_experts_down(omega_moe *m, int T)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, nullptr, T, false));
+    if (T == 0) return OMEGA_OK;
+    if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "experts: router has not run for this T");
+    return stage_experts(m, nullptr, T, 1);
+}
+
+int omega_moe_experts(omega_moe *m, const void *x, int T)
+{
+    int st = omega_moe_experts_up(m, x, T);
+    return st != OMEGA_OK ? st : omega_moe_experts_down(m, T);
+}
+
+int omega_moe_combine(omega_moe *m, int T, void *out)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, nullptr, T, false));
+    if (T == 0) return OMEGA_OK;
+    if (!out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "combine: out is NULL");
+    if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "combine: router has not run for this T");
+    return stage_combine(m, T, out);
+}
+
+int omega_moe_get_routing(omega_moe *m, int T, int32_t *ids, float *w, int32_t *counts, int32_t *offsets, int32_t *dst,
+                          int32_t *src_row)
+{
+    MOE_ENTER(m);
+    if (T < 0 || T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_routing: T exceeds the last forward");
+    const size_t P = (size_t)T * m->cfg.K;
+    hipStream_t s = ctx->stream;
+    if (ids && P) OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(ids, m->ids, P * 4, hipMemcpyDeviceToHost, s));
+    if (w && P) OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(w, m->w, P * 4, hipMemcpyDeviceToHost, s));
+    if (counts) OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(counts, m->counts, (size_t)m->cfg.E * 4, hipMemcpyDeviceToHost, s));
+    if (offsets) OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(offsets, m->offsets, (size_t)(m->cfg.E + 1) * 4, hipMemcpyDeviceToHost, s));
+    if (dst && P) OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(dst, m->dst, P * 4, hipMemcpyDeviceToHost, s));
+    if (src_row && P) OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(src_row, m->src_row, P * 4, hipMemcpyDeviceToHost, s));
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(s));
+    return OMEGA_OK;
+}
+
+int omega_moe_get_router_probs(omega_moe *m, const void *x, int T, float *logits, float *probs)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, x, T, true));
+    if (T == 0) return OMEGA_OK;
+    RUN(moe_reserve(m, T));
+    const size_t n = (size_t)T * m->cfg.E;
+    float *dl = nullptr, *dp = nullptr;
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&dl, n * 4));
+    hipError_t e = hipMalloc((void **)&dp, n * 4);
+    if (e == hipSuccess) e = launch_router(m, x, T, dl, dp, ctx->stream);
+    if (e == hipSuccess && logits) e = hipMemcpyAsync(logits, dl, n * 4, hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess && probs) e = hipMemcpyAsync(probs, dp, n * 4, hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    hipFree(dl);
+    if (dp) hipFree(dp);
+    OMEGA_HIP_CHECK(ctx, e);
+    return OMEGA_OK;
+}
+
+int omega_moe_workspace_ptr(omega_moe *m, int which, void **dptr)
+{
+    MOE_ENTER(m);
+    if (!dptr || which < 0 || which > 2) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "workspace_ptr: bad selector");
+    *dptr = which == 0 ? m->xg : which == 1 ? m->a : (void *)m->y;
+    return OMEGA_OK;
+}
+
+int omega_moe_time_stage(omega_moe *m, int stage, const void *x, int T, void *out, int warmup, int iters, float *ms_avg)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, x, T, stage == 0 || stage == 1 || stage == 5 || stage == 7));
+    if ((stage == 6 || stage == 7) && m->bm == 0) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: dispatch has not run");
+    if (!ms_avg || iters <= 0 || warmup < 0 || stage < 0 || stage > 7 || T <= 0)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: bad argument");
+    if ((stage == 4 || stage == 5) && !out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: out is NULL");
+    if (stage == 0 || stage == 5) RUN(moe_reserve(m, T));
+    else if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: earlier stages have not run for this T");
+    auto once = [&]() -> int {
+        switch (stage) {
+            case 0: return stage_router(m, x, T);
+            case 1: return stage_dispatch(m, x, T);
+            case 2: return stage_experts(m, x, T, 0);
+            case 3: return stage_experts(m, x, T, 1);
+            case 4: return stage_combine(m, T, out);
+            case 6:
+                OMEGA_HIP_CHECK(ctx, launch_dispatch_index(m, T, m->bm, ctx->stream));
+                return OMEGA_OK;
+            case 7:
+                OMEGA_HIP_CHECK(ctx, launch_dispatch_gather(m, x, T, ctx->stream));
+                return OMEGA_OK;
+            default:
+                RUN(stage_router(m, x, T));
+                RUN(stage_dispatch(m, x, T));
+                RUN(stage_experts(m, x, T, 0));
+                RUN(stage_experts(m, x, T, 1));
+                return stage_combine(m, T, out);
+        }
+    };
+    for (int i = 0; i < warmup; ++i) RUN(once());
+    OMEGA_HIP_CHECK(ctx, hipEventRecord(m->ev0, ctx->stream));
+    for (int i = 0; i < iters; ++i) RUN(once());
+    OMEGA_HIP_CHECK(ctx, hipEventRecord(m->ev1, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipEventSynchronize(m->ev1));
+    float ms = 0.0f;
+    OMEGA_HIP_CHECK(ctx, hipEventElapsedTime(&ms, m->ev0, m->ev1));
+    *ms_avg = ms / (float)iters;
+    return OMEGA_OK;
+}
+
+}  // extern "C"

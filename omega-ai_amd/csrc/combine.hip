@@ -1,0 +1,110 @@
+// Combine: out[t,:] = sum_j w[t,j] * y[dst[t*K+j],:] in slot order, then + the shared experts' rows.
+// One wave per token; each lane owns 4 (fp32 out) or 8 (bf16 out) consecutive columns, read from the
+// fp32 rows of y with 16-byte loads; products and sums are separate fp32 operations in slot order
+// (this file is compiled with -ffp-contract=off), the weighted sum of add_mul_kernel
+// (J/engine/gpu/BaseKernel.cu:228-241) generalised to K terms; shared rows are added as add_kernel
+// (J/engine/ad/op/gpu/OPKernel.cu:359-366).  No atomics: every output element has one writer.
+#include "common.h"
+
+#define MAXK 64
+
+template <int VEC, bool BF16>
+__global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ dst,
+                                                      const float *__restrict__ w, int T, int K, int d, int Es, int P,
+                                                      void *__restrict__ out)
+{
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    // lane j < K holds row index and weight of slot j; broadcast through cross-lane reads
+    int myrow = 0;
+    float myw = 0.0f;
+    if (lane < K) {
+        myrow = dst[(size_t)t * K + lane];
+        myw = w[(size_t)t * K + lane];
+    }
+    for (int c0 = lane * VEC; c0 < d; c0 += 64 * VEC) {
+        float acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+        for (int j = 0; j < K; ++j) {
+            const int row = __shfl(myrow, j, 64);
+            const float wj = __shfl(myw, j, 64);
+            const float4 *src = (const float4 *)(y + (size_t)row * d + c0);
+#pragma unroll
+            for (int q = 0; q < VEC / 4; ++q) {
+                const float4 v4 = src[q];
+                float term;
+                term = wj * v4.x; acc[q * 4 + 0] = acc[q * 4 + 0] + term;
+                term = wj * v4.y; acc[q * 4 + 1] = acc[q * 4 + 1] + term;
+                term = wj * v4.z; acc[q * 4 + 2] = acc[q * 4 + 2] + term;
+                term = wj * v4.w; acc[q * 4 + 3] = acc[q * 4 + 3] + term;
+            }
+        }
+        for (int s = 0; s < Es; ++s) {
+            const float4 *src = (const float4 *)(y + ((size_t)P + (size_t)s * T + t) * d + c0);
+#pragma unroll
+            for (int q = 0; q < VEC / 4; ++q) {
+                const float4 v4 = src[q];
+                acc[q * 4 + 0] = acc[q * 4 + 0] + v4.x;
+                acc[q * 4 + 1] = acc[q * 4 + 1] + v4.y;
+                acc[q * 4 + 2] = acc[q * 4 + 2] + v4.z;
+                acc[q * 4 + 3] = acc[q * 4 + 3] + v4.w;
+            }
+        }
+        if (BF16) {
+            uint32_t pk[VEC / 2];
+#pragma unroll
+            for (int v = 0; v < VEC / 2; ++v)
+                pk[v] = (uint32_t)f32_to_bf16(acc[2 * v]) | ((uint32_t)f32_to_bf16(acc[2 * v + 1]) << 16);
+            uint4 o = {pk[0], pk[1], pk[2], pk[3]};
+            *(uint4 *)((bf16_t *)out + (size_t)t * d + c0) = o;
+        } else {
+            float4 o = {acc[0], acc[1], acc[2], acc[3]};
+            *(float4 *)((float *)out + (size_t)t * d + c0) = o;
+        }
+    }
+}
+
+// Any d: scalar columns.
+template <bool BF16>
+__global__ __launch_bounds__(256) void combine_scalar_kernel(const float *__restrict__ y, const int32_t *__restrict__ dst,
+                                                             const float *__restrict__ w, int T, int K, int d, int Es,
+                                                             int P, void *__restrict__ out)
+{
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float acc = 0.0f;
+        for (int j = 0; j < K; ++j) {
+            const float term = w[(size_t)t * K + j] * y[(size_t)dst[(size_t)t * K + j] * d + c];
+            acc = acc + term;
+        }
+        for (int s = 0; s < Es; ++s) acc = acc + y[((size_t)P + (size_t)s * T + t) * d + c];
+        if (BF16) ((bf16_t *)out)[(size_t)t * d + c] = f32_to_bf16(acc);
+        else ((float *)out)[(size_t)t * d + c] = acc;
+    }
+}
+
+hipError_t launch_combine(const omega_moe *m, int T, void *out, hipStream_t s)
+{
+    const omega_moe_config &c = m->cfg;
+    const int P = T * c.K;
+    const bool bf = c.dtype == OMEGA_DTYPE_BF16;
+    const int vec = bf ? 8 : 4;
+    if (c.d % vec == 0 && ((uintptr_t)out % 16) == 0 && c.K <= MAXK) {
+        if (bf)
+            hipLaunchKernelGGL((combine_kernel<8, true>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dst, m->w, T,
+                               c.K, c.d, c.Es, P, out);
+        else
+            hipLaunchKernelGGL((combine_kernel<4, false>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dst, m->w, T,
+                               c.K, c.d, c.Es, P, out);
+    } else {
+        if (bf)
+            hipLaunchKernelGGL(combine_scalar_kernel<true>, dim3(T), dim3(256), 0, s, m->y, m->dst, m->w, T, c.K, c.d,
+                               c.Es, P, out);
+        else
+            hipLaunchKernelGGL(combine_scalar_kernel<false>, dim3(T), dim3(256), 0, s, m->y, m->dst, m->w, T, c.K, c.d,
+                               c.Es, P, out);
+    }
+    return hipGetLastError();
+}

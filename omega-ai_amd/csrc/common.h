@@ -1,0 +1,100 @@
+// Internal declarations shared by the translation units of libomega_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <mutex>
+#include <string>
+
+#include "omega_hip.h"
+
+typedef uint16_t bf16_t;  // raw bf16 bit pattern in device buffers
+
+struct omega_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::mutex mu;
+    std::string last_error;
+    int num_cus = 256;
+};
+
+// One entry per row tile of the grouped products: written on the device by the scan kernel.
+struct __attribute__((aligned(16))) omega_tile {
+    int32_t g;      // weight index: 0..E-1 routed, E..E+Es-1 shared
+    int32_t row0;   // first row in the a / y buffers (and in xg for routed experts)
+    int32_t rows;   // valid rows in this tile (1..BM)
+    int32_t xrow0;  // -1: A operand of the up product is xg[row0..]; >=0: it is x[xrow0..] (shared expert)
+};
+
+struct omega_moe {
+    omega_ctx *ctx = nullptr;
+    omega_moe_config cfg{};
+    int G = 0;            // E + Es
+    size_t esize = 4;     // bytes per element of the layer dtype
+    int T_cap = 0;        // tokens the workspace is sized for
+    int bm = 0;           // row-tile height the tile list was built for
+    // weights (layer dtype except bg)
+    void *Wg = nullptr;   // [E,d]
+    float *bg = nullptr;  // [E]
+    void *W1 = nullptr;   // [G,H,d]
+    void *W3 = nullptr;   // [G,H,d]
+    void *W2 = nullptr;   // [G,d,H]
+    // workspace
+    int32_t *ids = nullptr;          // [T,K]
+    float *w = nullptr;              // [T,K]
+    int32_t *tile_counts = nullptr;  // [n_tok_tiles,E] histogram per token tile (router)
+    int32_t *tile_base = nullptr;    // [n_tok_tiles,E] exclusive prefix of tile_counts over the tiles (scan)
+    int32_t *counts = nullptr;       // [E]
+    int32_t *offsets = nullptr;      // [E+1]
+    int32_t *dst = nullptr;          // [T*K]
+    int32_t *src_row = nullptr;      // [T*K]
+    omega_tile *tiles = nullptr;     // [max_m_tiles]
+    int32_t *tile_meta = nullptr;    // [0] = number of row tiles; [1+g] = first row tile of group g (G+1 entries)
+    void *xg = nullptr;              // [T*K,d]
+    void *a = nullptr;               // [T*K+Es*T,H]
+    float *y = nullptr;              // [T*K+Es*T,d]
+    int max_m_tiles = 0;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+};
+
+#define ROUTER_TOK_TILE 32
+
+__host__ __device__ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+int omega_set_error(omega_ctx *ctx, int status, const char *what, hipError_t herr, const char *file, int line);
+
+#define OMEGA_FAIL(ctx, status, what) return omega_set_error((ctx), (status), (what), hipSuccess, __FILE__, __LINE__)
+#define OMEGA_HIP_CHECK(ctx, expr)                                                             \
+    do {                                                                                       \
+        hipError_t _e = (expr);                                                                \
+        if (_e != hipSuccess)                                                                  \
+            return omega_set_error((ctx), _e == hipErrorOutOfMemory ? OMEGA_ERR_OOM : OMEGA_ERR_HIP, #expr, _e, \
+                                   __FILE__, __LINE__);                                        \
+    } while (0)
+
+// ---- launchers (one per .hip file); all asynchronous on `s`, returning the launch status ----
+hipError_t launch_fill_normal(void *dptr, uint64_t n, uint64_t seed, uint64_t stream_id, double std, uint64_t first,
+                              int dtype, hipStream_t s);
+hipError_t launch_convert(void *dst, int dst_dtype, const void *src, int src_dtype, uint64_t n, hipStream_t s);
+
+hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s);
+hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s);
+hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipStream_t s);
+hipError_t launch_experts_f32(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
+hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
+hipError_t launch_combine(const omega_moe *m, int T, void *out, hipStream_t s);
+int experts_bf16_tile_m(const omega_moe *m, int T);
+int experts_f32_tile_m(void);
+hipError_t experts_bf16_init(void);
+
+// ---- device helpers ----
+#ifdef __HIPCC__
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+__device__ __forceinline__ bf16_t f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+#endif

@@ -1,0 +1,278 @@
+"""Host side of the MoE layer over the C ABI, mirroring the reference's Layer contract.
+
+The reference is Java; no JDK is available to this build, so the host-side mirror used by the
+tests and the benchmark is this module (and host/MoELayer.hpp for C++ callers).  Method names,
+argument meaning and error behaviour follow the reference's layers:
+  * constructor in the house style of LlamaMLPLayer(embedDim, nChannel, multiple_of, bias, network)
+    (J/engine/nn/layer/llama/LlamaMLPLayer.java:47-63) with the explicit hidden size of
+    DiTSwiGLUFFN (J/engine/nn/layer/dit/org/DiTSwiGLUFFN.java)
+  * forward(input) = setInput -> init -> output (LlamaMLPLayer.java:200-217); getOutput()
+  * saveModel/loadModel: raw little-endian float32, no header, fixed order
+    (J/engine/nn/network/utils/ModelUtils.java:58-93; order w1,w3,w2 per expert as LlamaMLPLayer.java:273-283)
+  * a non-zero status from the library raises RuntimeError("Error code N:msg"), the checkCUDA style
+    (J/engine/gpu/CUDAMemoryManager.java:179-201); back/update raise: the path is forward-only.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib as L
+
+
+def _check(st, ctx_handle):
+    if st != L.OK:
+        msg = L.load_library().omega_hip_last_error(ctx_handle)
+        raise RuntimeError((msg or b"Error code %d" % st).decode())
+
+
+def f32_to_bf16_bits(a):
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + np.uint64(0x7FFF) + ((u >> np.uint64(16)) & np.uint64(1))) >> np.uint64(16)
+    return u.astype(np.uint16)
+
+
+def bf16_bits_to_f32(b):
+    return (np.ascontiguousarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+class Context:
+    """One device + one stream (replaces CUDAManager / CUDAPool for this path)."""
+
+    def __init__(self, device=0):
+        self.lib = L.load_library()
+        h = C.c_void_p()
+        st = self.lib.omega_hip_ctx_create(device, C.byref(h))
+        if st != L.OK:
+            raise RuntimeError((self.lib.omega_hip_last_error(None) or b"ctx_create failed").decode())
+        self.handle = h
+
+    def check(self, st):
+        _check(st, self.handle)
+
+    def sync(self):
+        self.check(self.lib.omega_hip_sync(self.handle))
+
+    def close(self):
+        if self.handle:
+            self.lib.omega_hip_ctx_destroy(self.handle)
+            self.handle = None
+
+
+class DeviceBuffer:
+    """Caller-owned device memory (the role of Tensor.gpuData, J/engine/tensor/Tensor.java:23-47)."""
+
+    def __init__(self, ctx, shape, dtype):
+        self.ctx, self.shape, self.dtype = ctx, tuple(shape), dtype
+        self.esize = 2 if dtype == "bf16" else 4
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.esize
+        p = C.c_void_p()
+        ctx.check(ctx.lib.omega_hip_malloc(ctx.handle, max(self.nbytes, 16), C.byref(p)))
+        self.ptr = p
+
+    @classmethod
+    def from_numpy(cls, ctx, a, dtype):
+        """a: fp32 values; stored as fp32 or as bf16 (round to nearest even)."""
+        b = cls(ctx, a.shape, dtype)
+        b.upload(a)
+        return b
+
+    def upload(self, a):
+        h = f32_to_bf16_bits(a) if self.dtype == "bf16" else np.ascontiguousarray(a, np.float32)
+        assert h.nbytes == self.nbytes
+        self.ctx.check(self.ctx.lib.omega_hip_memcpy_h2d(self.ctx.handle, self.ptr, h.ctypes.data, h.nbytes))
+
+    def to_numpy(self):
+        """Blocking copy to host (Tensor.syncHost); bf16 buffers come back widened to fp32."""
+        h = np.empty(self.shape, np.uint16 if self.dtype == "bf16" else np.float32)
+        self.ctx.check(self.ctx.lib.omega_hip_memcpy_d2h(self.ctx.handle, h.ctypes.data, self.ptr, h.nbytes))
+        return bf16_bits_to_f32(h) if self.dtype == "bf16" else h
+
+    def fill_normal(self, seed, stream, std, first=0):
+        n = int(np.prod(self.shape, dtype=np.int64))
+        self.ctx.check(self.ctx.lib.omega_hip_fill_normal(self.ctx.handle, self.ptr, n, seed, stream, float(std), first,
+                                                          L.DTYPE_BF16 if self.dtype == "bf16" else L.DTYPE_F32))
+
+    def free(self):
+        if self.ptr:
+            self.ctx.lib.omega_hip_free(self.ctx.handle, self.ptr)
+            self.ptr = None
+
+
+class MoELayer:
+    """Mixture-of-experts FFN layer, forward only."""
+
+    def __init__(self, embedDim, hidden, nExperts, topK, renorm=True, nShared=0, bias=False, ctx=None,
+                 dtype="f32", router_mode="exact", T_max=0):
+        self.ctx = ctx or Context(0)
+        self.lib = self.ctx.lib
+        self.embedDim, self.hidden, self.nExperts, self.topK = embedDim, hidden, nExperts, topK
+        self.renorm, self.nShared, self.hasBias, self.dtype = bool(renorm), nShared, bool(bias), dtype
+        self.oChannel, self.oHeight, self.oWidth = 1, 1, embedDim
+        self.number = 0
+        self.input = None
+        self.output_buf = None
+        cfg = L.MoEConfigStruct(T_max, embedDim, nExperts, topK, hidden, nShared, int(renorm), int(bias),
+                                L.DTYPE_BF16 if dtype == "bf16" else L.DTYPE_F32,
+                                L.ROUTER_EXACT if router_mode == "exact" else L.ROUTER_FAST)
+        h = C.c_void_p()
+        self.ctx.check(self.lib.omega_moe_create(self.ctx.handle, C.byref(cfg), C.byref(h)))
+        self.handle = h
+
+    # ---- parameters
+    def _upload(self, which, expert, a):
+        if which == L.W_GATE_BIAS or self.dtype == "f32":
+            h = np.ascontiguousarray(a, np.float32)
+        else:
+            h = f32_to_bf16_bits(a)
+        self.ctx.check(self.lib.omega_moe_set_weights(self.handle, which, expert, h.ctypes.data, 0))
+
+    def set_gate(self, Wg, bg=None):
+        assert Wg.shape == (self.nExperts, self.embedDim)
+        self._upload(L.W_GATE, 0, Wg)
+        if bg is not None:
+            assert self.hasBias and bg.shape == (self.nExperts,)
+            self._upload(L.W_GATE_BIAS, 0, bg)
+
+    def set_expert(self, g, W1, W3, W2):
+        assert W1.shape == (self.hidden, self.embedDim) and W3.shape == W1.shape
+        assert W2.shape == (self.embedDim, self.hidden)
+        self._upload(L.W_W1, g, W1)
+        self._upload(L.W_W3, g, W3)
+        self._upload(L.W_W2, g, W2)
+
+    def weight_ptr(self, which, expert=0):
+        p = C.c_void_p()
+        self.ctx.check(self.lib.omega_moe_weight_ptr(self.handle, which, expert, C.byref(p)))
+        return p
+
+    def init_synthetic(self, seed, cfgmod, cfg):
+        """Fills every weight in place on the device from the seeded generator (see configs.py)."""
+        dt = L.DTYPE_BF16 if self.dtype == "bf16" else L.DTYPE_F32
+        fill = self.lib.omega_hip_fill_normal
+        n_w = self.hidden * self.embedDim
+        self.ctx.check(fill(self.ctx.handle, self.weight_ptr(L.W_GATE), self.nExperts * self.embedDim, seed,
+                            cfgmod.STREAM_WG, cfgmod.tensor_std(cfg, "Wg"), 0, dt))
+        for g in range(self.nExperts + self.nShared):
+            for which, name in ((L.W_W1, "W1"), (L.W_W3, "W3"), (L.W_W2, "W2")):
+                self.ctx.check(fill(self.ctx.handle, self.weight_ptr(which, g), n_w, seed,
+                                    cfgmod.expert_stream(g, name), cfgmod.tensor_std(cfg, name), 0, dt))
+        bg = cfgmod.zipf_gate_bias(cfg, seed)
+        if bg is not None:
+            self._upload(L.W_GATE_BIAS, 0, bg)
+        self.ctx.sync()
+
+    # ---- Layer contract
+    def init(self):
+        """(Re)allocates the output when the batch size changes (LlamaMLPLayer.init)."""
+        self.number = self.input.shape[0]
+        if self.output_buf is None or self.output_buf.shape[0] != self.number:
+            if self.output_buf is not None:
+                self.output_buf.free()
+            self.output_buf = DeviceBuffer(self.ctx, (self.number, self.embedDim), self.dtype)
+
+    def setInput(self, inp):
+        if inp.shape[-1] != self.embedDim:
+            raise RuntimeError("Error code 1:input width does not match embedDim")
+        self.input = inp
+
+    def output(self):
+        self.ctx.check(self.lib.omega_moe_forward(self.handle, self.input.ptr, self.number, self.output_buf.ptr))
+
+    def forward(self, inp):
+        self.setInput(inp)
+        self.init()
+        self.output()
+        return self.output_buf
+
+    def getOutput(self):
+        return self.output_buf
+
+    def getLayerType(self):
+        return "feed_forward"
+
+    def back(self, delta=None):
+        raise NotImplementedError("MoELayer is forward-only")
+
+    backTemp = diff = update = initBack = back
+
+    def accGrad(self, scale):
+        raise NotImplementedError("MoELayer is forward-only")
+
+    # ---- stages and introspection
+    def stage(self, name, x=None, out=None):
+        T = self.number
+        f = {"router": lambda: self.lib.omega_moe_router(self.handle, x.ptr, T),
+             "dispatch": lambda: self.lib.omega_moe_dispatch(self.handle, x.ptr, T),
+             "experts": lambda: self.lib.omega_moe_experts(self.handle, x.ptr if x is not None else None, T),
+             "combine": lambda: self.lib.omega_moe_combine(self.handle, T, out.ptr)}[name]
+        self.ctx.check(f())
+
+    def time_stage(self, stage, x, T, out=None, warmup=2, iters=10):
+        ms = C.c_float()
+        self.ctx.check(self.lib.omega_moe_time_stage(self.handle, stage, x.ptr if x is not None else None, T,
+                                                     out.ptr if out is not None else None, warmup, iters, C.byref(ms)))
+        return ms.value
+
+    def routing(self, T=None):
+        T = self.number if T is None else T
+        K, E = self.topK, self.nExperts
+        r = dict(ids=np.empty((T, K), np.int32), w=np.empty((T, K), np.float32), counts=np.empty(E, np.int32),
+                 offsets=np.empty(E + 1, np.int32), dst=np.empty(T * K, np.int32), src_row=np.empty(T * K, np.int32))
+        self.ctx.check(self.lib.omega_moe_get_routing(self.handle, T, *[r[k].ctypes.data for k in
+                                                                         ("ids", "w", "counts", "offsets", "dst", "src_row")]))
+        return r
+
+    def router_probs(self, x, T):
+        lg = np.empty((T, self.nExperts), np.float32)
+        p = np.empty((T, self.nExperts), np.float32)
+        self.ctx.check(self.lib.omega_moe_get_router_probs(self.handle, x.ptr, T, lg.ctypes.data, p.ctypes.data))
+        return lg, p
+
+    def workspace(self, which, T):
+        """Host copy of a workspace buffer: 'xg' [T*K,d], 'a' [T*K+Es*T,H], 'y' [T*K+Es*T,d] (fp32 values)."""
+        idx = {"xg": 0, "a": 1, "y": 2}[which]
+        p = C.c_void_p()
+        self.ctx.check(self.lib.omega_moe_workspace_ptr(self.handle, idx, C.byref(p)))
+        P, R = T * self.topK, T * self.topK + self.nShared * T
+        shape = {"xg": (P, self.embedDim), "a": (R, self.hidden), "y": (R, self.embedDim)}[which]
+        raw_bf16 = self.dtype == "bf16" and which != "y"
+        h = np.empty(shape, np.uint16 if raw_bf16 else np.float32)
+        self.ctx.check(self.lib.omega_hip_memcpy_d2h(self.ctx.handle, h.ctypes.data, p, h.nbytes))
+        return bf16_bits_to_f32(h) if raw_bf16 else h
+
+    # ---- checkpoint: raw LE float32, order gate, (gate bias), then w1,w3,w2 per expert, routed then shared
+    def _download_weight(self, which, expert, shape):
+        p = self.weight_ptr(which, expert)
+        raw_bf16 = self.dtype == "bf16" and which != L.W_GATE_BIAS
+        h = np.empty(shape, np.uint16 if raw_bf16 else np.float32)
+        self.ctx.check(self.lib.omega_hip_memcpy_d2h(self.ctx.handle, h.ctypes.data, p, h.nbytes))
+        return bf16_bits_to_f32(h) if raw_bf16 else h
+
+    def _param_list(self):
+        items = [(L.W_GATE, 0, (self.nExperts, self.embedDim))]
+        if self.hasBias:
+            items.append((L.W_GATE_BIAS, 0, (self.nExperts,)))
+        for g in range(self.nExperts + self.nShared):
+            items += [(L.W_W1, g, (self.hidden, self.embedDim)), (L.W_W3, g, (self.hidden, self.embedDim)),
+                      (L.W_W2, g, (self.embedDim, self.hidden))]
+        return items
+
+    def saveModel(self, f):
+        for which, g, shape in self._param_list():
+            f.write(self._download_weight(which, g, shape).astype("<f4").tobytes())
+
+    def loadModel(self, f):
+        for which, g, shape in self._param_list():
+            n = int(np.prod(shape))
+            buf = f.read(4 * n)
+            if len(buf) != 4 * n:
+                raise RuntimeError("Error code 1:checkpoint ends early")
+            self._upload(which, g, np.frombuffer(buf, "<f4").reshape(shape))
+
+    def close(self):
+        if self.output_buf is not None:
+            self.output_buf.free()
+            self.output_buf = None
+        if self.handle:
+            self.lib.omega_moe_destroy(self.handle)
+            self.handle = None

@@ -1,0 +1,201 @@
+"""GPU parity tests: the HIP path through the C ABI against the CPU oracle on the same seeded inputs.
+
+Bars: expert ids, per-expert counts, offsets and the permutation bit-exact (exact router mode);
+layer output within 1e-5 relative L2 in fp32 and within 1e-2 relative L2 in bf16 (fp32 accumulate).
+"""
+import io
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from oracle import oracle_np as N
+from tests.synth import C, make_inputs, scaled
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-5
+BF16_TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def G():
+    from tests import gpu_util
+    return gpu_util
+
+
+def test_device_generator_matches_oracle_bitwise(G):
+    P = G.P
+    for dtype, n, seed, stream, std, first in (("f32", 300001, 7, 0, 1.0, 0), ("f32", 4097, 2**63 + 9, 33, 0.02, 2**34),
+                                               ("bf16", 100000, 5, 18, 1 / 64.0, 12345)):
+        b = P.DeviceBuffer(G.ctx(), (n,), dtype)
+        b.fill_normal(seed, stream, std, first)
+        got = b.to_numpy()
+        ref = O.fill_normal(n, seed, stream, std, first)
+        if dtype == "bf16":
+            ref = O.round_bf16(ref)
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+        b.free()
+
+
+def test_c1_tiny_fp32_full_parity(G):
+    cfg = C.CONFIGS["c1_tiny_f32"]
+    layer, x, out, r, ref, inp = G.run_case(cfg, seed=20251)
+    G.assert_routing_bit_exact(r, ref)
+    lg, p = layer.router_probs(x, cfg.T)
+    assert np.array_equal(lg.view(np.uint32), ref["logits"].view(np.uint32))
+    assert np.array_equal(p.view(np.uint32), ref["p"].view(np.uint32))
+    assert np.array_equal(layer.workspace("xg", cfg.T), inp["x"][ref["src_row"]])
+    assert N.rel_l2(out, ref["out"]) <= F32_TOL
+    # dense-MoE identity, independent of any permutation
+    dense = N.dense_moe_fp64(inp["x"], r["ids"], r["w"], inp["W1"], inp["W3"], inp["W2"], cfg.E)
+    assert N.rel_l2(out, dense) <= F32_TOL
+    layer.close()
+
+
+@pytest.mark.parametrize("T", [1, 2, 31, 33, 100, 257])
+def test_fp32_ragged_token_counts(G, T):
+    cfg = scaled(C.CONFIGS["c1_tiny_f32"], T=T)
+    layer, x, out, r, ref, inp = G.run_case(cfg, seed=3 + T)
+    G.assert_routing_bit_exact(r, ref)
+    assert N.rel_l2(out, ref["out"]) <= F32_TOL
+    layer.close()
+
+
+@pytest.mark.parametrize("E,K,Es,renorm,d,H,T", [
+    (1, 1, 0, True, 64, 96, 40),       # single expert == plain SwiGLU MLP
+    (5, 5, 0, False, 48, 80, 70),      # K == E, odd sizes (scalar fallbacks)
+    (16, 4, 1, True, 128, 192, 130),
+    (64, 6, 2, False, 64, 128, 200),   # fine-grained + shared experts, no renorm
+    (128, 8, 0, True, 64, 64, 300),
+    (200, 8, 0, True, 32, 64, 90),     # more experts than lanes in a wave, not a power of two
+])
+def test_fp32_shapes(G, E, K, Es, renorm, d, H, T):
+    cfg = C.MoEConfig("t", T=T, d=d, E=E, K=K, H=H, Es=Es, renorm=renorm, dtype="f32")
+    layer, x, out, r, ref, inp = G.run_case(cfg, seed=E * 1000 + K)
+    G.assert_routing_bit_exact(r, ref)
+    assert N.rel_l2(out, ref["out"]) <= F32_TOL
+    layer.close()
+
+
+def test_fp32_ties_and_empty_experts(G):
+    """All-equal gate rows: every token ties across all experts -> experts 0..K-1; the rest stay empty."""
+    cfg = C.MoEConfig("t", T=77, d=64, E=8, K=3, H=64, dtype="f32")
+    inp = make_inputs(cfg, seed=9)
+    inp["Wg"][:] = 0.0
+    layer = G.build_layer(cfg, inp)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], "f32")
+    out = layer.forward(x).to_numpy()
+    r = layer.routing()
+    ref = G.oracle_forward(cfg, inp)
+    G.assert_routing_bit_exact(r, ref)
+    assert r["ids"].tolist() == [[0, 1, 2]] * 77
+    assert r["counts"].tolist() == [77, 77, 77, 0, 0, 0, 0, 0]
+    assert N.rel_l2(out, ref["out"]) <= F32_TOL
+    # duplicated gate rows: pairwise ties between experts (1,5) and (2,6)
+    inp = make_inputs(cfg, seed=10)
+    inp["Wg"][5] = inp["Wg"][1]
+    inp["Wg"][6] = inp["Wg"][2]
+    layer2 = G.build_layer(cfg, inp)
+    x2 = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], "f32")
+    out2 = layer2.forward(x2).to_numpy()
+    ref2 = G.oracle_forward(cfg, inp)
+    G.assert_routing_bit_exact(layer2.routing(), ref2)
+    assert N.rel_l2(out2, ref2["out"]) <= F32_TOL
+    layer.close()
+    layer2.close()
+
+
+def test_zipf_bias_skewed_fp32(G):
+    cfg = scaled(C.CONFIGS["c5_skewed"], T=600, d=64, H=64, dtype="f32")
+    layer, x, out, r, ref, inp = G.run_case(cfg, seed=77)
+    G.assert_routing_bit_exact(r, ref)
+    assert (r["counts"] == 0).any()
+    assert N.rel_l2(out, ref["out"]) <= F32_TOL
+    layer.close()
+
+
+@pytest.mark.parametrize("name,kw", [
+    ("c2_mixtral", dict(T=512, d=512, H=1024)),
+    ("c2_mixtral", dict(T=1000, d=256, H=384)),        # ragged row tiles
+    ("c3_decode", dict(T=64, d=512, H=1024)),
+    ("c4_finegrained", dict(T=512, d=256, H=384)),     # 64 experts, 2 shared, no renorm
+    ("c5_skewed", dict(T=1024, d=256, H=256)),         # 128 experts, Zipf bias, empty experts
+])
+def test_bf16_scaled_configs(G, name, kw):
+    cfg = scaled(C.CONFIGS[name], **kw)
+    layer, x, out, r, ref, inp = G.run_case(cfg, seed=4242)
+    G.assert_routing_bit_exact(r, ref)
+    assert np.array_equal(layer.workspace("xg", cfg.T), inp["x"][ref["src_row"]])
+    err = N.rel_l2(out, ref["out"])
+    assert err <= BF16_TOL, err
+    # against the unrounded fp64 dense identity as well (looser: bf16 rounding of a and out)
+    dense = N.dense_moe_fp64(inp["x"], r["ids"], r["w"], inp["W1"], inp["W3"], inp["W2"], cfg.E, cfg.Es)
+    assert N.rel_l2(out, dense) <= BF16_TOL
+    layer.close()
+
+
+def test_bf16_fast_router_agrees(G):
+    cfg = scaled(C.CONFIGS["c2_mixtral"], T=512, d=512, H=1024)
+    layer, x, out, r, ref, inp = G.run_case(cfg, seed=4242, router_mode="fast")
+    agree = (r["ids"] == ref["ids"]).all(axis=1).mean()
+    assert agree >= 0.995
+    c2, o2, d2, s2 = N.dispatch_argsort(r["ids"], cfg.E)          # dispatch stays exact for the ids it got
+    assert np.array_equal(r["counts"], c2) and np.array_equal(r["dst"], d2) and np.array_equal(r["src_row"], s2)
+    assert N.rel_l2(out, ref["out"]) <= BF16_TOL
+    layer.close()
+
+
+def test_stage_entry_points_match_forward(G):
+    cfg = scaled(C.CONFIGS["c4_finegrained"], T=300, d=256, H=384)
+    inp = make_inputs(cfg, 5)
+    layer = G.build_layer(cfg, inp)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    full = layer.forward(x).to_numpy().copy()
+    out2 = G.P.DeviceBuffer(G.ctx(), (cfg.T, cfg.d), cfg.dtype)
+    for st in ("router", "dispatch", "experts", "combine"):
+        layer.stage(st, x=x, out=out2)
+    assert np.array_equal(out2.to_numpy(), full)
+    # repeating dispatch alone is idempotent
+    before = layer.routing()
+    layer.stage("dispatch", x=x)
+    after = layer.routing()
+    for k in before:
+        assert np.array_equal(before[k], after[k])
+    # growing and shrinking the batch on one layer
+    for T in (64, 700, 5):
+        i2 = make_inputs(cfg, 6, T)
+        xb = G.P.DeviceBuffer.from_numpy(G.ctx(), i2["x"], cfg.dtype)
+        o = layer.forward(xb).to_numpy()
+        i2.update({k: inp[k] for k in ("Wg", "bg", "W1", "W3", "W2")})
+        ref = G.oracle_forward(cfg, i2)
+        G.assert_routing_bit_exact(layer.routing(), ref)
+        assert N.rel_l2(o, ref["out"]) <= BF16_TOL
+    layer.close()
+
+
+def test_checkpoint_round_trip_and_errors(G):
+    cfg = C.MoEConfig("t", T=16, d=64, E=4, K=2, H=128, Es=1, dtype="f32", zipf_bias=1.2)
+    inp = make_inputs(cfg, 1)
+    layer = G.build_layer(cfg, inp)
+    f = io.BytesIO()
+    layer.saveModel(f)
+    raw = f.getvalue()
+    expect = np.concatenate([inp["Wg"].ravel(), inp["bg"].ravel()] +
+                            [np.concatenate([inp["W1"][g].ravel(), inp["W3"][g].ravel(), inp["W2"][g].ravel()])
+                             for g in range(5)]).astype("<f4").tobytes()
+    assert raw == expect                                   # byte-exact, order gate, bias, (w1,w3,w2) per expert
+    other = G.P.MoELayer(cfg.d, cfg.H, cfg.E, cfg.K, True, cfg.Es, True, ctx=G.ctx(), dtype="f32")
+    other.loadModel(io.BytesIO(raw))
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], "f32")
+    assert np.array_equal(other.forward(x).to_numpy(), layer.forward(x).to_numpy())
+    with pytest.raises(RuntimeError, match="Error code"):
+        other.loadModel(io.BytesIO(raw[:100]))
+    with pytest.raises(RuntimeError, match="Error code"):
+        G.P.MoELayer(64, 64, 4, 5, ctx=G.ctx())            # K > E
+    with pytest.raises(RuntimeError, match="Error code"):
+        G.P.MoELayer(100, 64, 4, 2, ctx=G.ctx(), dtype="bf16")   # unsupported bf16 width
+    with pytest.raises(RuntimeError, match="Error code"):
+        layer.forward(G.P.DeviceBuffer(G.ctx(), (4, 32), "f32"))
+    layer.close()
+    other.close()
