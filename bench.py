@@ -1,0 +1,165 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE-layer forward path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2_mixtral] [--no-cpu-baseline]
+
+A step is one forward pass of the layer over one batch of seeded synthetic tokens that already sit
+in HBM.  Prints ONE JSON line: whole-layer tokens/s, the roofline figure of the dominant kernel
+(the grouped up-projection, bf16 MFMA bound) measured with events on the library's own stream
+inside the timed forwards, per-stage figures, a sampled parity check, and a CPU baseline (the
+C restatement of the reference's CPU-style path, timed on a bounded token sample).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3
+PEAK_HBM_GBPS = 8000.0
+
+# HBM traffic per launch of the dominant kernel from the committed rocprofv3 --pmc runs
+# (profiles/experts_up_c2_mixtral_pmc.txt): FETCH_SIZE + WRITE_SIZE in bytes, scaled by the copy-kernel factor.
+TRAFFIC_BYTES = {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c2_mixtral")
+    ap.add_argument("--seed", type=int, default=20251)
+    ap.add_argument("--router", default="exact", choices=["exact", "fast"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample duration")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus above 1 is not supported (no collectives in this path)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    P = importlib.import_module("omega-ai_amd")
+    L = importlib.import_module("omega-ai_amd._lib")
+    C = P.configs
+    cfg = C.CONFIGS[a.config]
+    ctx = P.Context(0)
+    layer = P.MoELayer(cfg.d, cfg.H, cfg.E, cfg.K, renorm=cfg.renorm, nShared=cfg.Es, bias=cfg.has_gate_bias, ctx=ctx,
+                       dtype=cfg.dtype, router_mode=a.router, T_max=cfg.T)
+    layer.init_synthetic(a.seed, C, cfg)
+    x = P.DeviceBuffer(ctx, (cfg.T, cfg.d), cfg.dtype)
+    x.fill_normal(a.seed, C.STREAM_X, C.tensor_std(cfg, "x"))
+    ctx.sync()
+
+    for _ in range(a.warmup):
+        layer.forward(x)
+    ctx.sync()
+    layer.set_profiling(True)
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        layer.forward(x)
+    ctx.sync()
+    t1 = time.perf_counter()
+    stage_ms, n_prof = layer.get_profile()
+    layer.set_profiling(False)
+    ms_per_step = (t1 - t0) * 1e3 / a.steps
+    tokens_per_s = cfg.T / (ms_per_step * 1e-3)
+
+    b = 2 if cfg.dtype == "bf16" else 4
+    rows = cfg.P + cfg.Es * cfg.T
+    up_flops = 4.0 * cfg.d * cfg.H * rows
+    down_flops = 2.0 * cfg.d * cfg.H * rows
+    peak = PEAK_BF16_TFLOPS if cfg.dtype == "bf16" else PEAK_F32_TFLOPS
+    up_tflops = up_flops / (stage_ms["experts_up"] * 1e-3) / 1e12
+    down_tflops = down_flops / (stage_ms["experts_down"] * 1e-3) / 1e12
+    # algorithmic bytes of the bandwidth-bound stages
+    router_bytes = cfg.T * cfg.d * b + cfg.E * cfg.d * b + cfg.P * 8
+    dispatch_bytes = 2 * cfg.P * cfg.d * b + cfg.P * 12
+    combine_bytes = cfg.P * cfg.d * b + cfg.T * cfg.d * b + cfg.P * 8
+    gather_ms = layer.time_stage(L.STAGE_GATHER, x, cfg.T, warmup=2, iters=20)
+    index_ms = layer.time_stage(L.STAGE_INDEX, x, cfg.T, warmup=2, iters=20)
+
+    res = {
+        "metric": "MoE-layer fwd tokens/s (Mixtral shape, bf16); MFMA util %; dispatch GB/s",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": cfg.dtype, "data": "synthetic (seeded counter-based normal generator, generated in HBM)",
+        "config": {"workload": f"{cfg.name}: T={cfg.T} ({cfg.batch}x{cfg.seq}) d={cfg.d} E={cfg.E} K={cfg.K} H={cfg.H} "
+                               f"Es={cfg.Es} renorm={int(cfg.renorm)} {cfg.dtype}, fp32 accumulate",
+                   "router_mode": a.router, "seed": a.seed},
+        "roofline": {"bound": "mfma", "kernel": "experts_bf16_kernel<up>: a = silu(xg W1^T) * (xg W3^T)",
+                     "achieved": up_tflops, "peak": peak, "unit": "TFLOP/s", "frac": up_tflops / peak,
+                     "algorithmic_flops_per_launch": up_flops, "avg_launch_ms": stage_ms["experts_up"],
+                     "traffic": TRAFFIC_BYTES.get(cfg.name)},
+        "stages": {
+            "avg_ms": stage_ms, "profiled_forwards": n_prof,
+            "experts_down": {"TFLOP/s": down_tflops, "frac_mfma": down_tflops / peak},
+            "experts_total_frac_mfma": (up_flops + down_flops) / ((stage_ms["experts_up"] + stage_ms["experts_down"]) * 1e-3) / 1e12 / peak,
+            "router": {"GB/s": router_bytes / (stage_ms["router"] * 1e-3) / 1e9, "frac_hbm": router_bytes / (stage_ms["router"] * 1e-3) / 1e9 / PEAK_HBM_GBPS},
+            "dispatch": {"GB/s": dispatch_bytes / (stage_ms["dispatch"] * 1e-3) / 1e9,
+                         "frac_hbm": dispatch_bytes / (stage_ms["dispatch"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                         "gather_only_ms": gather_ms, "gather_only_GB/s": 2 * cfg.P * cfg.d * b / (gather_ms * 1e-3) / 1e9,
+                         "index_only_ms": index_ms},
+            "combine": {"GB/s": combine_bytes / (stage_ms["combine"] * 1e-3) / 1e9,
+                        "frac_hbm": combine_bytes / (stage_ms["combine"] * 1e-3) / 1e9 / PEAK_HBM_GBPS},
+        },
+    }
+
+    need_host = not (a.no_parity and a.no_cpu_baseline)
+    if need_host:
+        from oracle import oracle as O
+        from oracle import oracle_np as N
+        G = cfg.E + cfg.Es
+        xh = x.to_numpy()
+        Wg = layer._download_weight(L.W_GATE, 0, (cfg.E, cfg.d))
+        bg = C.zipf_gate_bias(cfg, a.seed)
+        W1 = np.empty((G, cfg.H, cfg.d), np.float32)
+        W3 = np.empty((G, cfg.H, cfg.d), np.float32)
+        W2 = np.empty((G, cfg.d, cfg.H), np.float32)
+        for g in range(G):
+            W1[g] = layer._download_weight(L.W_W1, g, (cfg.H, cfg.d))
+            W3[g] = layer._download_weight(L.W_W3, g, (cfg.H, cfg.d))
+            W2[g] = layer._download_weight(L.W_W2, g, (cfg.d, cfg.H))
+        bf = cfg.dtype == "bf16"
+        if not a.no_parity:
+            out = layer.forward(x).to_numpy()
+            r = layer.routing()
+            p = O.softmax(O.gate(xh, Wg, bg))
+            ids, w = O.topk(p, cfg.K, cfg.renorm)
+            counts, offsets, dst, src = O.dispatch(ids, cfg.E)
+            tok = np.unique(np.linspace(0, cfg.T - 1, 16).astype(np.int32))
+            ref = O.moe_tokens(xh, ids, w, W1, W3, W2, cfg.E, cfg.Es, tok, bf16=bf)
+            res["parity"] = {
+                "ids_bit_exact": bool(np.array_equal(r["ids"], ids)), "weights_bit_exact": bool(np.array_equal(r["w"], w)),
+                "counts_bit_exact": bool(np.array_equal(r["counts"], counts)),
+                "perm_bit_exact": bool(np.array_equal(r["dst"], dst) and np.array_equal(r["src_row"], src)),
+                "out_rel_l2_sampled_tokens": N.rel_l2(out[tok], ref), "sampled_tokens": int(len(tok)),
+                "tolerance": 1e-2 if bf else 1e-5}
+        if not a.no_cpu_baseline:
+            n_threads = min(16, os.cpu_count() or 1)
+            Ts, secs = min(16, cfg.T), 0.0
+            while True:
+                secs, _ = O.cpu_baseline_forward(np.ascontiguousarray(xh[:Ts]), Wg, bg, W1, W3, W2, cfg.K, cfg.renorm,
+                                                 cfg.Es, n_threads)
+                if secs >= a.cpu_seconds / 3 or Ts >= cfg.T:
+                    break
+                Ts = int(min(cfg.T, max(Ts * 2, Ts * a.cpu_seconds / max(secs, 1e-3))))
+            res["cpu_baseline"] = {
+                "value": Ts / secs, "unit": "tokens/s", "cores": min(n_threads, G), "kind": "port",
+                "sample": f"C restatement (no JDK) of the reference's CPU-style path (column-major j8->p->i sgemm, "
+                          f"one task per expert, {n_threads}-thread pool): first {Ts} tokens of the same batch, all "
+                          f"{G} experts' weights, fp32 arithmetic on the bf16-rounded values, {secs:.2f} s",
+                "host_cpus": os.cpu_count()}
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

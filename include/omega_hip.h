@@ -151,6 +151,15 @@ int omega_moe_workspace_ptr(omega_moe *moe, int which, void **dptr);
 int omega_moe_time_stage(omega_moe *moe, int stage, const void *x_dev, int T, void *out_dev, int warmup, int iters,
                          float *ms_avg);
 
+/* Per-stage timing of omega_moe_forward itself: while profiling is on, every forward records events
+ * on the context's stream around its five stages (router, dispatch, experts_up, experts_down,
+ * combine).  get_profile waits for the stream, returns the summed duration of each stage in
+ * milliseconds over the forwards since profiling was switched on (or since the last get_profile)
+ * and their number, and starts a new accumulation.  Replaces the hand-placed
+ * cudaDeviceSynchronize + System.nanoTime prints of J/engine/nn/network/Llama3.java:140-156. */
+int omega_moe_set_profiling(omega_moe *moe, int on);
+int omega_moe_get_profile(omega_moe *moe, float stage_ms_sum[5], int *n_calls);
+
 #ifdef __cplusplus
 }
 #endif

@@ -51,6 +51,8 @@ SIGNATURES = {
     "omega_moe_workspace_ptr": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]),
     "omega_moe_time_stage": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int,
                                        C.POINTER(C.c_float)]),
+    "omega_moe_set_profiling": (C.c_int, [C.c_void_p, C.c_int]),
+    "omega_moe_get_profile": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_int)]),
 }
 
 _lib = None

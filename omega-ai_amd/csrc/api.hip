@@ -285,6 +285,7 @@ int omega_moe_destroy(omega_moe *m)
         if (p) hipFree(p);
     hipEventDestroy(m->ev0);
     hipEventDestroy(m->ev1);
+    for (hipEvent_t ev : m->prof_events) hipEventDestroy(ev);
     delete m;
     return OMEGA_OK;
 }
@@ -387,11 +388,61 @@ int omega_moe_forward(omega_moe *m, const void *x, int T, void *out)
     if (T == 0) return OMEGA_OK;
     if (!out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "forward: out is NULL");
     RUN(moe_reserve(m, T));
+    if (m->profiling) {
+        // six events bracket the five stages; durations are read back by omega_moe_get_profile
+        if (m->prof_used + 6 > m->prof_events.size()) {
+            for (int i = 0; i < 6; ++i) {
+                hipEvent_t ev;
+                OMEGA_HIP_CHECK(ctx, hipEventCreate(&ev));
+                m->prof_events.push_back(ev);
+            }
+        }
+        hipEvent_t *ev = &m->prof_events[m->prof_used];
+        OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[0], ctx->stream));
+        RUN(stage_router(m, x, T));
+        OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[1], ctx->stream));
+        RUN(stage_dispatch(m, x, T));
+        OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[2], ctx->stream));
+        RUN(stage_experts(m, x, T, 0));
+        OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[3], ctx->stream));
+        RUN(stage_experts(m, x, T, 1));
+        OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[4], ctx->stream));
+        RUN(stage_combine(m, T, out));
+        OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[5], ctx->stream));
+        m->prof_used += 6;
+        return OMEGA_OK;
+    }
     RUN(stage_router(m, x, T));
     RUN(stage_dispatch(m, x, T));
     RUN(stage_experts(m, x, T, 0));
     RUN(stage_experts(m, x, T, 1));
     RUN(stage_combine(m, T, out));
+    return OMEGA_OK;
+}
+
+int omega_moe_set_profiling(omega_moe *m, int on)
+{
+    MOE_ENTER(m);
+    m->profiling = on != 0;
+    m->prof_used = 0;
+    return OMEGA_OK;
+}
+
+int omega_moe_get_profile(omega_moe *m, float *stage_ms_sum, int *n_calls)
+{
+    MOE_ENTER(m);
+    if (!stage_ms_sum || !n_calls) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_profile: NULL argument");
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    for (int i = 0; i < 5; ++i) stage_ms_sum[i] = 0.0f;
+    const size_t calls = m->prof_used / 6;
+    for (size_t c = 0; c < calls; ++c)
+        for (int i = 0; i < 5; ++i) {
+            float ms = 0.0f;
+            OMEGA_HIP_CHECK(ctx, hipEventElapsedTime(&ms, m->prof_events[c * 6 + i], m->prof_events[c * 6 + i + 1]));
+            stage_ms_sum[i] += ms;
+        }
+    *n_calls = (int)calls;
+    m->prof_used = 0;
     return OMEGA_OK;
 }
 

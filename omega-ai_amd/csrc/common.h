@@ -5,6 +5,7 @@
 
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "omega_hip.h"
 
@@ -55,6 +56,10 @@ struct omega_moe {
     float *y = nullptr;              // [T*K+Es*T,d]
     int max_m_tiles = 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // per-stage event profiling of forward calls (6 events per call), off by default
+    bool profiling = false;
+    std::vector<hipEvent_t> prof_events;
+    size_t prof_used = 0;
 };
 
 #define ROUTER_TOK_TILE 32

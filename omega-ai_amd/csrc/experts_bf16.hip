@@ -4,10 +4,20 @@
 // (J/engine/nn/layer/llama/LlamaMLPLayer.java:117-130; y = x W^T with W [out,in], J/engine/nn/layer/FullyLayer.java:181,235.)
 //
 // Both operands are K-contiguous ("NT" product), so a lane's 8 consecutive k values are one 16-byte LDS read.
-// Workgroup = 4 waves (2x2), tile 256 rows x 256 MFMA columns x 64 k, each wave 128x128 = 4x4 MFMA blocks.
-// For the up product the 256 MFMA columns are 128 columns of W1 and the same 128 columns of W3, arranged so
-// that a wave holds h1 and h3 of the same output element and applies silu(h1)*h3 in registers.
-// LDS: two stages of (A 256x64 + B 256x64) bf16 = 128 KiB, 16-byte chunks XOR-swizzled by row.
+// Workgroup = 4 waves (2x2), tile 256 rows x 256 MFMA columns x 64 k, each wave 128x128 = 4x4 MFMA blocks with
+// its 256 accumulators in AGPRs (one wave per SIMD).  For the up product the 256 MFMA columns are 128 columns
+// of W1 and the same 128 columns of W3, arranged so that a wave holds h1 and h3 of the same output element and
+// applies silu(h1)*h3 in registers.
+//
+// Data movement: global -> LDS directly (global_load_lds_dwordx4, no staging registers), two LDS stages of
+// (A 256x64 + B 256x64) bf16 = 128 KiB.  A wave-wide direct load fills 1 KiB of LDS in lane order = 8 rows of
+// 8 16-byte chunks; the XOR swizzle of the chunk index that keeps the MFMA operand reads free of bank conflicts
+// is applied by choosing which global chunk each lane fetches.
+// Pipeline per 64-k step: four phases of 16 MFMAs; the operand fragments of phase p+1 are read from LDS while
+// phase p computes; the one barrier per step sits before the last phase, after which the loads of the step
+// after next are issued into the stage just released and the first fragments of the next step are read, so
+// both latencies are covered by the 16 MFMAs of the last phase.
+//
 // Scheduling: the dispatch stage leaves a list of row tiles (never straddling two experts; empty experts
 // have none) and the first row tile of every expert; workgroup -> (expert, column tile, row tile) is
 // derived from those on the device, row tiles fastest so that the workgroups resident on one XCD share
@@ -19,16 +29,24 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
 #define BM 256
-#define BNT 256  // MFMA columns per tile
 #define BK 64
-#define STAGE_BYTES (BM * BK * 2)
-#define SMEM_BYTES (4 * STAGE_BYTES)
+#define TILE_BYTES (BM * BK * 2)      // one operand tile: 32 KiB
+#define STAGE_BYTES (2 * TILE_BYTES)  // A + B
+#define NSTAGE 2
+#define SMEM_BYTES (NSTAGE * STAGE_BYTES)
 #define NUM_XCD 8
 
 int experts_bf16_tile_m(const omega_moe *, int) { return BM; }
 
-__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
-__device__ __forceinline__ int lds_off(int row, int kc) { return row * (BK * 2) + ((kc ^ swz(row)) << 4); }
+// chunk-index swizzle: free of bank conflicts for 8 consecutive rows on 32 banks and 16 on 64 banks
+__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16*l.
+__device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(sbase), "v"(voff), "s"(lds_base)
+                 : "memory");
+}
 
 template <bool FUSED>
 __global__ __launch_bounds__(256, 1) void experts_bf16_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
@@ -36,7 +54,7 @@ __global__ __launch_bounds__(256, 1) void experts_bf16_kernel(const bf16_t *__re
                                                               void *__restrict__ Cout, const omega_tile *__restrict__ tiles,
                                                               const int32_t *__restrict__ tile_meta, int G, int N, int Kd)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     constexpr int NCOLS = FUSED ? 128 : 256;  // output columns per tile
     const int NT = N / NCOLS;
     // ---- workgroup -> tile ----
@@ -61,35 +79,59 @@ __global__ __launch_bounds__(256, 1) void experts_bf16_kernel(const bf16_t *__re
     const bf16_t *B0 = Wa + ((size_t)tl.g * N + n0) * Kd;
     const bf16_t *B1 = FUSED ? Wb + ((size_t)tl.g * N + n0) * Kd : B0 + (size_t)128 * Kd;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const int lrow = tid >> 3, lkc = tid & 7;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
 
-    int aoff[8], boff[8];
+    // ---- direct-load addressing: wave-load q (0..31) of an operand tile covers rows 8q..8q+7 ----
+    uint32_t aoff[8], boff[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int r = lrow + 32 * i;
-        aoff[i] = min(r, tl.rows - 1) * Kd + lkc * 8;
-        boff[i] = (r & 127) * Kd + lkc * 8;
+    for (int j = 0; j < 8; ++j) {
+        const int r = 8 * (wave + 4 * j) + (lane >> 3);
+        const int c = (lane & 7) ^ swz(r);
+        aoff[j] = (uint32_t)(min(r, tl.rows - 1) * Kd + c * 8) * 2u;
+        boff[j] = (uint32_t)((r & 127) * Kd + c * 8) * 2u;
     }
-    uint4 ra[8], rb[8];
-    auto gload = [&](int k0) {
+#define ISSUE_LOADS(stage, k0)                                                                      \
+    do {                                                                                            \
+        const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                              \
+        const uint32_t kb = (uint32_t)(k0) * 2u;                                                     \
+        _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                \
+        {                                                                                           \
+            dma16(A, aoff[j] + kb, sb + j * 4096);                                                   \
+            dma16(j < 4 ? B0 : B1, boff[j] + kb, sb + TILE_BYTES + j * 4096);                        \
+        }                                                                                           \
+    } while (0)
+
+    // ---- MFMA operand addressing ----
+    const int l32 = lane & 31, lhi = lane >> 5;
+    uint32_t a_rb[4], b_rb[4];
+    int a_sw[4], b_sw[4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            ra[i] = *(const uint4 *)(A + aoff[i] + k0);
-            rb[i] = *(const uint4 *)((i < 4 ? B0 : B1) + boff[i] + k0);
-        }
-    };
-    auto lstore = [&](int buf) {
-        unsigned char *as = smem + buf * STAGE_BYTES;
-        unsigned char *bs = smem + 2 * STAGE_BYTES + buf * STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int r = lrow + 32 * i;
-            *(uint4 *)(as + lds_off(r, lkc)) = ra[i];
-            *(uint4 *)(bs + lds_off(r, lkc)) = rb[i];
-        }
-    };
+    for (int i = 0; i < 4; ++i) {
+        const int ar = wm * 128 + i * 32 + l32;
+        const int br = FUSED ? ((i >> 1) * 128 + wn * 64 + (i & 1) * 32 + l32) : (wn * 128 + i * 32 + l32);
+        a_rb[i] = ar * (BK * 2);
+        b_rb[i] = TILE_BYTES + br * (BK * 2);
+        a_sw[i] = swz(ar);
+        b_sw[i] = swz(br);
+    }
+#define READ_FRAGS(AF, BF, stage, ks)                                                                       \
+    do {                                                                                                    \
+        const unsigned char *sp = smem + (stage) * STAGE_BYTES;                                              \
+        const int c = (ks) * 2 + lhi;                                                                        \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                        \
+        {                                                                                                   \
+            AF[i] = *(const bf16x8_t *)(sp + a_rb[i] + ((c ^ a_sw[i]) << 4));                                \
+            BF[i] = *(const bf16x8_t *)(sp + b_rb[i] + ((c ^ b_sw[i]) << 4));                                \
+        }                                                                                                   \
+    } while (0)
+#define MFMA16(AF, BF)                                                                                       \
+    do {                                                                                                    \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)           \
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0);            \
+    } while (0)
 
     f32x16_t acc[4][4];
 #pragma unroll
@@ -99,40 +141,35 @@ __global__ __launch_bounds__(256, 1) void experts_bf16_kernel(const bf16_t *__re
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    const int l32 = lane & 31, lhi = lane >> 5;
-    int arow[4], brow[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        arow[i] = wm * 128 + i * 32 + l32;
-        brow[i] = FUSED ? ((i >> 1) * 128 + wn * 64 + (i & 1) * 32 + l32) : (wn * 128 + i * 32 + l32);
-    }
-
     const int KT = Kd / BK;
-    gload(0);
-    lstore(0);
+    bf16x8_t af0[4], bf0[4], af1[4], bf1[4];
+
+    // prologue: stage 0 <- step 0, stage 1 <- step 1
+    ISSUE_LOADS(0, 0);
+    if (KT > 1) ISSUE_LOADS(1, BK);
+    if (KT > 1) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    READ_FRAGS(af0, bf0, 0, 0);
+
     for (int kt = 0; kt < KT; ++kt) {
         const int cur = kt & 1;
-        if (kt + 1 < KT) gload((kt + 1) * BK);
-        const unsigned char *as = smem + cur * STAGE_BYTES;
-        const unsigned char *bs = smem + 2 * STAGE_BYTES + cur * STAGE_BYTES;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            bf16x8_t af[4], bfr[4];
-            const int kc = ks * 2 + lhi;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                af[i] = *(const bf16x8_t *)(as + lds_off(arow[i], kc));
-                bfr[i] = *(const bf16x8_t *)(bs + lds_off(brow[i], kc));
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < KT) lstore(cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        READ_FRAGS(af1, bf1, cur, 1);
+        MFMA16(af0, bf0);
+        __builtin_amdgcn_sched_barrier(0);
+        READ_FRAGS(af0, bf0, cur, 2);
+        MFMA16(af1, bf1);
+        __builtin_amdgcn_sched_barrier(0);
+        READ_FRAGS(af1, bf1, cur, 3);
+        MFMA16(af0, bf0);
+        __builtin_amdgcn_sched_barrier(0);
+        // every wave has taken its last fragments of this stage; the other stage must have landed
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __syncthreads();
+        if (kt + 2 < KT) ISSUE_LOADS(cur, (kt + 2) * BK);
+        if (kt + 1 < KT) READ_FRAGS(af0, bf0, cur ^ 1, 0);
+        MFMA16(af1, bf1);
     }
 
     // ---- epilogue: lane holds column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4 ----

@@ -213,6 +213,17 @@ class MoELayer:
                                                      out.ptr if out is not None else None, warmup, iters, C.byref(ms)))
         return ms.value
 
+    def set_profiling(self, on):
+        self.ctx.check(self.lib.omega_moe_set_profiling(self.handle, int(on)))
+
+    def get_profile(self):
+        """(per-stage average ms dict, number of forwards) since profiling was switched on."""
+        ms = (C.c_float * 5)()
+        n = C.c_int()
+        self.ctx.check(self.lib.omega_moe_get_profile(self.handle, ms, C.byref(n)))
+        names = ("router", "dispatch", "experts_up", "experts_down", "combine")
+        return {k: ms[i] / max(n.value, 1) for i, k in enumerate(names)}, n.value
+
     def routing(self, T=None):
         T = self.number if T is None else T
         K, E = self.topK, self.nExperts
