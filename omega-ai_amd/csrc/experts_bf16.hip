@@ -29,23 +29,197 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
 #define BM 256
-#define BK 64
-#define TILE_BYTES (BM * BK * 2)      // one operand tile: 32 KiB
+#define BK 32
+#define TILE_BYTES (BM * BK * 2)      // one operand tile: 16 KiB
 #define STAGE_BYTES (2 * TILE_BYTES)  // A + B
-#define NSTAGE 2
-#define SMEM_BYTES (NSTAGE * STAGE_BYTES)
+#define NSTAGE 5
+#define SMEM_BYTES (NSTAGE * STAGE_BYTES)  // 160 KiB: all of a CU's LDS
+#define LOADS_PER_STEP 8                   // direct loads a wave issues per 32-k step (4 per operand)
 #define NUM_XCD 8
 
 int experts_bf16_tile_m(const omega_moe *, int) { return BM; }
 
-// chunk-index swizzle: free of bank conflicts for 8 consecutive rows on 32 banks and 16 on 64 banks
-__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+// swizzle of the 16-byte chunk index (4 chunks per 64-byte row): free of bank conflicts for 8 consecutive
+// rows on 32 banks and for 16 consecutive rows on 64 banks
+__device__ __forceinline__ int swz(int row) { return ((row >> 1) ^ (row >> 3)) & 3; }
 
 // 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16*l.
 __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_base)
 {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(sbase), "v"(voff), "s"(lds_base)
                  : "memory");
+}
+
+// One output tile.  NBLK = number of 32-row blocks of this wave that hold valid rows (the others are never
+// computed: a ragged last row tile of an expert costs only the blocks it fills).  NBLK == 0: the wave only
+// takes part in the loads and barriers.
+template <bool FUSED, int NBLK>
+__device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, const bf16_t *B0, const bf16_t *B1,
+                                         void *Cout, const omega_tile tl, int n0, int N, int Kd, int wave, int lane)
+{
+    constexpr int NB = NBLK > 0 ? NBLK : 1;
+    const int wm = wave >> 1, wn = wave & 1;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+
+    // ---- direct-load addressing: wave-load q (0..15) of an operand tile covers rows 16q..16q+15 ----
+    uint32_t aoff[4], boff[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int r = 16 * (wave + 4 * j) + (lane >> 2);
+        const int c = (lane & 3) ^ swz(r);
+        aoff[j] = (uint32_t)(min(r, tl.rows - 1) * Kd + c * 8) * 2u;
+        boff[j] = (uint32_t)((r & 127) * Kd + c * 8) * 2u;
+    }
+// direct loads j0..j1-1 (of 4 per operand) of one 32-k step into a stage
+#define ISSUE_LOADS(stage, k0, j0, j1)                                                              \
+    do {                                                                                            \
+        const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                              \
+        const uint32_t kb = (uint32_t)(k0) * 2u;                                                     \
+        _Pragma("unroll") for (int j = (j0); j < (j1); ++j)                                          \
+        {                                                                                           \
+            dma16(A, aoff[j] + kb, sb + j * 4096);                                                   \
+            dma16(j < 2 ? B0 : B1, boff[j] + kb, sb + TILE_BYTES + j * 4096);                        \
+        }                                                                                           \
+    } while (0)
+
+// direct load n (0..7) of one 32-k step: n -> (operand, j) = (n & 1 ? B : A, n >> 1)
+#define ISSUE_LOAD1(stage, k0, n)                                                                   \
+    do {                                                                                            \
+        const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                              \
+        const uint32_t kb = (uint32_t)(k0) * 2u;                                                     \
+        if (((n) & 1) == 0) dma16(A, aoff[(n) >> 1] + kb, sb + ((n) >> 1) * 4096);                   \
+        else dma16(((n) >> 1) < 2 ? B0 : B1, boff[(n) >> 1] + kb, sb + TILE_BYTES + ((n) >> 1) * 4096); \
+    } while (0)
+
+    // ---- MFMA operand addressing ----
+    const int l32 = lane & 31, lhi = lane >> 5;
+    uint32_t a_rb[NB], b_rb[4];
+    int a_sw[NB], b_sw[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ar = wm * 128 + i * 32 + l32;
+        const int br = FUSED ? ((i >> 1) * 128 + wn * 64 + (i & 1) * 32 + l32) : (wn * 128 + i * 32 + l32);
+        if (i < NB) {
+            a_rb[i] = ar * (BK * 2);
+            a_sw[i] = swz(ar);
+        }
+        b_rb[i] = TILE_BYTES + br * (BK * 2);
+        b_sw[i] = swz(br);
+    }
+#define READ_FRAGS(AF, BF, stage, ks)                                                                       \
+    do {                                                                                                    \
+        if (NBLK > 0) {                                                                                     \
+            const unsigned char *sp = smem + (stage) * STAGE_BYTES;                                          \
+            const int c = (ks) * 2 + lhi;                                                                    \
+            _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                   \
+                AF[i] = *(const bf16x8_t *)(sp + a_rb[i] + ((c ^ a_sw[i]) << 4));                            \
+            _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                    \
+                BF[i] = *(const bf16x8_t *)(sp + b_rb[i] + ((c ^ b_sw[i]) << 4));                            \
+        }                                                                                                   \
+    } while (0)
+#define MFMA4(AF, BF, i)                                                                                     \
+    do {                                                                                                    \
+        if ((i) < NBLK) {                                                                                   \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                    \
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0);        \
+        }                                                                                                   \
+    } while (0)
+#define MFMA16(AF, BF)                                                                                       \
+    do {                                                                                                    \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) MFMA4(AF, BF, i);                                       \
+    } while (0)
+
+    f32x16_t acc[NB][4];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    const int KT = Kd / BK;
+    bf16x8_t af0[NB], bf0[4], af1[NB], bf1[4];
+#define WAITCNT_STR2(n) "s_waitcnt vmcnt(" #n ") lgkmcnt(0)"
+#define WAITCNT_STR(n) WAITCNT_STR2(n)
+
+    // prologue: stages 0..NSTAGE-1 <- steps 0..NSTAGE-1; wait for step 0 only when all were issued
+    for (int st = 0; st < NSTAGE && st < KT; ++st) ISSUE_LOADS(st, st * BK, 0, 4);
+    if (KT >= NSTAGE) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");  // LOADS_PER_STEP * (NSTAGE - 1)
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    READ_FRAGS(af0, bf0, 0, 0);
+
+// One 32-k step on stage `cur`.  The 8 direct loads a wave owes per step are issued one per group of four
+// MFMAs (the address unit is shared by the four waves; a burst of loads would stall the MFMA issue):
+//   LOADS_B: first half of the loads of step kt+NSTAGE, into the stage this step releases at its barrier
+//   LOADS_A: second half of the loads of step kt-1+NSTAGE, into the stage the previous step released
+// STEADY: all loads up to step kt-1+NSTAGE exist, so exactly NSTAGE-2 younger steps may stay in flight at the
+// barrier; otherwise (tail) everything must have landed.
+#define K_STEP(kt, LOADS_A, LOADS_B, STEADY, NEXT)                                                  \
+    do {                                                                                            \
+        const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;                                            \
+        const int prv = cur == 0 ? NSTAGE - 1 : cur - 1;                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                          \
+        READ_FRAGS(af1, bf1, cur, 1);                                                               \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
+        {                                                                                           \
+            if (LOADS_A) ISSUE_LOAD1(prv, ((kt) - 1 + NSTAGE) * BK, 4 + i);                          \
+            MFMA4(af0, bf0, i);                                                                     \
+        }                                                                                           \
+        __builtin_amdgcn_sched_barrier(0);                                                          \
+        /* every wave has taken its last fragments of this stage; the next stage must have landed */ \
+        if (STEADY) asm volatile(WAITCNT_STR(24) ::: "memory"); /* LOADS_PER_STEP * (NSTAGE - 2) */  \
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                            \
+        __syncthreads();                                                                            \
+        if (NEXT) READ_FRAGS(af0, bf0, nxt, 0);                                                     \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
+        {                                                                                           \
+            if (LOADS_B) ISSUE_LOAD1(cur, ((kt) + NSTAGE) * BK, i);                                  \
+            MFMA4(af1, bf1, i);                                                                     \
+        }                                                                                           \
+        cur = nxt;                                                                                  \
+    } while (0)
+
+    int kt = 0, cur = 0;
+    if (KT > NSTAGE) {
+        K_STEP(kt, false, true, true, true);
+        for (kt = 1; kt + NSTAGE < KT; ++kt) K_STEP(kt, true, true, true, true);
+        K_STEP(kt, true, false, true, true);  // kt == KT - NSTAGE: last step of the steady wait count
+        ++kt;
+    } else if (KT == NSTAGE) {
+        K_STEP(kt, false, false, true, true);
+        ++kt;
+    }
+    for (; kt + 1 < KT; ++kt) K_STEP(kt, false, false, false, true);
+    K_STEP(kt, false, false, false, false);
+#undef K_STEP
+
+    // ---- epilogue: lane holds column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4 ----
+#pragma unroll
+    for (int i = 0; i < NBLK; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            if (row >= tl.rows) continue;
+            if (FUSED) {
+                bf16_t *out = (bf16_t *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 64 + l32;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const float h1 = acc[i][j][r], h3 = acc[i][j + 2][r];
+                    out[j * 32] = f32_to_bf16(h1 * __frcp_rn(1.0f + __expf(-h1)) * h3);
+                }
+            } else {
+                float *out = (float *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 128 + l32;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) out[j * 32] = acc[i][j][r];
+            }
+        }
+    }
+#undef ISSUE_LOADS
+#undef ISSUE_LOAD1
+#undef READ_FRAGS
+#undef MFMA4
+#undef MFMA16
 }
 
 template <bool FUSED>
@@ -81,117 +255,13 @@ __global__ __launch_bounds__(256, 1) void experts_bf16_kernel(const bf16_t *__re
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
-
-    // ---- direct-load addressing: wave-load q (0..31) of an operand tile covers rows 8q..8q+7 ----
-    uint32_t aoff[8], boff[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int r = 8 * (wave + 4 * j) + (lane >> 3);
-        const int c = (lane & 7) ^ swz(r);
-        aoff[j] = (uint32_t)(min(r, tl.rows - 1) * Kd + c * 8) * 2u;
-        boff[j] = (uint32_t)((r & 127) * Kd + c * 8) * 2u;
-    }
-#define ISSUE_LOADS(stage, k0)                                                                      \
-    do {                                                                                            \
-        const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                              \
-        const uint32_t kb = (uint32_t)(k0) * 2u;                                                     \
-        _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                \
-        {                                                                                           \
-            dma16(A, aoff[j] + kb, sb + j * 4096);                                                   \
-            dma16(j < 4 ? B0 : B1, boff[j] + kb, sb + TILE_BYTES + j * 4096);                        \
-        }                                                                                           \
-    } while (0)
-
-    // ---- MFMA operand addressing ----
-    const int l32 = lane & 31, lhi = lane >> 5;
-    uint32_t a_rb[4], b_rb[4];
-    int a_sw[4], b_sw[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ar = wm * 128 + i * 32 + l32;
-        const int br = FUSED ? ((i >> 1) * 128 + wn * 64 + (i & 1) * 32 + l32) : (wn * 128 + i * 32 + l32);
-        a_rb[i] = ar * (BK * 2);
-        b_rb[i] = TILE_BYTES + br * (BK * 2);
-        a_sw[i] = swz(ar);
-        b_sw[i] = swz(br);
-    }
-#define READ_FRAGS(AF, BF, stage, ks)                                                                       \
-    do {                                                                                                    \
-        const unsigned char *sp = smem + (stage) * STAGE_BYTES;                                              \
-        const int c = (ks) * 2 + lhi;                                                                        \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                        \
-        {                                                                                                   \
-            AF[i] = *(const bf16x8_t *)(sp + a_rb[i] + ((c ^ a_sw[i]) << 4));                                \
-            BF[i] = *(const bf16x8_t *)(sp + b_rb[i] + ((c ^ b_sw[i]) << 4));                                \
-        }                                                                                                   \
-    } while (0)
-#define MFMA16(AF, BF)                                                                                       \
-    do {                                                                                                    \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)           \
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0);            \
-    } while (0)
-
-    f32x16_t acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    const int KT = Kd / BK;
-    bf16x8_t af0[4], bf0[4], af1[4], bf1[4];
-
-    // prologue: stage 0 <- step 0, stage 1 <- step 1
-    ISSUE_LOADS(0, 0);
-    if (KT > 1) ISSUE_LOADS(1, BK);
-    if (KT > 1) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    READ_FRAGS(af0, bf0, 0, 0);
-
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        __builtin_amdgcn_sched_barrier(0);
-        READ_FRAGS(af1, bf1, cur, 1);
-        MFMA16(af0, bf0);
-        __builtin_amdgcn_sched_barrier(0);
-        READ_FRAGS(af0, bf0, cur, 2);
-        MFMA16(af1, bf1);
-        __builtin_amdgcn_sched_barrier(0);
-        READ_FRAGS(af1, bf1, cur, 3);
-        MFMA16(af0, bf0);
-        __builtin_amdgcn_sched_barrier(0);
-        // every wave has taken its last fragments of this stage; the other stage must have landed
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (kt + 2 < KT) ISSUE_LOADS(cur, (kt + 2) * BK);
-        if (kt + 1 < KT) READ_FRAGS(af0, bf0, cur ^ 1, 0);
-        MFMA16(af1, bf1);
-    }
-
-    // ---- epilogue: lane holds column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4 ----
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-            if (row >= tl.rows) continue;
-            if (FUSED) {
-                bf16_t *out = (bf16_t *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 64 + l32;
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const float h1 = acc[i][j][r], h3 = acc[i][j + 2][r];
-                    out[j * 32] = f32_to_bf16((h1 / (1.0f + __expf(-h1))) * h3);
-                }
-            } else {
-                float *out = (float *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 128 + l32;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) out[j * 32] = acc[i][j][r];
-            }
-        }
+    const int nblk = max(0, min(4, (tl.rows - (wave >> 1) * 128 + 31) >> 5));
+    switch (nblk) {
+        case 4: run_tile<FUSED, 4>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
+        case 3: run_tile<FUSED, 3>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
+        case 2: run_tile<FUSED, 2>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
+        case 1: run_tile<FUSED, 1>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
+        default: run_tile<FUSED, 0>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
     }
 }
 
