@@ -4,19 +4,20 @@
 // (J/engine/nn/layer/llama/LlamaMLPLayer.java:117-130; y = x W^T with W [out,in], J/engine/nn/layer/FullyLayer.java:181,235.)
 //
 // Both operands are K-contiguous ("NT" product), so a lane's 8 consecutive k values are one 16-byte LDS read.
-// Workgroup = 4 waves (2x2), tile 256 rows x 256 MFMA columns x 64 k, each wave 128x128 = 4x4 MFMA blocks with
-// its 256 accumulators in AGPRs (one wave per SIMD).  For the up product the 256 MFMA columns are 128 columns
-// of W1 and the same 128 columns of W3, arranged so that a wave holds h1 and h3 of the same output element and
-// applies silu(h1)*h3 in registers.
+// Workgroup = 8 waves (2 row halves x 4 column quarters, two waves per SIMD so that one computes while the
+// other waits on LDS, on the address unit or at the barrier); tile = 256 rows x 256 MFMA columns, each wave
+// 128x64 = 4x2 MFMA blocks with its 128 accumulators in AGPRs.  For the up product the 256 MFMA columns are
+// 128 columns of W1 and the same 128 columns of W3, arranged so that a wave holds h1 and h3 of the same
+// output element and applies silu(h1)*h3 in registers.
 //
-// Data movement: global -> LDS directly (global_load_lds_dwordx4, no staging registers), two LDS stages of
-// (A 256x64 + B 256x64) bf16 = 128 KiB.  A wave-wide direct load fills 1 KiB of LDS in lane order = 8 rows of
-// 8 16-byte chunks; the XOR swizzle of the chunk index that keeps the MFMA operand reads free of bank conflicts
-// is applied by choosing which global chunk each lane fetches.
-// Pipeline per 64-k step: four phases of 16 MFMAs; the operand fragments of phase p+1 are read from LDS while
-// phase p computes; the one barrier per step sits before the last phase, after which the loads of the step
-// after next are issued into the stage just released and the first fragments of the next step are read, so
-// both latencies are covered by the 16 MFMAs of the last phase.
+// Data movement: global -> LDS directly (global_load_lds_dwordx4, no staging registers) into a ring of five
+// stages of (A 256x32 + B 256x32) bf16 = 160 KiB, i.e. all of a CU's LDS.  A wave-wide direct load fills 1 KiB
+// of LDS in lane order = 16 rows of four 16-byte chunks; the XOR swizzle of the chunk index that keeps the MFMA
+// operand reads free of bank conflicts is applied by choosing which global chunk each lane fetches.
+// Pipeline per 32-k step and wave: two phases of 8 MFMAs; the fragments of the next phase are read from LDS
+// while the current one computes; one barrier per step, after which the stage just read is refilled with the
+// step five ahead.  The direct loads are issued one at a time between MFMAs because the address unit is
+// shared by all waves of the CU and a burst of loads stalls the issuing wave.
 //
 // Scheduling: the dispatch stage leaves a list of row tiles (never straddling two experts; empty experts
 // have none) and the first row tile of every expert; workgroup -> (expert, column tile, row tile) is
@@ -30,11 +31,12 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
 #define BM 256
 #define BK 32
-#define TILE_BYTES (BM * BK * 2)      // one operand tile: 16 KiB
-#define STAGE_BYTES (2 * TILE_BYTES)  // A + B
+#define TILE_BYTES (BM * BK * 2)           // one operand tile: 16 KiB
+#define STAGE_BYTES (2 * TILE_BYTES)       // A + B
 #define NSTAGE 5
 #define SMEM_BYTES (NSTAGE * STAGE_BYTES)  // 160 KiB: all of a CU's LDS
-#define LOADS_PER_STEP 8                   // direct loads a wave issues per 32-k step (4 per operand)
+#define NWAVES 8
+#define LOADS_PER_STEP 4                   // direct loads a wave issues per 32-k step (2 per operand)
 #define NUM_XCD 8
 
 int experts_bf16_tile_m(const omega_moe *, int) { return BM; }
@@ -58,53 +60,44 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
                                          void *Cout, const omega_tile tl, int n0, int N, int Kd, int wave, int lane)
 {
     constexpr int NB = NBLK > 0 ? NBLK : 1;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
 
-    // ---- direct-load addressing: wave-load q (0..15) of an operand tile covers rows 16q..16q+15 ----
-    uint32_t aoff[4], boff[4];
+    // ---- direct-load addressing: wave-load q (0..15) of an operand tile covers rows 16q..16q+15;
+    //      this wave issues q = wave and q = wave + 8 of both operands ----
+    uint32_t aoff[2], boff[2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int r = 16 * (wave + 4 * j) + (lane >> 2);
+    for (int j = 0; j < 2; ++j) {
+        const int r = 16 * (wave + 8 * j) + (lane >> 2);
         const int c = (lane & 3) ^ swz(r);
         aoff[j] = (uint32_t)(min(r, tl.rows - 1) * Kd + c * 8) * 2u;
         boff[j] = (uint32_t)((r & 127) * Kd + c * 8) * 2u;
     }
-// direct loads j0..j1-1 (of 4 per operand) of one 32-k step into a stage
-#define ISSUE_LOADS(stage, k0, j0, j1)                                                              \
-    do {                                                                                            \
-        const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                              \
-        const uint32_t kb = (uint32_t)(k0) * 2u;                                                     \
-        _Pragma("unroll") for (int j = (j0); j < (j1); ++j)                                          \
-        {                                                                                           \
-            dma16(A, aoff[j] + kb, sb + j * 4096);                                                   \
-            dma16(j < 2 ? B0 : B1, boff[j] + kb, sb + TILE_BYTES + j * 4096);                        \
-        }                                                                                           \
-    } while (0)
-
-// direct load n (0..7) of one 32-k step: n -> (operand, j) = (n & 1 ? B : A, n >> 1)
-#define ISSUE_LOAD1(stage, k0, n)                                                                   \
-    do {                                                                                            \
-        const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                              \
-        const uint32_t kb = (uint32_t)(k0) * 2u;                                                     \
-        if (((n) & 1) == 0) dma16(A, aoff[(n) >> 1] + kb, sb + ((n) >> 1) * 4096);                   \
-        else dma16(((n) >> 1) < 2 ? B0 : B1, boff[(n) >> 1] + kb, sb + TILE_BYTES + ((n) >> 1) * 4096); \
+// direct load n (0..3) of one 32-k step: n -> (operand, j) = (n & 1 ? B : A, n >> 1)
+#define ISSUE_LOAD1(stage, k0, n)                                                                          \
+    do {                                                                                                   \
+        const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                                     \
+        const uint32_t kb = (uint32_t)(k0) * 2u;                                                            \
+        if (((n) & 1) == 0) dma16(A, aoff[(n) >> 1] + kb, sb + ((n) >> 1) * 8192);                          \
+        else dma16(((n) >> 1) == 0 ? B0 : B1, boff[(n) >> 1] + kb, sb + TILE_BYTES + ((n) >> 1) * 8192);     \
     } while (0)
 
     // ---- MFMA operand addressing ----
     const int l32 = lane & 31, lhi = lane >> 5;
-    uint32_t a_rb[NB], b_rb[4];
-    int a_sw[NB], b_sw[4];
+    uint32_t a_rb[NB], b_rb[2];
+    int a_sw[NB], b_sw[2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NB; ++i) {
         const int ar = wm * 128 + i * 32 + l32;
-        const int br = FUSED ? ((i >> 1) * 128 + wn * 64 + (i & 1) * 32 + l32) : (wn * 128 + i * 32 + l32);
-        if (i < NB) {
-            a_rb[i] = ar * (BK * 2);
-            a_sw[i] = swz(ar);
-        }
-        b_rb[i] = TILE_BYTES + br * (BK * 2);
-        b_sw[i] = swz(br);
+        a_rb[i] = ar * (BK * 2);
+        a_sw[i] = swz(ar);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        // up product: block 0 = 32 columns of W1, block 1 = the same 32 columns of W3
+        const int br = FUSED ? (j * 128 + wn * 32 + l32) : (wn * 64 + j * 32 + l32);
+        b_rb[j] = TILE_BYTES + br * (BK * 2);
+        b_sw[j] = swz(br);
     }
 #define READ_FRAGS(AF, BF, stage, ks)                                                                       \
     do {                                                                                                    \
@@ -113,48 +106,45 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
             const int c = (ks) * 2 + lhi;                                                                    \
             _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                   \
                 AF[i] = *(const bf16x8_t *)(sp + a_rb[i] + ((c ^ a_sw[i]) << 4));                            \
-            _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                    \
-                BF[i] = *(const bf16x8_t *)(sp + b_rb[i] + ((c ^ b_sw[i]) << 4));                            \
+            _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                    \
+                BF[j] = *(const bf16x8_t *)(sp + b_rb[j] + ((c ^ b_sw[j]) << 4));                            \
         }                                                                                                   \
     } while (0)
-#define MFMA4(AF, BF, i)                                                                                     \
+// the two MFMAs of row block i
+#define MFMA2(AF, BF, i)                                                                                     \
     do {                                                                                                    \
         if ((i) < NBLK) {                                                                                   \
-            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                    \
+            _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                    \
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0);        \
         }                                                                                                   \
     } while (0)
-#define MFMA16(AF, BF)                                                                                       \
-    do {                                                                                                    \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) MFMA4(AF, BF, i);                                       \
-    } while (0)
 
-    f32x16_t acc[NB][4];
+    f32x16_t acc[NB][2];
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     const int KT = Kd / BK;
-    bf16x8_t af0[NB], bf0[4], af1[NB], bf1[4];
-#define WAITCNT_STR2(n) "s_waitcnt vmcnt(" #n ") lgkmcnt(0)"
-#define WAITCNT_STR(n) WAITCNT_STR2(n)
+    bf16x8_t af0[NB], bf0[2], af1[NB], bf1[2];
 
     // prologue: stages 0..NSTAGE-1 <- steps 0..NSTAGE-1; wait for step 0 only when all were issued
-    for (int st = 0; st < NSTAGE && st < KT; ++st) ISSUE_LOADS(st, st * BK, 0, 4);
-    if (KT >= NSTAGE) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");  // LOADS_PER_STEP * (NSTAGE - 1)
+    for (int st = 0; st < NSTAGE && st < KT; ++st) {
+#pragma unroll
+        for (int n = 0; n < LOADS_PER_STEP; ++n) ISSUE_LOAD1(st, st * BK, n);
+    }
+    if (KT >= NSTAGE) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // LOADS_PER_STEP * (NSTAGE - 1)
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     READ_FRAGS(af0, bf0, 0, 0);
 
-// One 32-k step on stage `cur`.  The 8 direct loads a wave owes per step are issued one per group of four
-// MFMAs (the address unit is shared by the four waves; a burst of loads would stall the MFMA issue):
+// One 32-k step on stage `cur`.  The 4 direct loads a wave owes per step are issued one per pair of row blocks:
 //   LOADS_B: first half of the loads of step kt+NSTAGE, into the stage this step releases at its barrier
 //   LOADS_A: second half of the loads of step kt-1+NSTAGE, into the stage the previous step released
-// STEADY: all loads up to step kt-1+NSTAGE exist, so exactly NSTAGE-2 younger steps may stay in flight at the
-// barrier; otherwise (tail) everything must have landed.
+// STEADY: all loads up to step kt-1+NSTAGE exist, so exactly NSTAGE-2 younger steps (12 loads) may stay in
+// flight at the barrier; otherwise (tail) everything must have landed.
 #define K_STEP(kt, LOADS_A, LOADS_B, STEADY, NEXT)                                                  \
     do {                                                                                            \
         const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;                                            \
@@ -163,19 +153,19 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
         READ_FRAGS(af1, bf1, cur, 1);                                                               \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
         {                                                                                           \
-            if (LOADS_A) ISSUE_LOAD1(prv, ((kt) - 1 + NSTAGE) * BK, 4 + i);                          \
-            MFMA4(af0, bf0, i);                                                                     \
+            if (LOADS_A && (i & 1) == 0) ISSUE_LOAD1(prv, ((kt) - 1 + NSTAGE) * BK, 2 + (i >> 1));   \
+            MFMA2(af0, bf0, i);                                                                     \
         }                                                                                           \
         __builtin_amdgcn_sched_barrier(0);                                                          \
         /* every wave has taken its last fragments of this stage; the next stage must have landed */ \
-        if (STEADY) asm volatile(WAITCNT_STR(24) ::: "memory"); /* LOADS_PER_STEP * (NSTAGE - 2) */  \
+        if (STEADY) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");                    \
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                            \
         __syncthreads();                                                                            \
         if (NEXT) READ_FRAGS(af0, bf0, nxt, 0);                                                     \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
         {                                                                                           \
-            if (LOADS_B) ISSUE_LOAD1(cur, ((kt) + NSTAGE) * BK, i);                                  \
-            MFMA4(af1, bf1, i);                                                                     \
+            if (LOADS_B && (i & 1) == 0) ISSUE_LOAD1(cur, ((kt) + NSTAGE) * BK, i >> 1);             \
+            MFMA2(af1, bf1, i);                                                                     \
         }                                                                                           \
         cur = nxt;                                                                                  \
     } while (0)
@@ -185,9 +175,6 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
         K_STEP(kt, false, true, true, true);
         for (kt = 1; kt + NSTAGE < KT; ++kt) K_STEP(kt, true, true, true, true);
         K_STEP(kt, true, false, true, true);  // kt == KT - NSTAGE: last step of the steady wait count
-        ++kt;
-    } else if (KT == NSTAGE) {
-        K_STEP(kt, false, false, true, true);
         ++kt;
     }
     for (; kt + 1 < KT; ++kt) K_STEP(kt, false, false, false, true);
@@ -202,31 +189,26 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
             const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
             if (row >= tl.rows) continue;
             if (FUSED) {
-                bf16_t *out = (bf16_t *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 64 + l32;
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const float h1 = acc[i][j][r], h3 = acc[i][j + 2][r];
-                    out[j * 32] = f32_to_bf16(h1 * __frcp_rn(1.0f + __expf(-h1)) * h3);
-                }
+                bf16_t *out = (bf16_t *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 32 + l32;
+                const float h1 = acc[i][0][r], h3 = acc[i][1][r];
+                out[0] = f32_to_bf16(h1 * __frcp_rn(1.0f + __expf(-h1)) * h3);
             } else {
-                float *out = (float *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 128 + l32;
+                float *out = (float *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 64 + l32;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) out[j * 32] = acc[i][j][r];
+                for (int j = 0; j < 2; ++j) out[j * 32] = acc[i][j][r];
             }
         }
     }
-#undef ISSUE_LOADS
 #undef ISSUE_LOAD1
 #undef READ_FRAGS
-#undef MFMA4
-#undef MFMA16
+#undef MFMA2
 }
 
 template <bool FUSED>
-__global__ __launch_bounds__(256, 1) void experts_bf16_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
-                                                              const bf16_t *__restrict__ Wa, const bf16_t *__restrict__ Wb,
-                                                              void *__restrict__ Cout, const omega_tile *__restrict__ tiles,
-                                                              const int32_t *__restrict__ tile_meta, int G, int N, int Kd)
+__global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
+                                                                   const bf16_t *__restrict__ Wa, const bf16_t *__restrict__ Wb,
+                                                                   void *__restrict__ Cout, const omega_tile *__restrict__ tiles,
+                                                                   const int32_t *__restrict__ tile_meta, int G, int N, int Kd)
 {
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     constexpr int NCOLS = FUSED ? 128 : 256;  // output columns per tile
@@ -255,7 +237,7 @@ __global__ __launch_bounds__(256, 1) void experts_bf16_kernel(const bf16_t *__re
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nblk = max(0, min(4, (tl.rows - (wave >> 1) * 128 + 31) >> 5));
+    const int nblk = max(0, min(4, (tl.rows - (wave >> 2) * 128 + 31) >> 5));
     switch (nblk) {
         case 4: run_tile<FUSED, 4>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
         case 3: run_tile<FUSED, 3>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
@@ -282,13 +264,13 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
     if (which == 0) {
         int grid = m->max_m_tiles * (c.H / 128);
         grid = (grid + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
-        hipLaunchKernelGGL(experts_bf16_kernel<true>, dim3(grid), dim3(256), SMEM_BYTES, s, (const bf16_t *)m->xg,
+        hipLaunchKernelGGL(experts_bf16_kernel<true>, dim3(grid), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
                            (const bf16_t *)x, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, m->tiles, m->tile_meta,
                            G, c.H, c.d);
     } else {
         int grid = m->max_m_tiles * (c.d / 256);
         grid = (grid + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
-        hipLaunchKernelGGL(experts_bf16_kernel<false>, dim3(grid), dim3(256), SMEM_BYTES, s, (const bf16_t *)m->a,
+        hipLaunchKernelGGL(experts_bf16_kernel<false>, dim3(grid), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
                            (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y, m->tiles,
                            m->tile_meta, G, c.d, c.H);
     }
