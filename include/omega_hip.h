@@ -98,13 +98,13 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **out);
 int omega_moe_destroy(omega_moe *moe);
 
-/* Load one weight tensor (layout [out,in] row-major, J/engine/nn/layer/FullyLayer.java:181) from host or
- * device memory, elements of the layer dtype (gate bias: fp32).  expert: 0..E-1 routed, E..E+Es-1
- * shared; ignored for the gate.  Stands in for FullyLayer.loadModel / weight upload
- * (J/engine/nn/layer/FullyLayer.java:854-866). */
+/* Load / read back one weight tensor in the reference's layout ([out,in] row-major,
+ * J/engine/nn/layer/FullyLayer.java:181), elements of the layer dtype (gate bias: fp32), from / to host or
+ * device memory.  expert: 0..E-1 routed, E..E+Es-1 shared; ignored for the gate.  The layer keeps bf16 expert
+ * weights in its own tiled order; these two calls convert.  Stand in for FullyLayer.loadModel / saveModel and
+ * the weight upload (J/engine/nn/layer/FullyLayer.java:854-866). */
 int omega_moe_set_weights(omega_moe *moe, int which, int expert, const void *src, int is_device);
-/* Device address of the layer-owned storage of one weight tensor (for in-place initialisation). */
-int omega_moe_weight_ptr(omega_moe *moe, int which, int expert, void **dptr);
+int omega_moe_get_weights(omega_moe *moe, int which, int expert, void *dst, int is_device);
 
 /* forward(Tensor): x_dev [T,d] -> out_dev [T,d], both of the layer dtype, caller-owned device
  * buffers.  Asynchronous on the context's stream; omega_hip_sync / memcpy_d2h make it visible.
@@ -139,9 +139,10 @@ int omega_moe_get_routing(omega_moe *moe, int T, int32_t *ids, float *w, int32_t
 /* Router intermediates, for tests: runs the router on x_dev and copies logits and probabilities
  * [T,E] to host (blocking).  Overwrites the routing state like omega_moe_router. */
 int omega_moe_get_router_probs(omega_moe *moe, const void *x_dev, int T, float *logits, float *probs);
-/* Device addresses of workspace buffers for inspection: which = 0 xg [T*K,d] (layer dtype),
- * 1 a [T*K+Es*T,H] (layer dtype), 2 y [T*K+Es*T,d] fp32. */
-int omega_moe_workspace_ptr(omega_moe *moe, int which, void **dptr);
+/* Host copy (blocking) of a workspace buffer of the last call, rows in logical order (row dst[p] of pair p,
+ * then T rows per shared expert), row-major: which = 0 xg [T*K,d] (layer dtype), 1 a [T*K+Es*T,H] (layer
+ * dtype), 2 y [T*K+Es*T,d] fp32.  For tests. */
+int omega_moe_get_workspace(omega_moe *moe, int which, int T, void *host_dst);
 
 /* Average duration in milliseconds of the launches of one stage, measured with events on the
  * context's stream: runs `iters` back-to-back repetitions of the stage (0 router, 1 dispatch,

@@ -38,7 +38,7 @@ SIGNATURES = {
     "omega_moe_create": (C.c_int, [C.c_void_p, C.POINTER(MoEConfigStruct), C.POINTER(C.c_void_p)]),
     "omega_moe_destroy": (C.c_int, [C.c_void_p]),
     "omega_moe_set_weights": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
-    "omega_moe_weight_ptr": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]),
+    "omega_moe_get_weights": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
     "omega_moe_forward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "omega_moe_router": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "omega_moe_dispatch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
@@ -48,7 +48,7 @@ SIGNATURES = {
     "omega_moe_combine": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "omega_moe_get_routing": (C.c_int, [C.c_void_p, C.c_int] + [C.c_void_p] * 6),
     "omega_moe_get_router_probs": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
-    "omega_moe_workspace_ptr": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p)]),
+    "omega_moe_get_workspace": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "omega_moe_time_stage": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int,
                                        C.POINTER(C.c_float)]),
     "omega_moe_set_profiling": (C.c_int, [C.c_void_p, C.c_int]),

@@ -153,10 +153,10 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 
 static void moe_free_workspace(omega_moe *m)
 {
-    void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->src_row, m->tiles, m->xg, m->a, m->y};
+    void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y};
     for (void *p : ptrs)
         if (p) hipFree(p);
-    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->src_row = nullptr;
+    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr;
     m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
     m->T_cap = 0;
 }
@@ -164,6 +164,12 @@ static void moe_free_workspace(omega_moe *m)
 static int moe_tile_m(const omega_moe *m, int T)
 {
     return m->cfg.dtype == OMEGA_DTYPE_BF16 ? experts_bf16_tile_m(m, T) : experts_f32_tile_m();
+}
+
+static int moe_max_m_tiles(const omega_moe *m, int T, int bm)
+{
+    const omega_moe_config &c = m->cfg;
+    return (T * c.K) / bm + c.E + c.Es * ceil_div(T, bm);
 }
 
 // Sizes the workspace for T tokens (grow-only, like the named caches of
@@ -175,29 +181,33 @@ static int moe_reserve(omega_moe *m, int T)
     OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
     moe_free_workspace(m);
     const omega_moe_config &c = m->cfg;
-    const size_t P = (size_t)T * c.K, R = P + (size_t)c.Es * T;
+    const size_t P = (size_t)T * c.K;
     const int n_tok_tiles = ceil_div(T, ROUTER_TOK_TILE);
-    // smallest row tile any kernel variant uses bounds the tile list
-    const int bm_min = c.dtype == OMEGA_DTYPE_BF16 ? 32 : experts_f32_tile_m();
-    const int max_tiles = (int)(P / bm_min) + c.E + c.Es * ceil_div(T, bm_min);
+    const int bm = moe_tile_m(m, T);
+    // every expert's rows start on a row-tile boundary: the buffers hold whole tiles
+    m->tiles_cap = moe_max_m_tiles(m, T, bm);
+    m->rows_cap = (size_t)m->tiles_cap * bm;
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->ids, P * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->w, P * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_counts, (size_t)n_tok_tiles * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_base, (size_t)n_tok_tiles * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->dst, P * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->dstp, P * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->src_row, P * 4));
-    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tiles, (size_t)max_tiles * sizeof(omega_tile)));
-    OMEGA_HIP_CHECK(ctx, hipMalloc(&m->xg, P * c.d * m->esize));
-    OMEGA_HIP_CHECK(ctx, hipMalloc(&m->a, R * c.H * m->esize));
-    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->y, R * c.d * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tiles, (size_t)m->tiles_cap * sizeof(omega_tile)));
+    OMEGA_HIP_CHECK(ctx, hipMalloc(&m->xg, m->rows_cap * c.d * m->esize));
+    OMEGA_HIP_CHECK(ctx, hipMalloc(&m->a, m->rows_cap * c.H * m->esize));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->y, m->rows_cap * c.d * 4));
+    // padding rows of xg / a are read by the product kernels (their results are discarded): keep them finite
+    OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->xg, 0, m->rows_cap * c.d * m->esize, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->a, 0, m->rows_cap * c.H * m->esize, ctx->stream));
+    if (c.dtype == OMEGA_DTYPE_BF16 && c.Es > 0) {
+        const size_t xs_rows = (size_t)ceil_div(T, bm) * bm;
+        OMEGA_HIP_CHECK(ctx, hipMalloc(&m->xs, xs_rows * c.d * m->esize));
+        OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->xs, 0, xs_rows * c.d * m->esize, ctx->stream));
+    }
     m->T_cap = T;
     return OMEGA_OK;
-}
-
-static int moe_max_m_tiles(const omega_moe *m, int T, int bm)
-{
-    const omega_moe_config &c = m->cfg;
-    return (T * c.K) / bm + c.E + c.Es * ceil_div(T, bm);
 }
 
 int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **out)
@@ -308,6 +318,13 @@ static int weight_slot(omega_moe *m, int which, int expert, void **ptr, size_t *
     }
 }
 
+static bool weight_is_packed(const omega_moe *m, int which)
+{
+    return m->cfg.dtype == OMEGA_DTYPE_BF16 && (which == OMEGA_W_W1 || which == OMEGA_W_W3 || which == OMEGA_W_W2);
+}
+
+// bf16 expert weights are stored as the packed tile image the product kernels load (pack.h); the caller
+// always sees the [out,in] row-major layout of J/engine/nn/layer/FullyLayer.java:181.
 int omega_moe_set_weights(omega_moe *m, int which, int expert, const void *src, int is_device)
 {
     if (!m) OMEGA_FAIL(nullptr, OMEGA_ERR_INVALID_ARG, "NULL layer");
@@ -316,19 +333,46 @@ int omega_moe_set_weights(omega_moe *m, int which, int expert, const void *src, 
     void *p; size_t bytes;
     if (!src || weight_slot(m, which, expert, &p, &bytes) != OMEGA_OK)
         OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "set_weights: bad kind, expert index or source");
-    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(p, src, bytes, is_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream));
-    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    if (!weight_is_packed(m, which)) {
+        OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(p, src, bytes, is_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+        return OMEGA_OK;
+    }
+    const int R = which == OMEGA_W_W2 ? m->cfg.d : m->cfg.H, Kd = which == OMEGA_W_W2 ? m->cfg.H : m->cfg.d;
+    void *stage = nullptr;
+    if (!is_device) {
+        OMEGA_HIP_CHECK(ctx, hipMalloc(&stage, bytes));
+        hipError_t e = hipMemcpyAsync(stage, src, bytes, hipMemcpyHostToDevice, ctx->stream);
+        if (e != hipSuccess) { hipFree(stage); OMEGA_HIP_CHECK(ctx, e); }
+    }
+    hipError_t e = launch_pack_rows(p, is_device ? src : stage, R, Kd, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (stage) hipFree(stage);
+    OMEGA_HIP_CHECK(ctx, e);
     return OMEGA_OK;
 }
 
-int omega_moe_weight_ptr(omega_moe *m, int which, int expert, void **dptr)
+int omega_moe_get_weights(omega_moe *m, int which, int expert, void *dst, int is_device)
 {
     if (!m) OMEGA_FAIL(nullptr, OMEGA_ERR_INVALID_ARG, "NULL layer");
     omega_ctx *ctx = m->ctx;
     CTX_ENTER(ctx);
-    size_t bytes;
-    if (!dptr || weight_slot(m, which, expert, dptr, &bytes) != OMEGA_OK)
-        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "weight_ptr: bad kind or expert index");
+    void *p; size_t bytes;
+    if (!dst || weight_slot(m, which, expert, &p, &bytes) != OMEGA_OK)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_weights: bad kind, expert index or destination");
+    if (!weight_is_packed(m, which)) {
+        OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(dst, p, bytes, is_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+        return OMEGA_OK;
+    }
+    const int R = which == OMEGA_W_W2 ? m->cfg.d : m->cfg.H, Kd = which == OMEGA_W_W2 ? m->cfg.H : m->cfg.d;
+    void *stage = nullptr;
+    if (!is_device) OMEGA_HIP_CHECK(ctx, hipMalloc(&stage, bytes));
+    hipError_t e = launch_unpack_rows(is_device ? dst : stage, p, R, Kd, ctx->stream);
+    if (e == hipSuccess && !is_device) e = hipMemcpyAsync(dst, stage, bytes, hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (stage) hipFree(stage);
+    OMEGA_HIP_CHECK(ctx, e);
     return OMEGA_OK;
 }
 
@@ -353,6 +397,7 @@ static int stage_dispatch(omega_moe *m, const void *x, int T)
     const int bm = moe_tile_m(m, T);
     m->bm = bm;
     m->max_m_tiles = moe_max_m_tiles(m, T, bm);
+    if (m->max_m_tiles > m->tiles_cap) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: workspace too small for this T");
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));
     return OMEGA_OK;
@@ -535,11 +580,43 @@ int omega_moe_get_router_probs(omega_moe *m, const void *x, int T, float *logits
     return OMEGA_OK;
 }
 
-int omega_moe_workspace_ptr(omega_moe *m, int which, void **dptr)
+// Host copy of a workspace buffer in logical row order (row r of expert e = offsets[e] + rank), row-major:
+// the padding between experts and the packed tile image of bf16 layers are undone here.
+int omega_moe_get_workspace(omega_moe *m, int which, int T, void *host_dst)
 {
     MOE_ENTER(m);
-    if (!dptr || which < 0 || which > 2) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "workspace_ptr: bad selector");
-    *dptr = which == 0 ? m->xg : which == 1 ? m->a : (void *)m->y;
+    if (!host_dst || which < 0 || which > 2 || T <= 0 || T > m->T_cap || m->bm == 0)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_workspace: bad selector, T, or no dispatch has run");
+    const omega_moe_config &c = m->cfg;
+    const int G = c.E + c.Es, bm = m->bm;
+    const int cols = which == 1 ? c.H : c.d;
+    const size_t es = which == 2 ? 4 : m->esize;
+    const bool packed = c.dtype == OMEGA_DTYPE_BF16 && which != 2;
+    const void *src = which == 0 ? m->xg : which == 1 ? m->a : (const void *)m->y;
+    const size_t bytes = m->rows_cap * cols * es;
+    std::vector<int32_t> meta(G + 2), off(c.E + 1);
+    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(meta.data(), m->tile_meta, meta.size() * 4, hipMemcpyDeviceToHost, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(off.data(), m->offsets, off.size() * 4, hipMemcpyDeviceToHost, ctx->stream));
+    void *stage = nullptr;
+    if (packed) {
+        OMEGA_HIP_CHECK(ctx, hipMalloc(&stage, bytes));
+        hipError_t e = launch_unpack_rows(stage, src, (int)m->rows_cap, cols, ctx->stream);
+        if (e != hipSuccess) { hipFree(stage); OMEGA_HIP_CHECK(ctx, e); }
+        src = stage;
+    }
+    std::vector<unsigned char> raw(bytes);
+    hipError_t e = hipMemcpyAsync(raw.data(), src, bytes, hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (stage) hipFree(stage);
+    OMEGA_HIP_CHECK(ctx, e);
+    const size_t rb = (size_t)cols * es, P = (size_t)T * c.K;
+    unsigned char *out = (unsigned char *)host_dst;
+    const int groups = which == 0 ? c.E : G;  // xg holds routed rows only
+    for (int g = 0; g < groups; ++g) {
+        const size_t rows = g < c.E ? (size_t)(off[g + 1] - off[g]) : (size_t)T;
+        const size_t l0 = g < c.E ? (size_t)off[g] : P + (size_t)(g - c.E) * T;
+        memcpy(out + l0 * rb, raw.data() + (size_t)meta[1 + g] * bm * rb, rows * rb);
+    }
     return OMEGA_OK;
 }
 

@@ -1,4 +1,5 @@
-// Combine: out[t,:] = sum_j w[t,j] * y[dst[t*K+j],:] in slot order, then + the shared experts' rows.
+// Combine: out[t,:] = sum_j w[t,j] * y[row of pair t*K+j,:] in slot order, then + the shared experts' rows
+// (rows are the physical rows the dispatch stage assigned; shared expert s owns rows first_tile[E+s]*bm + t).
 // One wave per token; each lane owns 4 (fp32 out) or 8 (bf16 out) consecutive columns, read from the
 // fp32 rows of y with 16-byte loads; products and sums are separate fp32 operations in slot order
 // (this file is compiled with -ffp-contract=off), the weighted sum of add_mul_kernel
@@ -10,7 +11,8 @@
 
 template <int VEC, bool BF16>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ dst,
-                                                      const float *__restrict__ w, int T, int K, int d, int Es, int P,
+                                                      const float *__restrict__ w, int T, int K, int d, int Es,
+                                                      const int32_t *__restrict__ tile_meta, int E, int bm,
                                                       void *__restrict__ out)
 {
     const int lane = threadIdx.x & 63;
@@ -42,7 +44,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
             }
         }
         for (int s = 0; s < Es; ++s) {
-            const float4 *src = (const float4 *)(y + ((size_t)P + (size_t)s * T + t) * d + c0);
+            const float4 *src = (const float4 *)(y + ((size_t)tile_meta[1 + E + s] * bm + t) * d + c0);
 #pragma unroll
             for (int q = 0; q < VEC / 4; ++q) {
                 const float4 v4 = src[q];
@@ -70,7 +72,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
 template <bool BF16>
 __global__ __launch_bounds__(256) void combine_scalar_kernel(const float *__restrict__ y, const int32_t *__restrict__ dst,
                                                              const float *__restrict__ w, int T, int K, int d, int Es,
-                                                             int P, void *__restrict__ out)
+                                                             const int32_t *__restrict__ tile_meta, int E, int bm,
+                                                             void *__restrict__ out)
 {
     const int t = blockIdx.x;
     for (int c = threadIdx.x; c < d; c += 256) {
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(256) void combine_scalar_kernel(const float *__rest
             const float term = w[(size_t)t * K + j] * y[(size_t)dst[(size_t)t * K + j] * d + c];
             acc = acc + term;
         }
-        for (int s = 0; s < Es; ++s) acc = acc + y[((size_t)P + (size_t)s * T + t) * d + c];
+        for (int s = 0; s < Es; ++s) acc = acc + y[((size_t)tile_meta[1 + E + s] * bm + t) * d + c];
         if (BF16) ((bf16_t *)out)[(size_t)t * d + c] = f32_to_bf16(acc);
         else ((float *)out)[(size_t)t * d + c] = acc;
     }
@@ -88,23 +91,22 @@ __global__ __launch_bounds__(256) void combine_scalar_kernel(const float *__rest
 hipError_t launch_combine(const omega_moe *m, int T, void *out, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
-    const int P = T * c.K;
     const bool bf = c.dtype == OMEGA_DTYPE_BF16;
     const int vec = bf ? 8 : 4;
     if (c.d % vec == 0 && ((uintptr_t)out % 16) == 0 && c.K <= MAXK) {
         if (bf)
-            hipLaunchKernelGGL((combine_kernel<8, true>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dst, m->w, T,
-                               c.K, c.d, c.Es, P, out);
+            hipLaunchKernelGGL((combine_kernel<8, true>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dstp, m->w, T,
+                               c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, out);
         else
-            hipLaunchKernelGGL((combine_kernel<4, false>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dst, m->w, T,
-                               c.K, c.d, c.Es, P, out);
+            hipLaunchKernelGGL((combine_kernel<4, false>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dstp, m->w, T,
+                               c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, out);
     } else {
         if (bf)
-            hipLaunchKernelGGL(combine_scalar_kernel<true>, dim3(T), dim3(256), 0, s, m->y, m->dst, m->w, T, c.K, c.d,
-                               c.Es, P, out);
+            hipLaunchKernelGGL(combine_scalar_kernel<true>, dim3(T), dim3(256), 0, s, m->y, m->dstp, m->w, T, c.K, c.d,
+                               c.Es, m->tile_meta, c.E, m->bm, out);
         else
-            hipLaunchKernelGGL(combine_scalar_kernel<false>, dim3(T), dim3(256), 0, s, m->y, m->dst, m->w, T, c.K, c.d,
-                               c.Es, P, out);
+            hipLaunchKernelGGL(combine_scalar_kernel<false>, dim3(T), dim3(256), 0, s, m->y, m->dstp, m->w, T, c.K, c.d,
+                               c.Es, m->tile_meta, c.E, m->bm, out);
     }
     return hipGetLastError();
 }

@@ -20,11 +20,16 @@ struct omega_ctx {
 };
 
 // One entry per row tile of the grouped products: written on the device by the scan kernel.
+// Rows of the expert-contiguous buffers xg / a / y are "physical" rows: expert g owns the row tiles
+// first_tile[g] .. first_tile[g+1]-1, each bm rows high, so every expert starts on a tile boundary and the
+// row tile with list index i covers physical rows i*bm .. i*bm+rows-1 (the rest of the tile is padding that
+// is never computed).  The logical row of a pair (offsets[e] + rank, what get_routing reports) and its
+// physical row (first_tile[e]*bm + rank) differ only by that padding.
 struct __attribute__((aligned(16))) omega_tile {
     int32_t g;      // weight index: 0..E-1 routed, E..E+Es-1 shared
-    int32_t row0;   // first row in the a / y buffers (and in xg for routed experts)
-    int32_t rows;   // valid rows in this tile (1..BM)
-    int32_t xrow0;  // -1: A operand of the up product is xg[row0..]; >=0: it is x[xrow0..] (shared expert)
+    int32_t row0;   // first physical row (= list index * bm)
+    int32_t rows;   // valid rows in this tile (1..bm)
+    int32_t xrow0;  // -1: routed expert; >=0: shared expert, first token of this tile (A operand = x rows)
 };
 
 struct omega_moe {
@@ -47,13 +52,17 @@ struct omega_moe {
     int32_t *tile_base = nullptr;    // [n_tok_tiles,E] exclusive prefix of tile_counts over the tiles (scan)
     int32_t *counts = nullptr;       // [E]
     int32_t *offsets = nullptr;      // [E+1]
-    int32_t *dst = nullptr;          // [T*K]
+    int32_t *dst = nullptr;          // [T*K] logical row of each pair
+    int32_t *dstp = nullptr;         // [T*K] physical row of each pair
     int32_t *src_row = nullptr;      // [T*K]
     omega_tile *tiles = nullptr;     // [max_m_tiles]
     int32_t *tile_meta = nullptr;    // [0] = number of row tiles; [1+g] = first row tile of group g (G+1 entries)
-    void *xg = nullptr;              // [T*K,d]
-    void *a = nullptr;               // [T*K+Es*T,H]
-    float *y = nullptr;              // [T*K+Es*T,d]
+    void *xg = nullptr;              // [rows_cap,d]  gathered tokens (bf16: packed tile image, see pack.h)
+    void *xs = nullptr;              // bf16 with shared experts: packed copy of x, [ceil(T/bm)*bm,d]
+    void *a = nullptr;               // [rows_cap,H]  (bf16: packed tile image)
+    float *y = nullptr;              // [rows_cap,d]  row-major fp32
+    size_t rows_cap = 0;             // physical rows the buffers hold: tile capacity * bm
+    int tiles_cap = 0;               // entries of `tiles`
     int max_m_tiles = 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     // per-stage event profiling of forward calls (6 events per call), off by default
@@ -88,6 +97,8 @@ hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipS
 hipError_t launch_experts_f32(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
 hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
 hipError_t launch_combine(const omega_moe *m, int T, void *out, hipStream_t s);
+hipError_t launch_pack_rows(void *dst_packed, const void *src_rowmajor, int R, int Kd, hipStream_t s);
+hipError_t launch_unpack_rows(void *dst_rowmajor, const void *src_packed, int R, int Kd, hipStream_t s);
 int experts_bf16_tile_m(const omega_moe *m, int T);
 int experts_f32_tile_m(void);
 hipError_t experts_bf16_init(void);

@@ -12,8 +12,10 @@
 //
 // Data movement: global -> LDS directly (global_load_lds_dwordx4, no staging registers) into a ring of five
 // stages of (A 256x32 + B 256x32) bf16 = 160 KiB, i.e. all of a CU's LDS.  A wave-wide direct load fills 1 KiB
-// of LDS in lane order = 16 rows of four 16-byte chunks; the XOR swizzle of the chunk index that keeps the MFMA
-// operand reads free of bank conflicts is applied by choosing which global chunk each lane fetches.
+// of LDS in lane order = 16 rows of four 16-byte chunks.  All three operands (weights, xg, a) are kept in
+// memory as that very image (pack.h: 1 KiB blocks of 16 rows x 32 k with the chunk index XOR-swizzled so the
+// MFMA operand reads are free of bank conflicts), so every direct load reads 1 KiB of contiguous memory.
+// The weights are packed once when they are set, xg by the gather kernel, a by the up product's epilogue.
 // Pipeline per 32-k step and wave: two phases of 8 MFMAs; the fragments of the next phase are read from LDS
 // while the current one computes; one barrier per step, after which the stage just read is refilled with the
 // step five ahead.  The direct loads are issued one at a time between MFMAs because the address unit is
@@ -25,6 +27,7 @@
 // weight tiles in its L2.  Consecutive workgroup ids go round-robin over the 8 XCDs, so the id is first
 // remapped to give each XCD a contiguous run of tiles.
 #include "common.h"
+#include "pack.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -41,9 +44,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
 int experts_bf16_tile_m(const omega_moe *, int) { return BM; }
 
-// swizzle of the 16-byte chunk index (4 chunks per 64-byte row): free of bank conflicts for 8 consecutive
-// rows on 32 banks and for 16 consecutive rows on 64 banks
-__device__ __forceinline__ int swz(int row) { return ((row >> 1) ^ (row >> 3)) & 3; }
+__device__ __forceinline__ int swz(int row) { return pk_swz(row); }
 
 // 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16*l.
 __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_base)
@@ -55,31 +56,29 @@ __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t
 // One output tile.  NBLK = number of 32-row blocks of this wave that hold valid rows (the others are never
 // computed: a ragged last row tile of an expert costs only the blocks it fills).  NBLK == 0: the wave only
 // takes part in the loads and barriers.
+// A: packed row group of the tile's first row; B0/B1: packed row groups of the two 128-row halves of the B tile.
 template <bool FUSED, int NBLK>
-__device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, const bf16_t *B0, const bf16_t *B1,
-                                         void *Cout, const omega_tile tl, int n0, int N, int Kd, int wave, int lane)
+__device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned char *A, const unsigned char *B0,
+                                         const unsigned char *B1, void *Cout, const omega_tile tl, int n0, int N, int Kd,
+                                         int wave, int lane)
 {
     constexpr int NB = NBLK > 0 ? NBLK : 1;
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
 
-    // ---- direct-load addressing: wave-load q (0..15) of an operand tile covers rows 16q..16q+15;
-    //      this wave issues q = wave and q = wave + 8 of both operands ----
-    uint32_t aoff[2], boff[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int r = 16 * (wave + 8 * j) + (lane >> 2);
-        const int c = (lane & 3) ^ swz(r);
-        aoff[j] = (uint32_t)(min(r, tl.rows - 1) * Kd + c * 8) * 2u;
-        boff[j] = (uint32_t)((r & 127) * Kd + c * 8) * 2u;
-    }
-// direct load n (0..3) of one 32-k step: n -> (operand, j) = (n & 1 ? B : A, n >> 1)
-#define ISSUE_LOAD1(stage, k0, n)                                                                          \
+    const int KT = Kd / BK;
+    // ---- direct-load addressing: wave-load q (0..15) of an operand tile is the packed block q % 8 of row
+    //      group q / 8; this wave issues q = wave and q = wave + 8 of both operands.  Consecutive k steps of
+    //      a row group are 8 KiB apart. ----
+    const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
+    const uint32_t a_rg1 = (uint32_t)KT * 8192u;  // second row group of the A tile
+// direct load n (0..3) of one 32-k step: n -> (operand, row group) = (n & 1 ? B : A, n >> 1)
+#define ISSUE_LOAD1(stage, kstep, n)                                                                       \
     do {                                                                                                   \
         const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                                     \
-        const uint32_t kb = (uint32_t)(k0) * 2u;                                                            \
-        if (((n) & 1) == 0) dma16(A, aoff[(n) >> 1] + kb, sb + ((n) >> 1) * 8192);                          \
-        else dma16(((n) >> 1) == 0 ? B0 : B1, boff[(n) >> 1] + kb, sb + TILE_BYTES + ((n) >> 1) * 8192);     \
+        const uint32_t kb = (uint32_t)(kstep) * 8192u + blk_off;                                            \
+        if (((n) & 1) == 0) dma16(A, kb + (((n) >> 1) ? a_rg1 : 0u), sb + ((n) >> 1) * 8192);               \
+        else dma16(((n) >> 1) == 0 ? B0 : B1, kb, sb + TILE_BYTES + ((n) >> 1) * 8192);                      \
     } while (0)
 
     // ---- MFMA operand addressing ----
@@ -110,12 +109,15 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
                 BF[j] = *(const bf16x8_t *)(sp + b_rb[j] + ((c ^ b_sw[j]) << 4));                            \
         }                                                                                                   \
     } while (0)
-// the two MFMAs of row block i
+// the two MFMAs of row block i.  The up product feeds the weights as the first operand, so that a lane ends
+// up with 4 consecutive output columns of one row (8 bytes of the packed `a`), the down product the rows, so
+// that 32 lanes hold 32 consecutive columns of one row of y.
 #define MFMA2(AF, BF, i)                                                                                     \
     do {                                                                                                    \
         if ((i) < NBLK) {                                                                                   \
             _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                    \
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0);        \
+                acc[i][j] = FUSED ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(BF[j], AF[i], acc[i][j], 0, 0, 0) \
+                                  : __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0); \
         }                                                                                                   \
     } while (0)
 
@@ -127,13 +129,12 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    const int KT = Kd / BK;
     bf16x8_t af0[NB], bf0[2], af1[NB], bf1[2];
 
     // prologue: stages 0..NSTAGE-1 <- steps 0..NSTAGE-1; wait for step 0 only when all were issued
     for (int st = 0; st < NSTAGE && st < KT; ++st) {
 #pragma unroll
-        for (int n = 0; n < LOADS_PER_STEP; ++n) ISSUE_LOAD1(st, st * BK, n);
+        for (int n = 0; n < LOADS_PER_STEP; ++n) ISSUE_LOAD1(st, st, n);
     }
     if (KT >= NSTAGE) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // LOADS_PER_STEP * (NSTAGE - 1)
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -153,7 +154,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
         READ_FRAGS(af1, bf1, cur, 1);                                                               \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
         {                                                                                           \
-            if (LOADS_A && (i & 1) == 0) ISSUE_LOAD1(prv, ((kt) - 1 + NSTAGE) * BK, 2 + (i >> 1));   \
+            if (LOADS_A && (i & 1) == 0) ISSUE_LOAD1(prv, (kt) - 1 + NSTAGE, 2 + (i >> 1));     \
             MFMA2(af0, bf0, i);                                                                     \
         }                                                                                           \
         __builtin_amdgcn_sched_barrier(0);                                                          \
@@ -164,7 +165,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
         if (NEXT) READ_FRAGS(af0, bf0, nxt, 0);                                                     \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
         {                                                                                           \
-            if (LOADS_B && (i & 1) == 0) ISSUE_LOAD1(cur, ((kt) + NSTAGE) * BK, i >> 1);             \
+            if (LOADS_B && (i & 1) == 0) ISSUE_LOAD1(cur, (kt) + NSTAGE, i >> 1);               \
             MFMA2(af1, bf1, i);                                                                     \
         }                                                                                           \
         cur = nxt;                                                                                  \
@@ -181,18 +182,43 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const bf16_t *A, c
     K_STEP(kt, false, false, false, false);
 #undef K_STEP
 
-    // ---- epilogue: lane holds column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4 ----
+    // ---- epilogue ----
+    if (FUSED) {
+        // lane: row l32 of block i; register r -> column 8*(r/4) + 4*lhi + r%4 of the wave's 32 columns, which are
+        // one k step of the packed `a` (K dimension = N): chunk r/4, bytes lhi*8 .. lhi*8+7
+        const int KTa = N / BK;
+        const int kba = (n0 >> 5) + wn;
 #pragma unroll
-    for (int i = 0; i < NBLK; ++i) {
+        for (int i = 0; i < NBLK; ++i) {
+            const int row = wm * 128 + i * 32 + l32;
+            if (row < tl.rows) {
+                const int prow = tl.row0 + row;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-            if (row >= tl.rows) continue;
-            if (FUSED) {
-                bf16_t *out = (bf16_t *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 32 + l32;
-                const float h1 = acc[i][0][r], h3 = acc[i][1][r];
-                out[0] = f32_to_bf16(h1 * __frcp_rn(1.0f + __expf(-h1)) * h3);
-            } else {
+                for (int t = 0; t < 4; ++t) {
+                    uint32_t pk[2];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        float v[2];
+#pragma unroll
+                        for (int u = 0; u < 2; ++u) {
+                            const float h1 = acc[i][0][t * 4 + h * 2 + u], h3 = acc[i][1][t * 4 + h * 2 + u];
+                            v[u] = h1 * __frcp_rn(1.0f + __expf(-h1)) * h3;
+                        }
+                        pk[h] = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+                    }
+                    uint2 o = {pk[0], pk[1]};
+                    *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, kba, t, KTa) + lhi * 8) = o;
+                }
+            }
+        }
+    } else {
+        // lane: column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4
+#pragma unroll
+        for (int i = 0; i < NBLK; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                if (row >= tl.rows) continue;
                 float *out = (float *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 64 + l32;
 #pragma unroll
                 for (int j = 0; j < 2; ++j) out[j * 32] = acc[i][j][r];
@@ -231,9 +257,13 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
     const omega_tile tl = tiles[mt0 + (l % Mg)];
     const int n0 = nt * NCOLS;
 
-    const bf16_t *A = (FUSED && tl.xrow0 >= 0) ? Ax + (size_t)tl.xrow0 * Kd : Axg + (size_t)tl.row0 * Kd;
-    const bf16_t *B0 = Wa + ((size_t)tl.g * N + n0) * Kd;
-    const bf16_t *B1 = FUSED ? Wb + ((size_t)tl.g * N + n0) * Kd : B0 + (size_t)128 * Kd;
+    // packed operands: a row group (128 rows) occupies KT * 8 KiB
+    const size_t rg_bytes = (size_t)(Kd / BK) * 8192;
+    const unsigned char *A = (FUSED && tl.xrow0 >= 0) ? (const unsigned char *)Ax + (size_t)(tl.xrow0 >> 7) * rg_bytes
+                                                      : (const unsigned char *)Axg + (size_t)(tl.row0 >> 7) * rg_bytes;
+    const size_t wrg = (size_t)tl.g * (N >> 7) + (n0 >> 7);  // row group of the weight tile
+    const unsigned char *B0 = (const unsigned char *)Wa + wrg * rg_bytes;
+    const unsigned char *B1 = FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : B0 + rg_bytes;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -265,7 +295,7 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
         int grid = m->max_m_tiles * (c.H / 128);
         grid = (grid + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
         hipLaunchKernelGGL(experts_bf16_kernel<true>, dim3(grid), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
-                           (const bf16_t *)x, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, m->tiles, m->tile_meta,
+                           (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, m->tiles, m->tile_meta,
                            G, c.H, c.d);
     } else {
         int grid = m->max_m_tiles * (c.d / 256);

@@ -140,22 +140,22 @@ class MoELayer:
         self._upload(L.W_W3, g, W3)
         self._upload(L.W_W2, g, W2)
 
-    def weight_ptr(self, which, expert=0):
-        p = C.c_void_p()
-        self.ctx.check(self.lib.omega_moe_weight_ptr(self.handle, which, expert, C.byref(p)))
-        return p
-
     def init_synthetic(self, seed, cfgmod, cfg):
-        """Fills every weight in place on the device from the seeded generator (see configs.py)."""
+        """Fills every weight on the device from the seeded generator (see configs.py): each tensor is drawn
+        into a row-major scratch buffer and handed to set_weights as a device source."""
         dt = L.DTYPE_BF16 if self.dtype == "bf16" else L.DTYPE_F32
         fill = self.lib.omega_hip_fill_normal
         n_w = self.hidden * self.embedDim
-        self.ctx.check(fill(self.ctx.handle, self.weight_ptr(L.W_GATE), self.nExperts * self.embedDim, seed,
-                            cfgmod.STREAM_WG, cfgmod.tensor_std(cfg, "Wg"), 0, dt))
+        tmp = DeviceBuffer(self.ctx, (max(n_w, self.nExperts * self.embedDim),), self.dtype)
+        self.ctx.check(fill(self.ctx.handle, tmp.ptr, self.nExperts * self.embedDim, seed, cfgmod.STREAM_WG,
+                            cfgmod.tensor_std(cfg, "Wg"), 0, dt))
+        self.ctx.check(self.lib.omega_moe_set_weights(self.handle, L.W_GATE, 0, tmp.ptr, 1))
         for g in range(self.nExperts + self.nShared):
             for which, name in ((L.W_W1, "W1"), (L.W_W3, "W3"), (L.W_W2, "W2")):
-                self.ctx.check(fill(self.ctx.handle, self.weight_ptr(which, g), n_w, seed,
-                                    cfgmod.expert_stream(g, name), cfgmod.tensor_std(cfg, name), 0, dt))
+                self.ctx.check(fill(self.ctx.handle, tmp.ptr, n_w, seed, cfgmod.expert_stream(g, name),
+                                    cfgmod.tensor_std(cfg, name), 0, dt))
+                self.ctx.check(self.lib.omega_moe_set_weights(self.handle, which, g, tmp.ptr, 1))
+        tmp.free()
         bg = cfgmod.zipf_gate_bias(cfg, seed)
         if bg is not None:
             self._upload(L.W_GATE_BIAS, 0, bg)
@@ -240,23 +240,21 @@ class MoELayer:
         return lg, p
 
     def workspace(self, which, T):
-        """Host copy of a workspace buffer: 'xg' [T*K,d], 'a' [T*K+Es*T,H], 'y' [T*K+Es*T,d] (fp32 values)."""
+        """Host copy of a workspace buffer in logical row order: 'xg' [T*K,d], 'a' [T*K+Es*T,H],
+        'y' [T*K+Es*T,d] (fp32 values)."""
         idx = {"xg": 0, "a": 1, "y": 2}[which]
-        p = C.c_void_p()
-        self.ctx.check(self.lib.omega_moe_workspace_ptr(self.handle, idx, C.byref(p)))
         P, R = T * self.topK, T * self.topK + self.nShared * T
         shape = {"xg": (P, self.embedDim), "a": (R, self.hidden), "y": (R, self.embedDim)}[which]
         raw_bf16 = self.dtype == "bf16" and which != "y"
-        h = np.empty(shape, np.uint16 if raw_bf16 else np.float32)
-        self.ctx.check(self.lib.omega_hip_memcpy_d2h(self.ctx.handle, h.ctypes.data, p, h.nbytes))
+        h = np.zeros(shape, np.uint16 if raw_bf16 else np.float32)
+        self.ctx.check(self.lib.omega_moe_get_workspace(self.handle, idx, T, h.ctypes.data))
         return bf16_bits_to_f32(h) if raw_bf16 else h
 
     # ---- checkpoint: raw LE float32, order gate, (gate bias), then w1,w3,w2 per expert, routed then shared
     def _download_weight(self, which, expert, shape):
-        p = self.weight_ptr(which, expert)
         raw_bf16 = self.dtype == "bf16" and which != L.W_GATE_BIAS
         h = np.empty(shape, np.uint16 if raw_bf16 else np.float32)
-        self.ctx.check(self.lib.omega_hip_memcpy_d2h(self.ctx.handle, h.ctypes.data, p, h.nbytes))
+        self.ctx.check(self.lib.omega_moe_get_weights(self.handle, which, expert, h.ctypes.data, 0))
         return bf16_bits_to_f32(h) if raw_bf16 else h
 
     def _param_list(self):
