@@ -2,7 +2,7 @@
 //
 // One workgroup (256 threads) routes a tile of 32 tokens.
 //  phase 1  logits[t,e] = sum_k x[t,k]*Wg[e,k] (+bg[e]): one lane per (token, expert); x and Wg are
-//           staged through LDS in chunks of 64 k.  EXACT mode adds the products one k at a time with
+//           staged through LDS in chunks of 64..256 k.  EXACT mode adds the products one k at a time with
 //           a separate multiply and add (this file is compiled with -ffp-contract=off), which is the
 //           summation order of the reference's CPU dot (J/common/utils/MatrixOperation.java:1472-1478);
 //           FAST mode uses fused multiply-adds (same order, one rounding per step).
@@ -16,12 +16,13 @@
 #include "common.h"
 
 #define TOK_TILE ROUTER_TOK_TILE
-#define KC 64
 
-template <int EP>
+// EP: experts padded to a power of two; KC: k per staged chunk (larger for few experts, where one chunk in
+// flight per workgroup would otherwise leave the kernel waiting on memory latency)
+template <int EP, int KC, bool EXACT>
 __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
                                                      const float *__restrict__ bg, int T, int d, int E, int K,
-                                                     int renorm, int exact, int32_t *__restrict__ ids,
+                                                     int renorm, int32_t *__restrict__ ids,
                                                      float *__restrict__ wout, int32_t *__restrict__ tile_counts,
                                                      float *__restrict__ logits_out, float *__restrict__ probs_out)
 {
@@ -29,8 +30,9 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
     constexpr int TPP = 256 / EP;            // tokens per pass
     constexpr int GS = EP < 64 ? EP : 64;    // lanes that share one token in phase 2
     constexpr int VPL = EP / GS;             // experts per lane in phase 2
-    __shared__ float xs[TOK_TILE][KC + 1];
-    __shared__ float ws[EP][KC + 1];
+    constexpr int LDW = KC + 4;  // LDS row stride in floats: rows stay 16-byte aligned and bank-staggered
+    __shared__ __attribute__((aligned(16))) float xs[TOK_TILE][LDW];
+    __shared__ __attribute__((aligned(16))) float ws[EP][LDW];
     __shared__ float lg[TOK_TILE][EP];
     __shared__ int hist[EP];
 
@@ -44,47 +46,113 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
 #pragma unroll
     for (int i = 0; i < NT; ++i) acc[i] = 0.0f;
 
+    // staging: every thread carries 8 consecutive k of one token and of WCH gate rows from global memory to LDS;
+    // the next 64-k chunk is fetched into registers while the current one is being summed
+    constexpr int XCH = KC / 64;
+    constexpr int WCH = (EP * (KC / 8) + 255) / 256;
+    const bool vec_ok = (d % 8 == 0) && (((uintptr_t)x | (uintptr_t)Wg) % 16 == 0);
+    const int x_tt = tid >> 3, x_ks = (tid & 7) * 8;
+    // raw staging registers: 8 k of bf16 = one uint4, 8 k of fp32 = two; conversion happens when they are
+    // written to LDS, so the global loads stay in flight during the sums of the current chunk
+    uint4 xr[XCH][2], wr[WCH][2];
+    auto load8 = [&](const void *base, bool valid, size_t row_off, int k, uint4 *out) {
+        out[0] = make_uint4(0, 0, 0, 0);
+        out[1] = make_uint4(0, 0, 0, 0);
+        if (valid && vec_ok && k + 8 <= d) {
+            if (dtype == OMEGA_DTYPE_BF16) {
+                out[0] = *(const uint4 *)((const bf16_t *)base + row_off + k);
+            } else {
+                out[0] = *(const uint4 *)((const float *)base + row_off + k);
+                out[1] = *(const uint4 *)((const float *)base + row_off + k + 4);
+            }
+        } else if (valid) {  // unaligned or ragged rows: element by element, packed into the same form
+            uint32_t u[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                u[q] = 0;
+                if (k + q < d)
+                    u[q] = dtype == OMEGA_DTYPE_BF16 ? (uint32_t)((const bf16_t *)base)[row_off + k + q]
+                                                     : __float_as_uint(((const float *)base)[row_off + k + q]);
+            }
+            if (dtype == OMEGA_DTYPE_BF16) {
+                out[0] = make_uint4(u[0] | (u[1] << 16), u[2] | (u[3] << 16), u[4] | (u[5] << 16), u[6] | (u[7] << 16));
+            } else {
+                out[0] = make_uint4(u[0], u[1], u[2], u[3]);
+                out[1] = make_uint4(u[4], u[5], u[6], u[7]);
+            }
+        }
+    };
+    auto widen = [&](const uint4 *in, float *dst) {  // 8 floats to LDS
+        float4 lo, hi;
+        if (dtype == OMEGA_DTYPE_BF16) {
+            lo = make_float4(__uint_as_float(in[0].x << 16), __uint_as_float(in[0].x & 0xffff0000u),
+                             __uint_as_float(in[0].y << 16), __uint_as_float(in[0].y & 0xffff0000u));
+            hi = make_float4(__uint_as_float(in[0].z << 16), __uint_as_float(in[0].z & 0xffff0000u),
+                             __uint_as_float(in[0].w << 16), __uint_as_float(in[0].w & 0xffff0000u));
+        } else {
+            lo = make_float4(__uint_as_float(in[0].x), __uint_as_float(in[0].y), __uint_as_float(in[0].z), __uint_as_float(in[0].w));
+            hi = make_float4(__uint_as_float(in[1].x), __uint_as_float(in[1].y), __uint_as_float(in[1].z), __uint_as_float(in[1].w));
+        }
+        *(float4 *)dst = lo;
+        *(float4 *)(dst + 4) = hi;
+    };
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < XCH; ++c) load8(x, t0 + x_tt < T, (size_t)(t0 + x_tt) * d, k0 + x_ks + 64 * c, xr[c]);
+#pragma unroll
+        for (int c = 0; c < WCH; ++c) {
+            const int idx = tid + c * 256;
+            const int e = idx / (KC / 8);
+            load8(Wg, idx < EP * (KC / 8) && e < E, (size_t)e * d, k0 + (idx % (KC / 8)) * 8, wr[c]);
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int c = 0; c < XCH; ++c) widen(xr[c], &xs[x_tt][x_ks + 64 * c]);
+#pragma unroll
+        for (int c = 0; c < WCH; ++c) {
+            const int idx = tid + c * 256;
+            if (idx < EP * (KC / 8)) widen(wr[c], &ws[idx / (KC / 8)][(idx % (KC / 8)) * 8]);
+        }
+    };
+
+    fetch(0);
     for (int k0 = 0; k0 < d; k0 += KC) {
         const int kend = min(KC, d - k0);
-        {   // x tile: 32 tokens x 64 k, 8 consecutive k per thread
-            const int tt = tid >> 3, ks = (tid & 7) * 8;
-            const int t = t0 + tt;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int k = k0 + ks + j;
-                float v = 0.0f;
-                if (t < T && k < d)
-                    v = dtype == OMEGA_DTYPE_BF16 ? bf16_to_f32(((const bf16_t *)x)[(size_t)t * d + k])
-                                                  : ((const float *)x)[(size_t)t * d + k];
-                xs[tt][ks + j] = v;
-            }
-        }
-        for (int idx = tid; idx < EP * KC; idx += 256) {
-            const int e = idx / KC, kk = idx % KC;
-            const int k = k0 + kk;
-            float v = 0.0f;
-            if (e < E && k < d)
-                v = dtype == OMEGA_DTYPE_BF16 ? bf16_to_f32(((const bf16_t *)Wg)[(size_t)e * d + k])
-                                              : ((const float *)Wg)[(size_t)e * d + k];
-            ws[e][kk] = v;
-        }
+        stash();
         __syncthreads();
-        if (exact) {
-            for (int k = 0; k < kend; ++k) {
-                const float wv = ws[e1][k];
-#pragma unroll
-                for (int i = 0; i < NT; ++i) {
-                    const float prod = xs[tg + i * TPP][k] * wv;
-                    acc[i] = acc[i] + prod;
-                }
-            }
+        if (k0 + KC < d) fetch(k0 + KC);
+        // the products are added one k at a time in index order: EXACT with a separate multiply and add,
+        // FAST with a fused multiply-add (one rounding per step)
+#define ROUTER_K4(k4)                                                                  \
+    do {                                                                               \
+        const float4 wv = *(const float4 *)&ws[e1][(k4) * 4];                          \
+        _Pragma("unroll") for (int i = 0; i < NT; ++i)                                 \
+        {                                                                              \
+            const float4 xv = *(const float4 *)&xs[tg + i * TPP][(k4) * 4];            \
+            if (EXACT) {                                                               \
+                float prod;                                                            \
+                prod = xv.x * wv.x; acc[i] = acc[i] + prod;                            \
+                prod = xv.y * wv.y; acc[i] = acc[i] + prod;                            \
+                prod = xv.z * wv.z; acc[i] = acc[i] + prod;                            \
+                prod = xv.w * wv.w; acc[i] = acc[i] + prod;                            \
+            } else {                                                                   \
+                acc[i] = fmaf(xv.x, wv.x, acc[i]);                                     \
+                acc[i] = fmaf(xv.y, wv.y, acc[i]);                                     \
+                acc[i] = fmaf(xv.z, wv.z, acc[i]);                                     \
+                acc[i] = fmaf(xv.w, wv.w, acc[i]);                                     \
+            }                                                                          \
+        }                                                                              \
+    } while (0)
+        if (kend == KC) {
+            // whole chunk: no exit test inside, so the LDS reads of later steps are issued ahead of the sums
+#pragma unroll(NT >= 8 ? 4 : 16)
+            for (int k4 = 0; k4 < KC / 4; ++k4) ROUTER_K4(k4);
         } else {
-            for (int k = 0; k < kend; ++k) {
-                const float wv = ws[e1][k];
-#pragma unroll
-                for (int i = 0; i < NT; ++i) acc[i] = fmaf(xs[tg + i * TPP][k], wv, acc[i]);
-            }
+            // last, partial chunk (zero-filled beyond d: a +0 product leaves every sum unchanged)
+            for (int k4 = 0; k4 * 4 < kend; ++k4) ROUTER_K4(k4);
         }
+#undef ROUTER_K4
         __syncthreads();
     }
     {
@@ -177,15 +245,22 @@ hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits
     const int tiles = ceil_div(T, TOK_TILE);
     const int exact = c.router_mode == OMEGA_ROUTER_EXACT;
     const float *bg = c.has_gate_bias ? m->bg : nullptr;
-#define ROUTER_LAUNCH(EPV)                                                                                         \
-    hipLaunchKernelGGL(router_kernel<EPV>, dim3(tiles), dim3(256), 0, s, x, c.dtype, m->Wg, bg, T, c.d, c.E, c.K,   \
-                       c.renorm, exact, m->ids, m->w, m->tile_counts, logits_out, probs_out)
-    if (c.E <= 8) ROUTER_LAUNCH(8);
-    else if (c.E <= 16) ROUTER_LAUNCH(16);
-    else if (c.E <= 32) ROUTER_LAUNCH(32);
-    else if (c.E <= 64) ROUTER_LAUNCH(64);
-    else if (c.E <= 128) ROUTER_LAUNCH(128);
-    else ROUTER_LAUNCH(256);
+#define ROUTER_LAUNCH(EPV, KCV)                                                                                    \
+    do {                                                                                                           \
+        if (exact)                                                                                                 \
+            hipLaunchKernelGGL((router_kernel<EPV, KCV, true>), dim3(tiles), dim3(256), 0, s, x, c.dtype, m->Wg, bg, \
+                               T, c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out, probs_out);   \
+        else                                                                                                       \
+            hipLaunchKernelGGL((router_kernel<EPV, KCV, false>), dim3(tiles), dim3(256), 0, s, x, c.dtype, m->Wg,    \
+                               bg, T, c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out,           \
+                               probs_out);                                                                         \
+    } while (0)
+    if (c.E <= 8) ROUTER_LAUNCH(8, 256);
+    else if (c.E <= 16) ROUTER_LAUNCH(16, 256);
+    else if (c.E <= 32) ROUTER_LAUNCH(32, 128);
+    else if (c.E <= 64) ROUTER_LAUNCH(64, 64);
+    else if (c.E <= 128) ROUTER_LAUNCH(128, 64);
+    else ROUTER_LAUNCH(256, 64);
 #undef ROUTER_LAUNCH
     return hipGetLastError();
 }
