@@ -1,0 +1,246 @@
+// C++ host side of the MoE layer over the C ABI of libomega_hip.so, mirroring the reference's Java Layer
+// contract (the reference is Java; this build has no JDK, so the compiled-language mirror is C++).
+//
+//   omega::Tensor    the fields of J/engine/tensor/Tensor.java:23-47 the path uses: number/channel/height/width,
+//                    host float data, a device address, hostToDevice()/syncHost() (Tensor.java:559-579)
+//   omega::Layer     the abstract methods of J/engine/nn/layer/Layer.java:66-104
+//   omega::MoELayer  constructor in the house style of LlamaMLPLayer(embedDim, nChannel, multiple_of, bias, network)
+//                    (J/engine/nn/layer/llama/LlamaMLPLayer.java:47-63) with the explicit hidden size of DiTSwiGLUFFN;
+//                    forward(Tensor) = setInput -> init -> output (LlamaMLPLayer.java:200-217);
+//                    saveModel/loadModel write raw little-endian float32 in the order gate, (gate bias), then
+//                    w1,w3,w2 per expert (routed, then shared), as LlamaMLPLayer.java:273-283 does for one MLP;
+//                    a failing library call throws std::runtime_error("Error code N:msg"), the checkCUDA style
+//                    (J/engine/gpu/CUDAMemoryManager.java:179-201); back/update throw: the path is forward-only.
+// Host tensors are fp32 like the reference's; a bf16 layer converts on the device at the boundary.
+#pragma once
+#include <cstdint>
+#include <cstdio>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "omega_hip.h"
+
+namespace omega {
+
+inline void check(omega_ctx *ctx, int st)
+{
+    if (st != OMEGA_OK) {
+        const char *msg = omega_hip_last_error(ctx);
+        throw std::runtime_error(msg && *msg ? msg : "Error code " + std::to_string(st));
+    }
+}
+
+// One device + one stream (replaces CUDAManager / CUDAPool for this path).
+class Context {
+public:
+    explicit Context(int device = 0)
+    {
+        int st = omega_hip_ctx_create(device, &ctx_);
+        if (st != OMEGA_OK) throw std::runtime_error(omega_hip_last_error(nullptr));
+    }
+    ~Context() { omega_hip_ctx_destroy(ctx_); }
+    Context(const Context &) = delete;
+    Context &operator=(const Context &) = delete;
+    omega_ctx *get() const { return ctx_; }
+    void sync() { check(ctx_, omega_hip_sync(ctx_)); }
+
+private:
+    omega_ctx *ctx_ = nullptr;
+};
+
+struct Tensor {
+    int number = 0, channel = 0, height = 0, width = 0;
+    std::vector<float> data;   // host copy (fp32)
+    void *gpuData = nullptr;   // device address, fp32 [number*channel*height*width]
+    Context *ctx = nullptr;
+
+    Tensor() = default;
+    Tensor(int n, int c, int h, int w, Context *cx, bool hasGPU = true) : number(n), channel(c), height(h), width(w), ctx(cx)
+    {
+        data.assign((size_t)n * c * h * w, 0.0f);
+        if (hasGPU) check(ctx->get(), omega_hip_malloc(ctx->get(), data.size() * 4, &gpuData));
+    }
+    Tensor(const Tensor &) = delete;
+    Tensor &operator=(const Tensor &) = delete;
+    ~Tensor()
+    {
+        if (gpuData) omega_hip_free(ctx->get(), gpuData);
+    }
+    size_t dataLength() const { return data.size(); }
+    bool isHasGPU() const { return gpuData != nullptr; }
+    void hostToDevice() { check(ctx->get(), omega_hip_memcpy_h2d(ctx->get(), gpuData, data.data(), data.size() * 4)); }
+    void syncHost() { check(ctx->get(), omega_hip_memcpy_d2h(ctx->get(), data.data(), gpuData, data.size() * 4)); }
+};
+
+class Layer {
+public:
+    virtual ~Layer() = default;
+    int number = 0, channel = 0, height = 0, width = 0, oChannel = 0, oHeight = 0, oWidth = 0;
+    Tensor *input = nullptr;
+    virtual void init() = 0;
+    virtual void initBack() = 0;
+    virtual void initParam() = 0;
+    virtual void output() = 0;
+    virtual Tensor *getOutput() = 0;
+    virtual void diff() = 0;
+    virtual void forward() = 0;
+    virtual void back() = 0;
+    virtual void forward(Tensor &input) = 0;
+    virtual void back(Tensor &delta) = 0;
+    virtual void update() = 0;
+    virtual void accGrad(float scale) = 0;
+    virtual const char *getLayerType() const = 0;
+    void setInput(Tensor &in) { input = &in; }
+};
+
+class MoELayer : public Layer {
+public:
+    MoELayer(int embedDim, int hidden, int nExperts, int topK, bool renorm, int nShared, bool bias, Context &ctx,
+             int dtype = OMEGA_DTYPE_F32, int routerMode = OMEGA_ROUTER_EXACT)
+        : ctx_(ctx), embedDim_(embedDim), hidden_(hidden), nExperts_(nExperts), topK_(topK), nShared_(nShared), bias_(bias),
+          dtype_(dtype)
+    {
+        oChannel = 1;
+        oHeight = 1;
+        oWidth = embedDim;
+        omega_moe_config cfg{0, embedDim, nExperts, topK, hidden, nShared, renorm ? 1 : 0, bias ? 1 : 0, dtype, routerMode};
+        check(ctx_.get(), omega_moe_create(ctx_.get(), &cfg, &moe_));
+    }
+    ~MoELayer() override
+    {
+        omega_moe_destroy(moe_);
+        if (xLow_) omega_hip_free(ctx_.get(), xLow_);
+        if (outLow_) omega_hip_free(ctx_.get(), outLow_);
+    }
+
+    // parameters arrive as fp32 host arrays in the reference's [out,in] layout
+    void setGate(const float *Wg, const float *bg = nullptr)
+    {
+        upload(OMEGA_W_GATE, 0, Wg, (size_t)nExperts_ * embedDim_);
+        if (bg) check(ctx_.get(), omega_moe_set_weights(moe_, OMEGA_W_GATE_BIAS, 0, bg, 0));
+    }
+    void setExpert(int g, const float *W1, const float *W3, const float *W2)
+    {
+        const size_t n = (size_t)hidden_ * embedDim_;
+        upload(OMEGA_W_W1, g, W1, n);
+        upload(OMEGA_W_W3, g, W3, n);
+        upload(OMEGA_W_W2, g, W2, n);
+    }
+
+    void init() override
+    {
+        number = input->number;
+        if (!output_ || output_->number != number) {
+            output_.reset(new Tensor(number, oChannel, oHeight, oWidth, &ctx_, true));
+            if (dtype_ == OMEGA_DTYPE_BF16) {
+                if (xLow_) omega_hip_free(ctx_.get(), xLow_);
+                if (outLow_) omega_hip_free(ctx_.get(), outLow_);
+                check(ctx_.get(), omega_hip_malloc(ctx_.get(), (size_t)number * embedDim_ * 2, &xLow_));
+                check(ctx_.get(), omega_hip_malloc(ctx_.get(), (size_t)number * embedDim_ * 2, &outLow_));
+            }
+        }
+    }
+    void initBack() override {}
+    void initParam() override {}
+    void output() override
+    {
+        const size_t n = (size_t)number * embedDim_;
+        if (dtype_ == OMEGA_DTYPE_BF16) {
+            check(ctx_.get(), omega_hip_convert(ctx_.get(), xLow_, OMEGA_DTYPE_BF16, input->gpuData, OMEGA_DTYPE_F32, n));
+            check(ctx_.get(), omega_moe_forward(moe_, xLow_, number, outLow_));
+            check(ctx_.get(), omega_hip_convert(ctx_.get(), output_->gpuData, OMEGA_DTYPE_F32, outLow_, OMEGA_DTYPE_BF16, n));
+        } else {
+            check(ctx_.get(), omega_moe_forward(moe_, input->gpuData, number, output_->gpuData));
+        }
+    }
+    Tensor *getOutput() override { return output_.get(); }
+    void forward() override
+    {
+        init();
+        output();
+    }
+    void forward(Tensor &in) override
+    {
+        if (in.width != embedDim_ || !in.isHasGPU()) throw std::runtime_error("Error code 1:input width does not match embedDim or tensor has no device data");
+        setInput(in);
+        init();
+        output();
+    }
+    void diff() override { unsupported(); }
+    void back() override { unsupported(); }
+    void back(Tensor &) override { unsupported(); }
+    void update() override { unsupported(); }
+    void accGrad(float) override { unsupported(); }
+    const char *getLayerType() const override { return "feed_forward"; }
+
+    void getRouting(std::vector<int32_t> &ids, std::vector<float> &w, std::vector<int32_t> &counts)
+    {
+        ids.resize((size_t)number * topK_);
+        w.resize(ids.size());
+        counts.resize(nExperts_);
+        check(ctx_.get(), omega_moe_get_routing(moe_, number, ids.data(), w.data(), counts.data(), nullptr, nullptr, nullptr));
+    }
+
+    void saveModel(FILE *f) { eachParam([&](int which, int g, size_t n) { std::vector<float> h = download(which, g, n); if (fwrite(h.data(), 4, n, f) != n) throw std::runtime_error("Error code 1:short write"); }); }
+    void loadModel(FILE *f) { eachParam([&](int which, int g, size_t n) { std::vector<float> h(n); if (fread(h.data(), 4, n, f) != n) throw std::runtime_error("Error code 1:checkpoint ends early"); if (which == OMEGA_W_GATE_BIAS) check(ctx_.get(), omega_moe_set_weights(moe_, which, g, h.data(), 0)); else upload(which, g, h.data(), n); }); }
+
+private:
+    [[noreturn]] static void unsupported() { throw std::logic_error("MoELayer is forward-only"); }
+    template <class F> void eachParam(F f)
+    {
+        f(OMEGA_W_GATE, 0, (size_t)nExperts_ * embedDim_);
+        if (bias_) f(OMEGA_W_GATE_BIAS, 0, (size_t)nExperts_);
+        for (int g = 0; g < nExperts_ + nShared_; ++g) {
+            f(OMEGA_W_W1, g, (size_t)hidden_ * embedDim_);
+            f(OMEGA_W_W3, g, (size_t)hidden_ * embedDim_);
+            f(OMEGA_W_W2, g, (size_t)hidden_ * embedDim_);
+        }
+    }
+    // fp32 host array -> layer dtype on the device -> layer storage
+    void upload(int which, int g, const float *h, size_t n)
+    {
+        if (dtype_ == OMEGA_DTYPE_F32) {
+            check(ctx_.get(), omega_moe_set_weights(moe_, which, g, h, 0));
+            return;
+        }
+        void *f32 = nullptr, *low = nullptr;
+        check(ctx_.get(), omega_hip_malloc(ctx_.get(), n * 4, &f32));
+        check(ctx_.get(), omega_hip_malloc(ctx_.get(), n * 2, &low));
+        int st = omega_hip_memcpy_h2d(ctx_.get(), f32, h, n * 4);
+        if (st == OMEGA_OK) st = omega_hip_convert(ctx_.get(), low, OMEGA_DTYPE_BF16, f32, OMEGA_DTYPE_F32, n);
+        if (st == OMEGA_OK) st = omega_moe_set_weights(moe_, which, g, low, 1);
+        omega_hip_free(ctx_.get(), f32);
+        omega_hip_free(ctx_.get(), low);
+        check(ctx_.get(), st);
+    }
+    std::vector<float> download(int which, int g, size_t n)
+    {
+        std::vector<float> h(n);
+        if (dtype_ == OMEGA_DTYPE_F32 || which == OMEGA_W_GATE_BIAS) {
+            check(ctx_.get(), omega_moe_get_weights(moe_, which, g, h.data(), 0));
+            return h;
+        }
+        void *f32 = nullptr, *low = nullptr;
+        check(ctx_.get(), omega_hip_malloc(ctx_.get(), n * 4, &f32));
+        check(ctx_.get(), omega_hip_malloc(ctx_.get(), n * 2, &low));
+        int st = omega_moe_get_weights(moe_, which, g, low, 1);
+        if (st == OMEGA_OK) st = omega_hip_convert(ctx_.get(), f32, OMEGA_DTYPE_F32, low, OMEGA_DTYPE_BF16, n);
+        if (st == OMEGA_OK) st = omega_hip_memcpy_d2h(ctx_.get(), h.data(), f32, n * 4);
+        omega_hip_free(ctx_.get(), f32);
+        omega_hip_free(ctx_.get(), low);
+        check(ctx_.get(), st);
+        return h;
+    }
+
+    Context &ctx_;
+    omega_moe *moe_ = nullptr;
+    int embedDim_, hidden_, nExperts_, topK_, nShared_;
+    bool bias_;
+    int dtype_;
+    std::unique_ptr<Tensor> output_;
+    void *xLow_ = nullptr, *outLow_ = nullptr;
+};
+
+}  // namespace omega

@@ -1,0 +1,65 @@
+// Drives omega::MoELayer the way a transformer block drives its FFN slot
+// (J/engine/nn/layer/llama/LlamaTransformerBlock.java:135: getMlp().forward(norm2.getOutput())).
+// Reads inputs and weights as raw little-endian float32 files, runs forward, writes the output and
+// the routing; used by tests/test_gpu_host_cpp.py, which compares against the CPU oracle.
+//   moe_host_demo <dir> T d E K H Es renorm dtype(0|1)
+#include <cstdlib>
+#include <cstring>
+
+#include "MoELayer.hpp"
+
+static std::vector<float> read_f32(const std::string &path, size_t n)
+{
+    std::vector<float> v(n);
+    FILE *f = fopen(path.c_str(), "rb");
+    if (!f || fread(v.data(), 4, n, f) != n) throw std::runtime_error("cannot read " + path);
+    fclose(f);
+    return v;
+}
+
+int main(int argc, char **argv)
+{
+    if (argc != 10) { fprintf(stderr, "usage: %s dir T d E K H Es renorm dtype\n", argv[0]); return 2; }
+    try {
+        const std::string dir = argv[1];
+        const int T = atoi(argv[2]), d = atoi(argv[3]), E = atoi(argv[4]), K = atoi(argv[5]), H = atoi(argv[6]),
+                  Es = atoi(argv[7]), renorm = atoi(argv[8]), dtype = atoi(argv[9]);
+        omega::Context ctx(0);
+        omega::MoELayer mlp(d, H, E, K, renorm != 0, Es, false, ctx, dtype);
+        FILE *ck = fopen((dir + "/model.bin").c_str(), "rb");
+        if (!ck) throw std::runtime_error("cannot open model.bin");
+        mlp.loadModel(ck);
+        fclose(ck);
+        omega::Tensor x(T, 1, 1, d, &ctx, true);
+        x.data = read_f32(dir + "/x.bin", (size_t)T * d);
+        x.hostToDevice();
+        mlp.forward(x);
+        omega::Tensor *out = mlp.getOutput();
+        out->syncHost();
+        FILE *fo = fopen((dir + "/out.bin").c_str(), "wb");
+        fwrite(out->data.data(), 4, out->data.size(), fo);
+        fclose(fo);
+        std::vector<int32_t> ids, counts;
+        std::vector<float> w;
+        mlp.getRouting(ids, w, counts);
+        FILE *fi = fopen((dir + "/ids.bin").c_str(), "wb");
+        fwrite(ids.data(), 4, ids.size(), fi);
+        fclose(fi);
+        // round trip of the checkpoint format
+        FILE *sv = fopen((dir + "/model_saved.bin").c_str(), "wb");
+        mlp.saveModel(sv);
+        fclose(sv);
+        // error convention: a mismatching input must raise, not crash
+        omega::Tensor bad(T, 1, 1, d + 1, &ctx, true);
+        bool raised = false;
+        try { mlp.forward(bad); } catch (const std::runtime_error &) { raised = true; }
+        if (!raised) throw std::runtime_error("mismatching input was accepted");
+        try { mlp.update(); raised = false; } catch (const std::logic_error &) { raised = true; }
+        if (!raised) throw std::runtime_error("update() did not raise");
+        printf("ok layerType=%s T=%d\n", mlp.getLayerType(), T);
+        return 0;
+    } catch (const std::exception &e) {
+        fprintf(stderr, "moe_host_demo: %s\n", e.what());
+        return 1;
+    }
+}

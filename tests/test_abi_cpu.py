@@ -1,0 +1,68 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares, and fails
+cleanly (status + message, no abort) when there is no device or a handle is NULL.  No compute is launched."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from tests.conftest import load_pkg
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return load_pkg().load_library()
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "omega_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(omega_(?:hip|moe)_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    L = load_pkg("_lib")
+    names = declared_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/omega_hip.h but not exported"
+        assert n in L.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(L.SIGNATURES) <= set(names)
+
+
+def test_version_and_error_paths_without_a_device(lib):
+    assert lib.omega_hip_version() >= 100
+    assert lib.omega_hip_ctx_create(0, None) == 1                       # INVALID_ARG
+    assert b"Error code" in lib.omega_hip_last_error(None)
+    import torch
+    if not torch.cuda.is_available():
+        h = C.c_void_p()
+        st = lib.omega_hip_ctx_create(0, C.byref(h))
+        assert st != 0 and not h.value
+        assert b"Error code" in lib.omega_hip_last_error(None)
+    # NULL handles are rejected, never dereferenced
+    assert lib.omega_hip_sync(None) == 1
+    assert lib.omega_moe_forward(None, None, 4, None) == 1
+    assert lib.omega_moe_get_routing(None, 1, None, None, None, None, None, None) == 1
+    assert lib.omega_moe_destroy(None) == 0 and lib.omega_hip_ctx_destroy(None) == 0
+
+
+def test_host_mirror_keeps_the_layer_contract():
+    P = load_pkg()
+    for name in ("init", "initBack", "output", "getOutput", "forward", "back", "update", "accGrad", "getLayerType",
+                 "saveModel", "loadModel", "setInput"):
+        assert hasattr(P.MoELayer, name)
+    hpp = open(os.path.join(ROOT, "omega-ai_amd", "host", "MoELayer.hpp")).read()
+    for name in ("init()", "initBack()", "initParam()", "output()", "getOutput()", "forward(Tensor", "back(Tensor",
+                 "update()", "accGrad(", "getLayerType()", "saveModel(", "loadModel("):
+        assert name in hpp
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    L = load_pkg("_lib")
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setattr(L, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        L.load_library()

@@ -1,0 +1,50 @@
+"""Golden fixtures (tests/golden/*.npz, written by tests/golden/make_fixtures.py from the pinned oracle).
+
+CPU: the oracle still reproduces every fixture bit for bit (guards the oracle against drift).
+GPU: the HIP path reproduces the routing arrays bit for bit and the output within tolerance."""
+import importlib.util
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle_np as N
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(HERE, "golden", "make_fixtures.py"))
+MF = importlib.util.module_from_spec(spec)
+spec.loader.exec_module(MF)
+
+
+def load(name):
+    return dict(np.load(os.path.join(HERE, "golden", name + ".npz")))
+
+
+@pytest.mark.parametrize("name", sorted(MF.CASES))
+def test_oracle_reproduces_fixture(name):
+    want, got = load(name), MF.expected(MF.CASES[name])
+    assert sorted(want) == sorted(got)
+    for k in want:
+        assert np.array_equal(want[k], got[k]), (name, k)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(MF.CASES))
+def test_hip_path_reproduces_fixture(name):
+    from tests import gpu_util as G
+    case = MF.CASES[name]
+    cfg, want = case["cfg"], load(name)
+    inp = MF.case_inputs(case)
+    layer = G.build_layer(cfg, inp)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    out = layer.forward(x).to_numpy()
+    r = layer.routing()
+    for k in ("ids", "counts", "offsets", "dst", "src_row"):
+        assert np.array_equal(r[k], want[k]), (name, k)
+    assert np.array_equal(r["w"].view(np.uint32), want["w"].view(np.uint32))
+    tol = 1e-2 if cfg.dtype == "bf16" else 1e-5
+    assert N.rel_l2(out[:4], want["out_head"]) <= tol and N.rel_l2(out[-2:], want["out_tail"]) <= tol
+    o64 = out.astype(np.float64)
+    assert abs(np.sqrt((o64 ** 2).sum()) - want["out_l2"]) <= tol * want["out_l2"]
+    assert abs(o64.sum() - want["out_sum"]) <= tol * want["out_abs_sum"]
+    layer.close()

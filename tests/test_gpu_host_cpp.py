@@ -1,0 +1,41 @@
+"""The C++ host mirror of the layer (omega-ai_amd/host/MoELayer.hpp) driven as a transformer block drives its
+FFN slot, checked against the CPU oracle.  The demo binary is built by __graft_entry__.build()."""
+import os
+import subprocess
+import tempfile
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from oracle import oracle_np as N
+from tests.synth import C, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEMO = os.path.join(ROOT, "omega-ai_amd", "host", "moe_host_demo")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_cpp_layer_forward_and_checkpoint(dtype):
+    assert os.path.exists(DEMO), "build omega-ai_amd/host/moe_host_demo first (__graft_entry__.build())"
+    cfg = C.MoEConfig("t", T=200, d=256, E=8, K=2, H=384, Es=1, renorm=True, dtype=dtype)
+    inp = make_inputs(cfg, 17)
+    G = cfg.E + cfg.Es
+    with tempfile.TemporaryDirectory() as td:
+        inp["x"].astype("<f4").tofile(os.path.join(td, "x.bin"))
+        model = np.concatenate([inp["Wg"].ravel()] + [np.concatenate([inp["W1"][g].ravel(), inp["W3"][g].ravel(),
+                                                                     inp["W2"][g].ravel()]) for g in range(G)])
+        model.astype("<f4").tofile(os.path.join(td, "model.bin"))
+        r = subprocess.run([DEMO, td, str(cfg.T), str(cfg.d), str(cfg.E), str(cfg.K), str(cfg.H), str(cfg.Es), "1",
+                            "1" if dtype == "bf16" else "0"], capture_output=True, text=True, timeout=100)
+        assert r.returncode == 0, r.stderr
+        assert "layerType=feed_forward" in r.stdout
+        out = np.fromfile(os.path.join(td, "out.bin"), "<f4").reshape(cfg.T, cfg.d)
+        ids = np.fromfile(os.path.join(td, "ids.bin"), "<i4").reshape(cfg.T, cfg.K)
+        saved = np.fromfile(os.path.join(td, "model_saved.bin"), "<f4")
+    ref = O.moe_forward(inp["x"], inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es, bf16=dtype == "bf16")
+    assert np.array_equal(ids, ref["ids"])
+    assert N.rel_l2(out, ref["out"]) <= (1e-2 if dtype == "bf16" else 1e-5)
+    assert np.array_equal(saved, model.astype(np.float32))      # checkpoint round trip is byte-exact
