@@ -41,6 +41,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample duration")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain 256 MiB device copy (convert_kernel fp32->fp32) three times, so that "
+                         "FETCH_SIZE / WRITE_SIZE of a profiled run can be scaled by a kernel of known traffic")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus above 1 is not supported (no collectives in this path)",
@@ -59,6 +62,14 @@ def main():
     x.fill_normal(a.seed, C.STREAM_X, C.tensor_std(cfg, "x"))
     ctx.sync()
 
+    if a.copy_calibration:
+        n = 64 * 1024 * 1024
+        src, dst = P.DeviceBuffer(ctx, (n,), "f32"), P.DeviceBuffer(ctx, (n,), "f32")
+        for _ in range(3):
+            ctx.check(ctx.lib.omega_hip_convert(ctx.handle, dst.ptr, L.DTYPE_F32, src.ptr, L.DTYPE_F32, n))
+        ctx.sync()
+        src.free()
+        dst.free()
     for _ in range(a.warmup):
         layer.forward(x)
     ctx.sync()

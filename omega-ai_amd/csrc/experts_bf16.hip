@@ -71,14 +71,18 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
     //      group q / 8; this wave issues q = wave and q = wave + 8 of both operands.  Consecutive k steps of
     //      a row group are 8 KiB apart. ----
     const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
-    const uint32_t a_rg1 = (uint32_t)KT * 8192u;  // second row group of the A tile
+    // A blocks that hold no valid row (ragged last tile of an expert) are never used by an MFMA whose result is
+    // kept: their loads are pointed at block 0 of the tile, which another wave loads in the same step anyway,
+    // so they cost no extra L2 traffic while every wave still issues the same number of loads per step
+    const uint32_t a_off0 = (16 * wave < tl.rows ? (uint32_t)wave * 1024u : 0u) + (uint32_t)lane * 16u;
+    const uint32_t a_off1 = 16 * (wave + 8) < tl.rows ? (uint32_t)KT * 8192u + blk_off : (uint32_t)lane * 16u;
 // direct load n (0..3) of one 32-k step: n -> (operand, row group) = (n & 1 ? B : A, n >> 1)
 #define ISSUE_LOAD1(stage, kstep, n)                                                                       \
     do {                                                                                                   \
         const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                                     \
-        const uint32_t kb = (uint32_t)(kstep) * 8192u + blk_off;                                            \
-        if (((n) & 1) == 0) dma16(A, kb + (((n) >> 1) ? a_rg1 : 0u), sb + ((n) >> 1) * 8192);               \
-        else dma16(((n) >> 1) == 0 ? B0 : B1, kb, sb + TILE_BYTES + ((n) >> 1) * 8192);                      \
+        const uint32_t kb = (uint32_t)(kstep) * 8192u;                                                      \
+        if (((n) & 1) == 0) dma16(A, kb + (((n) >> 1) ? a_off1 : a_off0), sb + ((n) >> 1) * 8192);          \
+        else dma16(((n) >> 1) == 0 ? B0 : B1, kb + blk_off, sb + TILE_BYTES + ((n) >> 1) * 8192);            \
     } while (0)
 
     // ---- MFMA operand addressing ----
