@@ -153,10 +153,11 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 
 static void moe_free_workspace(omega_moe *m)
 {
-    void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y};
+    void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y,
+                    m->desc_up, m->desc_down};
     for (void *p : ptrs)
         if (p) hipFree(p);
-    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr;
+    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr;
     m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
     m->T_cap = 0;
 }
@@ -201,6 +202,10 @@ static int moe_reserve(omega_moe *m, int T)
     // padding rows of xg / a are read by the product kernels (their results are discarded): keep them finite
     OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->xg, 0, m->rows_cap * c.d * m->esize, ctx->stream));
     OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->a, 0, m->rows_cap * c.H * m->esize, ctx->stream));
+    if (c.dtype == OMEGA_DTYPE_BF16) {
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_up, ((size_t)m->tiles_cap * (c.H / 128) + OMEGA_TAIL_EXTRA) * sizeof(omega_tile_desc)));
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_down, ((size_t)m->tiles_cap * (c.d / 256) + OMEGA_TAIL_EXTRA) * sizeof(omega_tile_desc)));
+    }
     if (c.dtype == OMEGA_DTYPE_BF16 && c.Es > 0) {
         const size_t xs_rows = (size_t)ceil_div(T, bm) * bm;
         OMEGA_HIP_CHECK(ctx, hipMalloc(&m->xs, xs_rows * c.d * m->esize));
@@ -250,7 +255,7 @@ int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **ou
     alloc0(&m->W2, wsz);
     alloc0((void **)&m->counts, (size_t)c.E * 4);
     alloc0((void **)&m->offsets, (size_t)(c.E + 1) * 4);
-    alloc0((void **)&m->tile_meta, (size_t)(m->G + 2) * 4);
+    alloc0((void **)&m->tile_meta, (size_t)(m->G + 4) * 4);
     if (e == hipSuccess) e = hipEventCreate(&m->ev0);
     if (e == hipSuccess) e = hipEventCreate(&m->ev1);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);

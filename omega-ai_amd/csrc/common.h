@@ -32,6 +32,17 @@ struct __attribute__((aligned(16))) omega_tile {
     int32_t xrow0;  // -1: routed expert; >=0: shared expert, first token of this tile (A operand = x rows)
 };
 
+// One entry per work item of a grouped product, in launch order (expert, column tile, row tile - row tiles
+// fastest): everything a workgroup needs to start, in one 32-byte load.  A work item is an output tile or, for the
+// last tiles of a launch that would leave most compute units idle, a slice of 64 or 128 rows of one (row0 is then
+// not a multiple of the tile height).  The table can hold OMEGA_TAIL_EXTRA entries more than there are tiles.
+#define OMEGA_TAIL_EXTRA 192
+struct __attribute__((aligned(32))) omega_tile_desc {
+    int32_t g, row0, rows, xrow0;  // as omega_tile
+    int32_t n0;                    // first output column of the tile
+    int32_t pad[3];
+};
+
 struct omega_moe {
     omega_ctx *ctx = nullptr;
     omega_moe_config cfg{};
@@ -56,7 +67,10 @@ struct omega_moe {
     int32_t *dstp = nullptr;         // [T*K] physical row of each pair
     int32_t *src_row = nullptr;      // [T*K]
     omega_tile *tiles = nullptr;     // [max_m_tiles]
-    int32_t *tile_meta = nullptr;    // [0] = number of row tiles; [1+g] = first row tile of group g (G+1 entries)
+    int32_t *tile_meta = nullptr;    // [0] = number of row tiles; [1+g] = first row tile of group g (G+1 entries);
+                                     // [G+2], [G+3] = entries of desc_up, desc_down
+    omega_tile_desc *desc_up = nullptr;    // bf16: [tiles_cap * H/128] output tiles of the up product
+    omega_tile_desc *desc_down = nullptr;  // bf16: [tiles_cap * d/256] output tiles of the down product
     void *xg = nullptr;              // [rows_cap,d]  gathered tokens (bf16: packed tile image, see pack.h)
     void *xs = nullptr;              // bf16 with shared experts: packed copy of x, [ceil(T/bm)*bm,d]
     void *a = nullptr;               // [rows_cap,H]  (bf16: packed tile image)

@@ -61,7 +61,10 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
                                                             int32_t *__restrict__ dst, int32_t *__restrict__ dstp,
                                                             int32_t *__restrict__ src_row,
                                                             omega_tile *__restrict__ tiles,
-                                                            int32_t *__restrict__ tile_meta)
+                                                            int32_t *__restrict__ tile_meta,
+                                                            omega_tile_desc *__restrict__ desc_up, int nt_up, int ncols_up,
+                                                            omega_tile_desc *__restrict__ desc_down, int nt_down,
+                                                            int ncols_down)
 {
     __shared__ int off_s[MAXE + 1];        // logical first row of each expert
     __shared__ int mt_s[MAXE + 64 + 1];    // first row tile of each group (routed, then shared)
@@ -133,6 +136,55 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
         if (tid == 0) tile_meta[0] = mt_s[G];
         for (int g = tid; g <= G; g += 256) tile_meta[1 + g] = mt_s[g];
     }
+
+    // ---- work-item tables of the two grouped products (bf16 layers) ----
+    // Tile number first_tile[g]*NT + n*Mg + m = (expert g, column tile n, row tile m): row tiles fastest, so that
+    // tiles that run at the same time share weight tiles.  The compute units take 256 tiles at a time; when the
+    // last r = Nt mod 256 tiles would occupy at most half of them, each of those tiles is cut into S = 2 or 4
+    // slices of bm/S rows (adjacent entries, so that the slices of a tile run side by side on one XCD and share
+    // the weight tile in its L2).  Group g is written by workgroup g (mod grid).
+    if (desc_up != nullptr || desc_down != nullptr) {
+        const int G = E + Es;
+        if (tile == 0 && tid < 2) {
+            const int Nt = mt_s[G] * (tid == 0 ? nt_up : nt_down), r = Nt % 256;
+            const int S = (r == 0 || r > 128) ? 1 : (r > 64 ? 2 : 4);
+            tile_meta[G + 2 + tid] = Nt - r + r * S;
+        }
+        for (int g = tile; g < G; g += gridDim.x) {
+            const int rows = g < E ? off_s[g + 1] - off_s[g] : T;
+            const int Mg = mt_s[g + 1] - mt_s[g];
+            for (int pass = 0; pass < 2; ++pass) {
+                omega_tile_desc *desc = pass == 0 ? desc_up : desc_down;
+                const int NT = pass == 0 ? nt_up : nt_down, ncols = pass == 0 ? ncols_up : ncols_down;
+                if (desc == nullptr) continue;
+                const int Nt = mt_s[G] * NT, r = Nt % 256;
+                const int S = (r == 0 || r > 128) ? 1 : (r > 64 ? 2 : 4);
+                for (int l = tid; l < Mg * NT; l += 256) {
+                    const int mt = l % Mg, n = l / Mg;
+                    const int at = mt_s[g] * NT + l;
+                    const int trows = min(bm, rows - mt * bm);
+                    omega_tile_desc dsc;
+                    dsc.g = g;
+                    dsc.n0 = n * ncols;
+                    dsc.pad[0] = dsc.pad[1] = dsc.pad[2] = 0;
+                    if (at < Nt - r) {
+                        dsc.row0 = (mt_s[g] + mt) * bm;
+                        dsc.rows = trows;
+                        dsc.xrow0 = g < E ? -1 : mt * bm;
+                        desc[at] = dsc;
+                    } else {
+                        const int slice = bm / S;
+                        for (int sl = 0; sl < S; ++sl) {
+                            dsc.row0 = (mt_s[g] + mt) * bm + sl * slice;
+                            dsc.rows = max(0, min(slice, trows - sl * slice));  // 0: nothing to do
+                            dsc.xrow0 = g < E ? -1 : mt * bm + sl * slice;
+                            desc[Nt - r + (at - (Nt - r)) * S + sl] = dsc;
+                        }
+                    }
+                }
+            }
+        }
+    }
 }
 
 // One wave per token; 16-byte chunks; up to 8 chunks in flight per lane.  PACKED: destination rows are in the
@@ -191,7 +243,8 @@ hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t 
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(dispatch_rank_kernel, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_base, m->counts, T, c.K,
-                       c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles, m->tile_meta);
+                       c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles, m->tile_meta, m->desc_up, c.H / 128, 128,
+                       m->desc_down, c.d / 256, 256);
     return hipGetLastError();
 }
 

@@ -6,7 +6,7 @@
 // Both operands are K-contiguous ("NT" product), so a lane's 8 consecutive k values are one 16-byte LDS read.
 // Workgroup = 8 waves (2 row halves x 4 column quarters, two waves per SIMD so that one computes while the
 // other waits on LDS, on the address unit or at the barrier); tile = 256 rows x 256 MFMA columns, each wave
-// 128x64 = 4x2 MFMA blocks with its 128 accumulators in AGPRs.  For the up product the 256 MFMA columns are
+// 4x2 MFMA blocks (the 32-row blocks of the tile alternate between the row halves, so a ragged tile splits evenly) with its 128 accumulators in AGPRs.  For the up product the 256 MFMA columns are
 // 128 columns of W1 and the same 128 columns of W3, arranged so that a wave holds h1 and h3 of the same
 // output element and applies silu(h1)*h3 in registers.
 //
@@ -21,11 +21,9 @@
 // step five ahead.  The direct loads are issued one at a time between MFMAs because the address unit is
 // shared by all waves of the CU and a burst of loads stalls the issuing wave.
 //
-// Scheduling: the dispatch stage leaves a list of row tiles (never straddling two experts; empty experts
-// have none) and the first row tile of every expert; workgroup -> (expert, column tile, row tile) is
-// derived from those on the device, row tiles fastest so that the workgroups resident on one XCD share
-// weight tiles in its L2.  Consecutive workgroup ids go round-robin over the 8 XCDs, so the id is first
-// remapped to give each XCD a contiguous run of tiles.
+// Scheduling: the dispatch stage leaves a table of output tiles (one 32-byte descriptor each; row tiles never
+// straddle two experts, empty experts have none) ordered (expert, column tile, row tile) with row tiles
+// fastest, so that the workgroups resident on one XCD share weight tiles in its L2.
 #include "common.h"
 #include "pack.h"
 
@@ -45,6 +43,16 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 int experts_bf16_tile_m(const omega_moe *, int) { return BM; }
 
 __device__ __forceinline__ int swz(int row) { return pk_swz(row); }
+
+// two floats -> two bf16 (round to nearest even) in one instruction, v_cvt_pk_bf16_f32; lo in bits 0..15
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
+{
+    const f32x2_t v = {lo, hi};
+    const bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+    return *(const uint32_t *)&r;
+}
 
 // 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16*l.
 __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_base)
@@ -74,8 +82,11 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
     // A blocks that hold no valid row (ragged last tile of an expert) are never used by an MFMA whose result is
     // kept: their loads are pointed at block 0 of the tile, which another wave loads in the same step anyway,
     // so they cost no extra L2 traffic while every wave still issues the same number of loads per step
-    const uint32_t a_off0 = (16 * wave < tl.rows ? (uint32_t)wave * 1024u : 0u) + (uint32_t)lane * 16u;
-    const uint32_t a_off1 = 16 * (wave + 8) < tl.rows ? (uint32_t)KT * 8192u + blk_off : (uint32_t)lane * 16u;
+    // (A points at the row group of the whole tile; a slice starts blk0 16-row blocks into it)
+    const int blk0 = (tl.row0 & (BM - 1)) >> 4;
+    const int qa0 = blk0 + (16 * wave < tl.rows ? wave : 0), qa1 = blk0 + (16 * (wave + 8) < tl.rows ? wave + 8 : 0);
+    const uint32_t a_off0 = (uint32_t)(qa0 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa0 & 7) * 1024u + (uint32_t)lane * 16u;
+    const uint32_t a_off1 = (uint32_t)(qa1 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa1 & 7) * 1024u + (uint32_t)lane * 16u;
 // direct load n (0..3) of one 32-k step: n -> (operand, row group) = (n & 1 ? B : A, n >> 1)
 #define ISSUE_LOAD1(stage, kstep, n)                                                                       \
     do {                                                                                                   \
@@ -91,7 +102,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
     int a_sw[NB], b_sw[2];
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-        const int ar = wm * 128 + i * 32 + l32;
+        const int ar = (2 * i + wm) * 32 + l32;
         a_rb[i] = ar * (BK * 2);
         a_sw[i] = swz(ar);
     }
@@ -194,7 +205,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
         const int kba = (n0 >> 5) + wn;
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
-            const int row = wm * 128 + i * 32 + l32;
+            const int row = (2 * i + wm) * 32 + l32;
             if (row < tl.rows) {
                 const int prow = tl.row0 + row;
 #pragma unroll
@@ -206,9 +217,9 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
 #pragma unroll
                         for (int u = 0; u < 2; ++u) {
                             const float h1 = acc[i][0][t * 4 + h * 2 + u], h3 = acc[i][1][t * 4 + h * 2 + u];
-                            v[u] = h1 * __frcp_rn(1.0f + __expf(-h1)) * h3;
+                            v[u] = h1 * __builtin_amdgcn_rcpf(1.0f + __expf(-h1)) * h3;  // v_exp_f32, v_rcp_f32: 1 ulp each
                         }
-                        pk[h] = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+                        pk[h] = pack_bf16x2(v[0], v[1]);
                     }
                     uint2 o = {pk[0], pk[1]};
                     *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, kba, t, KTa) + lhi * 8) = o;
@@ -221,7 +232,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
         for (int i = 0; i < NBLK; ++i) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                const int row = (2 * i + wm) * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
                 if (row >= tl.rows) continue;
                 float *out = (float *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 64 + l32;
 #pragma unroll
@@ -237,41 +248,42 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
 template <bool FUSED>
 __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
                                                                    const bf16_t *__restrict__ Wa, const bf16_t *__restrict__ Wb,
-                                                                   void *__restrict__ Cout, const omega_tile *__restrict__ tiles,
-                                                                   const int32_t *__restrict__ tile_meta, int G, int N, int Kd)
+                                                                   void *__restrict__ Cout, const omega_tile_desc *__restrict__ desc,
+                                                                   const int32_t *__restrict__ tile_meta, int total_slot, int N, int Kd)
 {
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     constexpr int NCOLS = FUSED ? 128 : 256;  // output columns per tile
     const int NT = N / NCOLS;
     // ---- workgroup -> tile ----
-    const int total = tile_meta[0] * NT;
-    const int chunk = (total + NUM_XCD - 1) / NUM_XCD;
+    // Consecutive workgroup ids go round-robin over the 8 XCDs, and an XCD (32 compute units, one workgroup each)
+    // starts its workgroups in id order.  The table is cut into rounds of 256 consecutive entries; within a round
+    // XCD x takes a contiguous eighth - of what is left, in the last round, so that a short tail (or a launch of
+    // fewer than 256 tiles) still spreads over all eight L2s.
+    const int total = tile_meta[total_slot];
     const int pid = blockIdx.x;
-    const int slot = pid / NUM_XCD;
-    const int L = (pid % NUM_XCD) * chunk + slot;
-    if (slot >= chunk || L >= total) return;
-    int lo = 0, hi = G;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (tile_meta[1 + mid] * NT <= L) lo = mid; else hi = mid;
-    }
-    const int mt0 = tile_meta[1 + lo], Mg = tile_meta[2 + lo] - mt0;
-    const int l = L - mt0 * NT;
-    const int nt = l / Mg;
-    const omega_tile tl = tiles[mt0 + (l % Mg)];
-    const int n0 = nt * NCOLS;
+    const int q = pid / NUM_XCD, base = (q >> 5) * 256;
+    const int left = min(256, total - base);
+    if (left <= 0) return;
+    const int per = (left + NUM_XCD - 1) / NUM_XCD;
+    const int L = base + (pid % NUM_XCD) * per + (q & 31);
+    if ((q & 31) >= per || L >= base + left) return;
+    const omega_tile_desc dsc = desc[L];
+    const omega_tile tl = {dsc.g, dsc.row0, dsc.rows, dsc.xrow0};
+    if (tl.rows <= 0) return;  // empty slice of a ragged tile
+    const int n0 = dsc.n0;
 
     // packed operands: a row group (128 rows) occupies KT * 8 KiB
     const size_t rg_bytes = (size_t)(Kd / BK) * 8192;
-    const unsigned char *A = (FUSED && tl.xrow0 >= 0) ? (const unsigned char *)Ax + (size_t)(tl.xrow0 >> 7) * rg_bytes
-                                                      : (const unsigned char *)Axg + (size_t)(tl.row0 >> 7) * rg_bytes;
+    const unsigned char *A = (FUSED && tl.xrow0 >= 0) ? (const unsigned char *)Ax + (size_t)(tl.xrow0 / BM * 2) * rg_bytes
+                                                      : (const unsigned char *)Axg + (size_t)(tl.row0 / BM * 2) * rg_bytes;
     const size_t wrg = (size_t)tl.g * (N >> 7) + (n0 >> 7);  // row group of the weight tile
     const unsigned char *B0 = (const unsigned char *)Wa + wrg * rg_bytes;
     const unsigned char *B1 = FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : B0 + rg_bytes;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nblk = max(0, min(4, (tl.rows - (wave >> 2) * 128 + 31) >> 5));
+    // 32-row blocks alternate between the two row halves of the workgroup: block b belongs to waves with wm = b % 2
+    const int nblk = max(0, min(4, (((tl.rows + 31) >> 5) + 1 - (wave >> 2)) >> 1));
     switch (nblk) {
         case 4: run_tile<FUSED, 4>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
         case 3: run_tile<FUSED, 3>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
@@ -294,19 +306,18 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
 {
     const omega_moe_config &c = m->cfg;
     (void)T;
-    const int G = c.E + c.Es;
     if (which == 0) {
-        int grid = m->max_m_tiles * (c.H / 128);
-        grid = (grid + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
+        int grid = m->max_m_tiles * (c.H / 128) + OMEGA_TAIL_EXTRA;
+        grid = (grid + 255) / 256 * 256;
         hipLaunchKernelGGL(experts_bf16_kernel<true>, dim3(grid), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
-                           (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, m->tiles, m->tile_meta,
-                           G, c.H, c.d);
+                           (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, m->desc_up, m->tile_meta,
+                           c.E + c.Es + 2, c.H, c.d);
     } else {
-        int grid = m->max_m_tiles * (c.d / 256);
-        grid = (grid + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
+        int grid = m->max_m_tiles * (c.d / 256) + OMEGA_TAIL_EXTRA;
+        grid = (grid + 255) / 256 * 256;
         hipLaunchKernelGGL(experts_bf16_kernel<false>, dim3(grid), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
-                           (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y, m->tiles,
-                           m->tile_meta, G, c.d, c.H);
+                           (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y, m->desc_down,
+                           m->tile_meta, c.E + c.Es + 3, c.d, c.H);
     }
     return hipGetLastError();
 }
