@@ -5,6 +5,7 @@
 #include <new>
 
 #include "common.h"
+#include <algorithm>
 
 #define OMEGA_VERSION 100  // 0.1.0
 
@@ -154,10 +155,10 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 static void moe_free_workspace(omega_moe *m)
 {
     void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y,
-                    m->desc_up, m->desc_down};
+                    m->desc_up, m->desc_down, m->wq_up, m->wq_down};
     for (void *p : ptrs)
         if (p) hipFree(p);
-    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr;
+    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr;
     m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
     m->T_cap = 0;
 }
@@ -205,6 +206,14 @@ static int moe_reserve(omega_moe *m, int T)
     if (c.dtype == OMEGA_DTYPE_BF16) {
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_up, ((size_t)m->tiles_cap * (c.H / 128) + OMEGA_TAIL_EXTRA) * sizeof(omega_tile_desc)));
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_down, ((size_t)m->tiles_cap * (c.d / 256) + OMEGA_TAIL_EXTRA) * sizeof(omega_tile_desc)));
+        m->n_wg = std::min(256, ctx->num_cus / 8 * 8);
+        const size_t q_up = ((size_t)m->tiles_cap * (c.H / 128) + OMEGA_TAIL_EXTRA) / m->n_wg + 2;
+        const size_t q_down = ((size_t)m->tiles_cap * (c.d / 256) + OMEGA_TAIL_EXTRA) / m->n_wg + 2;
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->wq_up, q_up * m->n_wg * sizeof(omega_tile_desc)));
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->wq_down, q_down * m->n_wg * sizeof(omega_tile_desc)));
+        // an all-zero queue is an empty one: the product kernels return at once if no dispatch has run yet
+        OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->wq_up, 0, q_up * m->n_wg * sizeof(omega_tile_desc), ctx->stream));
+        OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->wq_down, 0, q_down * m->n_wg * sizeof(omega_tile_desc), ctx->stream));
     }
     if (c.dtype == OMEGA_DTYPE_BF16 && c.Es > 0) {
         const size_t xs_rows = (size_t)ceil_div(T, bm) * bm;
@@ -230,8 +239,8 @@ int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **ou
     if (c.E > 256) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: more than 256 routed experts");
     if (c.Es > 64) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: more than 64 shared experts");
     if (c.K > 64 || (c.E <= 8 && c.K > 8)) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: K above 64");
-    if (c.dtype == OMEGA_DTYPE_BF16 && (c.d % 256 != 0 || c.H % 128 != 0))
-        OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: bf16 layers need d % 256 == 0 and H % 128 == 0");
+    if (c.dtype == OMEGA_DTYPE_BF16 && (c.d % 256 != 0 || c.H % 128 != 0 || c.H < 256))
+        OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: bf16 layers need d % 256 == 0, H % 128 == 0 and H >= 256");
     if ((double)c.T_max * c.K * (double)(c.d > c.H ? c.d : c.H) > 2.0e9)
         OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "moe_create: T_max*K*max(d,H) exceeds 2e9 elements");
 

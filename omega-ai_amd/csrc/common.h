@@ -71,6 +71,10 @@ struct omega_moe {
                                      // [G+2], [G+3] = entries of desc_up, desc_down
     omega_tile_desc *desc_up = nullptr;    // bf16: [tiles_cap * H/128] output tiles of the up product
     omega_tile_desc *desc_down = nullptr;  // bf16: [tiles_cap * d/256] output tiles of the down product
+    // bf16: the same work items as one queue per workgroup of the (persistent) product kernels, entry q of workgroup w
+    // at [q * n_wg + w]; a queue ends with an entry of 0 rows
+    omega_tile_desc *wq_up = nullptr, *wq_down = nullptr;
+    int n_wg = 0;                          // workgroups of a product launch: one per compute unit, a multiple of 8
     void *xg = nullptr;              // [rows_cap,d]  gathered tokens (bf16: packed tile image, see pack.h)
     void *xs = nullptr;              // bf16 with shared experts: packed copy of x, [ceil(T/bm)*bm,d]
     void *a = nullptr;               // [rows_cap,H]  (bf16: packed tile image)

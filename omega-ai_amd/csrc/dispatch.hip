@@ -187,15 +187,148 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     }
 }
 
+// Per-workgroup queues of the persistent product kernels.  A product launch has n_wg workgroups, one per compute
+// unit; workgroup w runs on XCD w % 8.  The table is consumed in rounds of n_wg consecutive entries, XCD x taking a
+// contiguous eighth of each round (of what is left, in the last one), so the tiles in flight on one XCD are
+// neighbours in the table and share operand tiles in its L2.  Within a round the entries of an XCD are dealt to its
+// workgroups cheapest entry to the workgroup with the most work so far (ragged row tiles cost less than full ones),
+// which keeps the queues' total work level without any run-time arbitration.
+// One workgroup of 256 threads per (product, XCD); it runs as one of the first workgroups of the gather launch, which
+// needs nothing from it, so its time is hidden.  Three steps per chunk of SCHED_RC rounds: all threads fetch the
+// costs; wave 0 deals the rounds one after the other (lane j < n_wg/8 stands for workgroup j*8 + x); all threads
+// copy the descriptors to their queue slots.
+#define SCHED_RC 256  // rounds per chunk (LDS: 32 bytes of cost + 64 bytes of placement per round)
+#define SCHED_WGS 16  // 2 products x 8 XCDs
+
+__device__ __forceinline__ int work_item_cost(int rows)
+{
+    if (rows <= 0) return 0;
+    const int nb = (((rows + 31) >> 5) + 1) >> 1;  // 32-row blocks per wave of the busier row half
+    return nb == 1 ? 5 : nb == 2 ? 9 : nb == 3 ? 12 : 16;  // sixteenths of a full tile; the loads and the fixed part do not shrink
+}
+
+struct sched_args {
+    const omega_tile_desc *desc_up, *desc_down;
+    omega_tile_desc *wq_up, *wq_down;
+    const int32_t *tile_meta;
+    int G, n_wg;
+};
+
+__device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
+{
+    __shared__ unsigned char cost_s[SCHED_RC * 32];
+    __shared__ unsigned short place_s[SCHED_RC * 32];  // [round][workgroup j] = 0x8000 | (queue slot - len0) << 5 | source lane
+    __shared__ int len0_s[32];
+    const int pass = which >> 3, x = which & 7, tid = threadIdx.x, lane = tid & 63;
+    const omega_tile_desc *desc = pass == 0 ? a.desc_up : a.desc_down;
+    omega_tile_desc *wq = pass == 0 ? a.wq_up : a.wq_down;
+    const int n_wg = a.n_wg, wpx = n_wg >> 3;
+    const int total = a.tile_meta[a.G + 2 + pass];
+    const int rounds = (total + n_wg - 1) / n_wg;
+    // entry of (round r, place i of this XCD), or -1
+    auto entry = [&](int r, int i) {
+        const int base = r * n_wg, left = min(n_wg, total - base);
+        const int per = (left + 7) >> 3;
+        const int L = base + x * per + i;
+        return (i < per && L < base + left) ? L : -1;
+    };
+    int work = 0, len = 0;  // wave 0, lane j: total cost and length of the queue of workgroup j*8 + x
+    for (int r0 = 0; r0 < rounds; r0 += SCHED_RC) {
+        const int nr = min(SCHED_RC, rounds - r0);
+        for (int i0 = 0; i0 < nr * 32; i0 += 4 * 256) {  // four independent loads in flight per thread
+            int rows[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = i0 + u * 256 + tid;
+                const int L = idx < nr * 32 ? entry(r0 + (idx >> 5), idx & 31) : -1;
+                rows[u] = L >= 0 ? desc[L].rows : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = i0 + u * 256 + tid;
+                if (idx < nr * 32) cost_s[idx] = (unsigned char)work_item_cost(rows[u]);
+            }
+        }
+        if (tid < 32) len0_s[tid] = len;
+        __syncthreads();
+        if (tid < 64) {
+            int c_next = lane < 32 ? cost_s[lane] : 0;
+            for (int r = 0; r < nr; ++r) {
+                const int c = c_next;
+                c_next = (lane < 32 && r + 1 < nr) ? cost_s[(r + 1) * 32 + lane] : 0;
+                // place of the lane's entry by rising cost (costs take five values: count with ballots) and of its
+                // workgroup by falling work; lanes that stand for no workgroup keep their own place
+                int rank_c = 0;
+#pragma unroll
+                for (int v = 0; v <= 16; ++v) {
+                    if (v != 0 && v != 5 && v != 9 && v != 12 && v != 16) continue;
+                    const unsigned long long m = __ballot(c == v && lane < wpx);
+                    if (c > v) rank_c += __popcll(m);
+                    else if (c == v) rank_c += __popcll(m & ((1ull << lane) - 1));
+                }
+                // keys are unique (ties go to the lower lane), so a place is a count of larger keys; lane o's key is
+                // broadcast through a scalar register
+                const int key = lane < wpx ? (work << 6) | (63 - lane) : -1;
+                int rank_w = 0;
+#pragma unroll
+                for (int o = 0; o < 32; ++o) rank_w += __builtin_amdgcn_readlane(key, o) > key ? 1 : 0;
+                if (lane >= wpx) rank_c = rank_w = lane;
+                // lane p receives the entry whose cost has place p, then every workgroup fetches the entry of its place
+                const int sorted = __builtin_amdgcn_ds_permute(rank_c << 2, (c << 8) | lane);
+                const int mine = __builtin_amdgcn_ds_bpermute(rank_w << 2, sorted);
+                const int ce = mine >> 8, src = mine & 31;
+                if (lane < 32) {
+                    unsigned short pl = 0;
+                    if (lane < wpx && ce > 0) {
+                        pl = (unsigned short)(0x8000 | ((len - len0_s[lane]) << 5) | src);
+                        work += ce;
+                        ++len;
+                    }
+                    place_s[r * 32 + lane] = pl;
+                }
+            }
+        }
+        __syncthreads();
+        for (int i0 = 0; i0 < nr * 32; i0 += 2 * 256) {  // two independent copies in flight per thread
+            const int idx0 = i0 + tid, idx1 = i0 + 256 + tid;
+            const unsigned short pl0 = idx0 < nr * 32 ? place_s[idx0] : 0, pl1 = idx1 < nr * 32 ? place_s[idx1] : 0;
+            const uint4 *sp0 = (const uint4 *)(desc + (pl0 ? entry(r0 + (idx0 >> 5), pl0 & 31) : 0));
+            const uint4 *sp1 = (const uint4 *)(desc + (pl1 ? entry(r0 + (idx1 >> 5), pl1 & 31) : 0));
+            const uint4 lo0 = sp0[0], hi0 = sp0[1], lo1 = sp1[0], hi1 = sp1[1];
+            if (pl0) {
+                uint4 *dp = (uint4 *)(wq + (size_t)(len0_s[idx0 & 31] + ((pl0 >> 5) & 0x3ff)) * n_wg + (idx0 & 31) * 8 + x);
+                dp[0] = lo0;
+                dp[1] = hi0;
+            }
+            if (pl1) {
+                uint4 *dp = (uint4 *)(wq + (size_t)(len0_s[idx1 & 31] + ((pl1 >> 5) & 0x3ff)) * n_wg + (idx1 & 31) * 8 + x);
+                dp[0] = lo1;
+                dp[1] = hi1;
+            }
+        }
+        __syncthreads();
+    }
+    if (tid < wpx) {
+        omega_tile_desc z = {};
+        wq[(size_t)len * n_wg + tid * 8 + x] = z;
+    }
+}
+
 // One wave per token; 16-byte chunks; up to 8 chunks in flight per lane.  PACKED: destination rows are in the
 // packed tile image (chunk index = 4*kstep + c) and, when xs != nullptr, the token is also copied to row t of xs.
+// The first n_sched workgroups build the product kernels' queues instead (see schedule_queues).
 template <bool PACKED>
 __global__ __launch_bounds__(256) void dispatch_gather_kernel(const uint4 *__restrict__ x, const int32_t *__restrict__ dstp,
                                                               int T, int K, int chunks_per_row,
-                                                              unsigned char *__restrict__ xg, unsigned char *__restrict__ xs)
+                                                              unsigned char *__restrict__ xg, unsigned char *__restrict__ xs,
+                                                              int n_sched, sched_args sa)
 {
+    if (PACKED && (int)blockIdx.x < n_sched) {
+        schedule_queues(sa, blockIdx.x);
+        return;
+    }
     const int lane = threadIdx.x & 63;
-    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int t = ((int)blockIdx.x - n_sched) * 4 + (threadIdx.x >> 6);
     if (t >= T) return;
     const uint4 *src = x + (size_t)t * chunks_per_row;
     const int KT = chunks_per_row >> 2;
@@ -204,7 +337,7 @@ __global__ __launch_bounds__(256) void dispatch_gather_kernel(const uint4 *__res
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int c = c0 + u * 64 + lane;
-            if (c < chunks_per_row) v[u] = src[c];
+            v[u] = c < chunks_per_row ? src[c] : uint4{0u, 0u, 0u, 0u};  // always assigned: the array stays in registers
         }
         const int nd = K + ((PACKED && xs != nullptr) ? 1 : 0);
         for (int j = 0; j < nd; ++j) {
@@ -253,11 +386,12 @@ hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipS
     const omega_moe_config &c = m->cfg;
     const size_t row_bytes = (size_t)c.d * m->esize;
     if (c.dtype == OMEGA_DTYPE_BF16) {  // d % 256 == 0 is guaranteed at creation: rows are whole 64-byte k steps
-        hipLaunchKernelGGL(dispatch_gather_kernel<true>, dim3(ceil_div(T, 4)), dim3(256), 0, s, (const uint4 *)x, m->dstp,
-                           T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs);
+        sched_args sa = {m->desc_up, m->desc_down, m->wq_up, m->wq_down, m->tile_meta, c.E + c.Es, m->n_wg};
+        hipLaunchKernelGGL(dispatch_gather_kernel<true>, dim3(ceil_div(T, 4) + SCHED_WGS), dim3(256), 0, s, (const uint4 *)x,
+                           m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs, SCHED_WGS, sa);
     } else if (row_bytes % 16 == 0 && ((uintptr_t)x % 16) == 0) {
         hipLaunchKernelGGL(dispatch_gather_kernel<false>, dim3(ceil_div(T, 4)), dim3(256), 0, s, (const uint4 *)x,
-                           m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)nullptr);
+                           m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)nullptr, 0, sched_args{});
     } else {
         hipLaunchKernelGGL(dispatch_gather_bytes_kernel, dim3(T), dim3(256), 0, s, (const unsigned char *)x, m->dstp, T,
                            c.K, row_bytes, (unsigned char *)m->xg);

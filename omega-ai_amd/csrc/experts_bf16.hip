@@ -21,9 +21,13 @@
 // step five ahead.  The direct loads are issued one at a time between MFMAs because the address unit is
 // shared by all waves of the CU and a burst of loads stalls the issuing wave.
 //
-// Scheduling: the dispatch stage leaves a table of output tiles (one 32-byte descriptor each; row tiles never
-// straddle two experts, empty experts have none) ordered (expert, column tile, row tile) with row tiles
-// fastest, so that the workgroups resident on one XCD share weight tiles in its L2.
+// Scheduling: persistent, one workgroup per compute unit.  The dispatch stage leaves every workgroup a queue of
+// work items (32-byte descriptors: an output tile, or a slice of the rows of one for the last tiles of a launch;
+// row tiles never straddle two experts, empty experts have none), dealt so that the workgroups of an XCD work on
+// neighbouring tiles - (expert, column tile, row tile) with row tiles fastest - at the same time and share weight
+// tiles in its L2, and so that all queues hold the same amount of work.  The ring of LDS stages runs on from one
+// item to the next: the last steps of an item already fetch the first steps of the next, so a workgroup pays
+// the load latency once per launch, not once per tile.
 #include "common.h"
 #include "pack.h"
 
@@ -61,67 +65,109 @@ __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t
                  : "memory");
 }
 
-// One output tile.  NBLK = number of 32-row blocks of this wave that hold valid rows (the others are never
+// Everything the loads of one work item need (uniform over the workgroup except the two lane offsets).
+// A: packed row group of the tile's first row; B0/B1: packed row groups of the two 128-row halves of the B tile.
+struct TileCtx {
+    const unsigned char *A, *B0, *B1;
+    uint32_t a_off0, a_off1;  // this lane's byte offsets of its two A blocks within a k step
+    int row0, rows, n0;
+};
+
+__device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char *p)
+{
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const unsigned char *)(((uint64_t)hi << 32) | lo);
+}
+
+template <bool FUSED>
+__device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa,
+                                            const bf16_t *Wb, int N, int Kd, int wave, int lane)
+{
+    TileCtx c;
+    const int KT = Kd / BK;
+    const size_t rg_bytes = (size_t)KT * 8192;  // a packed row group (128 rows) occupies KT * 8 KiB
+    c.row0 = d.row0;
+    c.rows = d.rows;
+    c.n0 = d.n0;
+    c.A = uniform_ptr((FUSED && d.xrow0 >= 0) ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
+                                              : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes);
+    const size_t wrg = (size_t)d.g * (N >> 7) + (d.n0 >> 7);  // row group of the weight tile
+    c.B0 = uniform_ptr((const unsigned char *)Wa + wrg * rg_bytes);
+    c.B1 = uniform_ptr(FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : c.B0 + rg_bytes);
+    // Wave-load q (0..15) of an operand tile is the packed block q % 8 of row group q / 8; this wave issues q = wave
+    // and q = wave + 8 of both operands.  A points at the row group of the whole row tile; a slice starts blk0
+    // 16-row blocks into it.  A blocks that hold no valid row (ragged tile) are never used by an MFMA whose result
+    // is kept: their loads are pointed at the first block, which another wave loads in the same step anyway, so
+    // they cost no extra L2 traffic while every wave still issues the same number of loads per step.
+    const int blk0 = (d.row0 & (BM - 1)) >> 4;
+    const int qa0 = blk0 + (16 * wave < d.rows ? wave : 0), qa1 = blk0 + (16 * (wave + 8) < d.rows ? wave + 8 : 0);
+    c.a_off0 = (uint32_t)(qa0 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa0 & 7) * 1024u + (uint32_t)lane * 16u;
+    c.a_off1 = (uint32_t)(qa1 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa1 & 7) * 1024u + (uint32_t)lane * 16u;
+    return c;
+}
+
+// direct load n (0..3) of k step `kstep` of a work item into ring stage `stage`: n -> (operand, row group) =
+// (n & 1 ? B : A, n >> 1)
+__device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, uint32_t blk_off, int stage, int kstep, int n)
+{
+    const uint32_t sb = lds_wave + stage * STAGE_BYTES;
+    const uint32_t kb = (uint32_t)kstep * 8192u;
+    if ((n & 1) == 0) dma16(c.A, kb + ((n >> 1) ? c.a_off1 : c.a_off0), sb + (n >> 1) * 8192);
+    else dma16((n >> 1) == 0 ? c.B0 : c.B1, kb + blk_off, sb + TILE_BYTES + (n >> 1) * 8192);
+}
+
+// One work item.  NBLK = number of 32-row blocks of this wave that hold valid rows (the others are never
 // computed: a ragged last row tile of an expert costs only the blocks it fills).  NBLK == 0: the wave only
 // takes part in the loads and barriers.
-// A: packed row group of the tile's first row; B0/B1: packed row groups of the two 128-row halves of the B tile.
+// The ring of stages runs on across work items: on entry, stage `cur` holds (or is about to receive) k step 0 of this
+// item, k steps 0..NSTAGE-2 and the first half of step NSTAGE-1 are in flight, and the barrier that makes step 0
+// visible has been passed.  The last NSTAGE steps issue the first loads of the next item (dn, if it has rows)
+// instead of their own, so the matrix cores of the next item start on data that travelled during this item's
+// epilogue.
 template <bool FUSED, int NBLK>
-__device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned char *A, const unsigned char *B0,
-                                         const unsigned char *B1, void *Cout, const omega_tile tl, int n0, int N, int Kd,
-                                         int wave, int lane)
+__device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx, TileCtx &nx, const omega_tile_desc &dn,
+                                         const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa, const bf16_t *Wb, int &cur,
+                                         void *Cout, int N, int Kd, int wave, int lane)
 {
     constexpr int NB = NBLK > 0 ? NBLK : 1;
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
-
-    const int KT = Kd / BK;
-    // ---- direct-load addressing: wave-load q (0..15) of an operand tile is the packed block q % 8 of row
-    //      group q / 8; this wave issues q = wave and q = wave + 8 of both operands.  Consecutive k steps of
-    //      a row group are 8 KiB apart. ----
+    const uint32_t lds_wave = lds0 + wave * 1024;
     const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
-    // A blocks that hold no valid row (ragged last tile of an expert) are never used by an MFMA whose result is
-    // kept: their loads are pointed at block 0 of the tile, which another wave loads in the same step anyway,
-    // so they cost no extra L2 traffic while every wave still issues the same number of loads per step
-    // (A points at the row group of the whole tile; a slice starts blk0 16-row blocks into it)
-    const int blk0 = (tl.row0 & (BM - 1)) >> 4;
-    const int qa0 = blk0 + (16 * wave < tl.rows ? wave : 0), qa1 = blk0 + (16 * (wave + 8) < tl.rows ? wave + 8 : 0);
-    const uint32_t a_off0 = (uint32_t)(qa0 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa0 & 7) * 1024u + (uint32_t)lane * 16u;
-    const uint32_t a_off1 = (uint32_t)(qa1 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa1 & 7) * 1024u + (uint32_t)lane * 16u;
-// direct load n (0..3) of one 32-k step: n -> (operand, row group) = (n & 1 ? B : A, n >> 1)
-#define ISSUE_LOAD1(stage, kstep, n)                                                                       \
-    do {                                                                                                   \
-        const uint32_t sb = lds0 + (stage) * STAGE_BYTES + wave * 1024;                                     \
-        const uint32_t kb = (uint32_t)(kstep) * 8192u;                                                      \
-        if (((n) & 1) == 0) dma16(A, kb + (((n) >> 1) ? a_off1 : a_off0), sb + ((n) >> 1) * 8192);          \
-        else dma16(((n) >> 1) == 0 ? B0 : B1, kb + blk_off, sb + TILE_BYTES + ((n) >> 1) * 8192);            \
+    const int KT = Kd / BK;
+    const bool has_next = dn.rows > 0;
+
+// load n of virtual k step v: steps beyond this item's last belong to the next item
+#define ISSUE_V(stage, v, n)                                                              \
+    do {                                                                                  \
+        if ((v) < KT) issue_load(ctx, lds_wave, blk_off, stage, v, n);                    \
+        else if (has_next) issue_load(nx, lds_wave, blk_off, stage, (v) - KT, n);          \
     } while (0)
 
     // ---- MFMA operand addressing ----
+    // Row (2i + wm)*32 + l32 of A, row j*128 + wn*32 + l32 (up: block 0 = 32 columns of W1, block 1 = the same 32
+    // columns of W3) or wn*64 + j*32 + l32 (down) of B.  The chunk swizzle depends on the row only through l32
+    // (rows differ by multiples of 32), so one swizzled k offset serves every block and the blocks are constant
+    // byte offsets.
     const int l32 = lane & 31, lhi = lane >> 5;
-    uint32_t a_rb[NB], b_rb[2];
-    int a_sw[NB], b_sw[2];
+    const int sw = swz(l32);
+    uint32_t pa[2], pb[2];
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
-        const int ar = (2 * i + wm) * 32 + l32;
-        a_rb[i] = ar * (BK * 2);
-        a_sw[i] = swz(ar);
+    for (int ks = 0; ks < 2; ++ks) {
+        const uint32_t ko = (uint32_t)((ks * 2 + lhi) ^ sw) << 4;
+        pa[ks] = (uint32_t)(wm * 32 + l32) * (BK * 2) + ko;
+        pb[ks] = TILE_BYTES + (uint32_t)((FUSED ? wn * 32 : wn * 64) + l32) * (BK * 2) + ko;
     }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        // up product: block 0 = 32 columns of W1, block 1 = the same 32 columns of W3
-        const int br = FUSED ? (j * 128 + wn * 32 + l32) : (wn * 64 + j * 32 + l32);
-        b_rb[j] = TILE_BYTES + br * (BK * 2);
-        b_sw[j] = swz(br);
-    }
+    constexpr uint32_t A_BLK = 64 * BK * 2, B_BLK = (FUSED ? 128 : 32) * BK * 2;
 #define READ_FRAGS(AF, BF, stage, ks)                                                                       \
     do {                                                                                                    \
         if (NBLK > 0) {                                                                                     \
             const unsigned char *sp = smem + (stage) * STAGE_BYTES;                                          \
-            const int c = (ks) * 2 + lhi;                                                                    \
             _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                   \
-                AF[i] = *(const bf16x8_t *)(sp + a_rb[i] + ((c ^ a_sw[i]) << 4));                            \
+                AF[i] = *(const bf16x8_t *)(sp + pa[ks] + i * A_BLK);                                        \
             _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                    \
-                BF[j] = *(const bf16x8_t *)(sp + b_rb[j] + ((c ^ b_sw[j]) << 4));                            \
+                BF[j] = *(const bf16x8_t *)(sp + pb[ks] + j * B_BLK);                                        \
         }                                                                                                   \
     } while (0)
 // the two MFMAs of row block i.  The up product feeds the weights as the first operand, so that a lane ends
@@ -145,56 +191,49 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     bf16x8_t af0[NB], bf0[2], af1[NB], bf1[2];
+    READ_FRAGS(af0, bf0, cur, 0);
 
-    // prologue: stages 0..NSTAGE-1 <- steps 0..NSTAGE-1; wait for step 0 only when all were issued
-    for (int st = 0; st < NSTAGE && st < KT; ++st) {
-#pragma unroll
-        for (int n = 0; n < LOADS_PER_STEP; ++n) ISSUE_LOAD1(st, st, n);
-    }
-    if (KT >= NSTAGE) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // LOADS_PER_STEP * (NSTAGE - 1)
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    READ_FRAGS(af0, bf0, 0, 0);
-
-// One 32-k step on stage `cur`.  The 4 direct loads a wave owes per step are issued one per pair of row blocks:
-//   LOADS_B: first half of the loads of step kt+NSTAGE, into the stage this step releases at its barrier
-//   LOADS_A: second half of the loads of step kt-1+NSTAGE, into the stage the previous step released
-// STEADY: all loads up to step kt-1+NSTAGE exist, so exactly NSTAGE-2 younger steps (12 loads) may stay in
-// flight at the barrier; otherwise (tail) everything must have landed.
-#define K_STEP(kt, LOADS_A, LOADS_B, STEADY, NEXT)                                                  \
-    do {                                                                                            \
-        const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;                                            \
-        const int prv = cur == 0 ? NSTAGE - 1 : cur - 1;                                            \
-        __builtin_amdgcn_sched_barrier(0);                                                          \
-        READ_FRAGS(af1, bf1, cur, 1);                                                               \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
-        {                                                                                           \
-            if (LOADS_A && (i & 1) == 0) ISSUE_LOAD1(prv, (kt) - 1 + NSTAGE, 2 + (i >> 1));     \
-            MFMA2(af0, bf0, i);                                                                     \
-        }                                                                                           \
-        __builtin_amdgcn_sched_barrier(0);                                                          \
-        /* every wave has taken its last fragments of this stage; the next stage must have landed */ \
-        if (STEADY) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");                    \
-        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                            \
-        __syncthreads();                                                                            \
-        if (NEXT) READ_FRAGS(af0, bf0, nxt, 0);                                                     \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
-        {                                                                                           \
-            if (LOADS_B && (i & 1) == 0) ISSUE_LOAD1(cur, (kt) + NSTAGE, i >> 1);               \
-            MFMA2(af1, bf1, i);                                                                     \
-        }                                                                                           \
-        cur = nxt;                                                                                  \
+    // One 32-k step on stage `cur`.  The 4 direct loads a wave owes per step are issued one per pair of row blocks:
+    //   before the barrier: second half of the loads of step kt-1+NSTAGE, into the stage the previous step released
+    //   after the barrier:  first half of the loads of step kt+NSTAGE, into the stage this step releases
+    // While loads keep coming (this item's or the next one's) exactly NSTAGE-2 younger steps (12 loads) may stay in
+    // flight at the barrier; when they have stopped (last steps of a queue) everything must have landed.
+    // GEN = false: every load belongs to this item (kt < KT - NSTAGE), no run-time decisions in the loop.
+#define K_STEP(GEN)                                                                                          \
+    do {                                                                                                    \
+        const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;                                                    \
+        const int prv = cur == 0 ? NSTAGE - 1 : cur - 1;                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                                  \
+        READ_FRAGS(af1, bf1, cur, 1);                                                                       \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
+        {                                                                                                   \
+            if ((i & 1) == 0) {                                                                             \
+                if (GEN) ISSUE_V(prv, kt - 1 + NSTAGE, 2 + (i >> 1));                                       \
+                else issue_load(ctx, lds_wave, blk_off, prv, kt - 1 + NSTAGE, 2 + (i >> 1));                \
+            }                                                                                               \
+            MFMA2(af0, bf0, i);                                                                             \
+        }                                                                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                                  \
+        /* every wave has taken its last fragments of this stage; the next stage must have landed */        \
+        if (!GEN || has_next || kt + NSTAGE <= KT) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory"); \
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                                    \
+        __syncthreads();                                                                                    \
+        if (!GEN || kt + 1 < KT) READ_FRAGS(af0, bf0, nxt, 0);                                              \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
+        {                                                                                                   \
+            if ((i & 1) == 0) {                                                                             \
+                if (GEN) ISSUE_V(cur, kt + NSTAGE, i >> 1);                                                 \
+                else issue_load(ctx, lds_wave, blk_off, cur, kt + NSTAGE, i >> 1);                          \
+            }                                                                                               \
+            MFMA2(af1, bf1, i);                                                                             \
+        }                                                                                                   \
+        cur = nxt;                                                                                          \
     } while (0)
 
-    int kt = 0, cur = 0;
-    if (KT > NSTAGE) {
-        K_STEP(kt, false, true, true, true);
-        for (kt = 1; kt + NSTAGE < KT; ++kt) K_STEP(kt, true, true, true, true);
-        K_STEP(kt, true, false, true, true);  // kt == KT - NSTAGE: last step of the steady wait count
-        ++kt;
-    }
-    for (; kt + 1 < KT; ++kt) K_STEP(kt, false, false, false, true);
-    K_STEP(kt, false, false, false, false);
+    int kt = 0;
+    for (; kt < KT - NSTAGE; ++kt) K_STEP(false);
+    nx = make_ctx<FUSED>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
+    for (; kt < KT; ++kt) K_STEP(true);
 #undef K_STEP
 
     // ---- epilogue ----
@@ -202,12 +241,12 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
         // lane: row l32 of block i; register r -> column 8*(r/4) + 4*lhi + r%4 of the wave's 32 columns, which are
         // one k step of the packed `a` (K dimension = N): chunk r/4, bytes lhi*8 .. lhi*8+7
         const int KTa = N / BK;
-        const int kba = (n0 >> 5) + wn;
+        const int kba = (ctx.n0 >> 5) + wn;
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
             const int row = (2 * i + wm) * 32 + l32;
-            if (row < tl.rows) {
-                const int prow = tl.row0 + row;
+            if (row < ctx.rows) {
+                const int prow = ctx.row0 + row;
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     uint32_t pk[2];
@@ -233,63 +272,62 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const unsigned cha
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = (2 * i + wm) * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                if (row >= tl.rows) continue;
-                float *out = (float *)Cout + (size_t)(tl.row0 + row) * N + n0 + wn * 64 + l32;
+                if (row >= ctx.rows) continue;
+                float *out = (float *)Cout + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l32;
 #pragma unroll
                 for (int j = 0; j < 2; ++j) out[j * 32] = acc[i][j][r];
             }
         }
     }
-#undef ISSUE_LOAD1
+#undef ISSUE_V
 #undef READ_FRAGS
 #undef MFMA2
 }
 
+// Persistent: one workgroup per compute unit walks its queue of work items (built by the dispatch stage).
 template <bool FUSED>
 __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
                                                                    const bf16_t *__restrict__ Wa, const bf16_t *__restrict__ Wb,
-                                                                   void *__restrict__ Cout, const omega_tile_desc *__restrict__ desc,
-                                                                   const int32_t *__restrict__ tile_meta, int total_slot, int N, int Kd)
+                                                                   void *__restrict__ Cout, const omega_tile_desc *__restrict__ wq,
+                                                                   int N, int Kd)
 {
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    constexpr int NCOLS = FUSED ? 128 : 256;  // output columns per tile
-    const int NT = N / NCOLS;
-    // ---- workgroup -> tile ----
-    // Consecutive workgroup ids go round-robin over the 8 XCDs, and an XCD (32 compute units, one workgroup each)
-    // starts its workgroups in id order.  The table is cut into rounds of 256 consecutive entries; within a round
-    // XCD x takes a contiguous eighth - of what is left, in the last round, so that a short tail (or a launch of
-    // fewer than 256 tiles) still spreads over all eight L2s.
-    const int total = tile_meta[total_slot];
-    const int pid = blockIdx.x;
-    const int q = pid / NUM_XCD, base = (q >> 5) * 256;
-    const int left = min(256, total - base);
-    if (left <= 0) return;
-    const int per = (left + NUM_XCD - 1) / NUM_XCD;
-    const int L = base + (pid % NUM_XCD) * per + (q & 31);
-    if ((q & 31) >= per || L >= base + left) return;
-    const omega_tile_desc dsc = desc[L];
-    const omega_tile tl = {dsc.g, dsc.row0, dsc.rows, dsc.xrow0};
-    if (tl.rows <= 0) return;  // empty slice of a ragged tile
-    const int n0 = dsc.n0;
-
-    // packed operands: a row group (128 rows) occupies KT * 8 KiB
-    const size_t rg_bytes = (size_t)(Kd / BK) * 8192;
-    const unsigned char *A = (FUSED && tl.xrow0 >= 0) ? (const unsigned char *)Ax + (size_t)(tl.xrow0 / BM * 2) * rg_bytes
-                                                      : (const unsigned char *)Axg + (size_t)(tl.row0 / BM * 2) * rg_bytes;
-    const size_t wrg = (size_t)tl.g * (N >> 7) + (n0 >> 7);  // row group of the weight tile
-    const unsigned char *B0 = (const unsigned char *)Wa + wrg * rg_bytes;
-    const unsigned char *B1 = FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : B0 + rg_bytes;
-
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // 32-row blocks alternate between the two row halves of the workgroup: block b belongs to waves with wm = b % 2
-    const int nblk = max(0, min(4, (((tl.rows + 31) >> 5) + 1 - (wave >> 2)) >> 1));
-    switch (nblk) {
-        case 4: run_tile<FUSED, 4>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
-        case 3: run_tile<FUSED, 3>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
-        case 2: run_tile<FUSED, 2>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
-        case 1: run_tile<FUSED, 1>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
-        default: run_tile<FUSED, 0>(smem, A, B0, B1, Cout, tl, n0, N, Kd, wave, lane); break;
+    const int n_wg = gridDim.x, wg = blockIdx.x;
+
+    omega_tile_desc d = wq[wg];
+    if (d.rows <= 0) return;
+    TileCtx cur_ctx = make_ctx<FUSED>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
+    {
+        // first item: k steps 0..NSTAGE-2 and the first half of step NSTAGE-1 into stages 0..NSTAGE-1
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+        const uint32_t lds_wave = lds0 + wave * 1024;
+        const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
+        for (int st = 0; st < NSTAGE - 1; ++st) {
+#pragma unroll
+            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load(cur_ctx, lds_wave, blk_off, st, st, n);
+        }
+        issue_load(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 0);
+        issue_load(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 1);
+        asm volatile("s_waitcnt vmcnt(14)" ::: "memory");  // all but steps 1.. : LOADS_PER_STEP * (NSTAGE - 2) + 2
+        __syncthreads();
+    }
+    int stage = 0;
+    TileCtx nx = cur_ctx;
+    for (int q = 1;; ++q) {
+        const omega_tile_desc dn = wq[(size_t)q * n_wg + wg];
+        // 32-row blocks alternate between the two row halves of the workgroup: block b belongs to waves with wm = b % 2
+        const int nblk = max(0, min(4, (((cur_ctx.rows + 31) >> 5) + 1 - (wave >> 2)) >> 1));
+        switch (nblk) {
+            case 4: run_tile<FUSED, 4>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
+            case 3: run_tile<FUSED, 3>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
+            case 2: run_tile<FUSED, 2>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
+            case 1: run_tile<FUSED, 1>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
+            default: run_tile<FUSED, 0>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
+        }
+        if (dn.rows <= 0) break;
+        cur_ctx = nx;
     }
 }
 
@@ -306,18 +344,16 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
 {
     const omega_moe_config &c = m->cfg;
     (void)T;
+    (void)x;
+    // the ring must be shorter than an item: K >= (NSTAGE + 1) * BK (guaranteed at creation: d, H >= 256)
+    if ((which == 0 ? c.d : c.H) < (NSTAGE + 1) * BK) return hipErrorInvalidValue;
     if (which == 0) {
-        int grid = m->max_m_tiles * (c.H / 128) + OMEGA_TAIL_EXTRA;
-        grid = (grid + 255) / 256 * 256;
-        hipLaunchKernelGGL(experts_bf16_kernel<true>, dim3(grid), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
-                           (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, m->desc_up, m->tile_meta,
-                           c.E + c.Es + 2, c.H, c.d);
+        hipLaunchKernelGGL(experts_bf16_kernel<true>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
+                           (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, m->wq_up, c.H, c.d);
     } else {
-        int grid = m->max_m_tiles * (c.d / 256) + OMEGA_TAIL_EXTRA;
-        grid = (grid + 255) / 256 * 256;
-        hipLaunchKernelGGL(experts_bf16_kernel<false>, dim3(grid), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
-                           (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y, m->desc_down,
-                           m->tile_meta, c.E + c.Es + 3, c.d, c.H);
+        hipLaunchKernelGGL(experts_bf16_kernel<false>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
+                           (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y, m->wq_down,
+                           c.d, c.H);
     }
     return hipGetLastError();
 }
