@@ -139,7 +139,10 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
 
     // ---- work-item tables of the two grouped products (bf16 layers) ----
     // Tile number first_tile[g]*NT + n*Mg + m = (expert g, column tile n, row tile m): row tiles fastest, so that
-    // tiles that run at the same time share weight tiles.  The compute units take 256 tiles at a time; when the
+    // tiles that run at the same time share weight tiles.  The rows of a group are dealt evenly (in blocks of 32) to
+    // its row tiles, instead of full tiles and a ragged last one: the same number of tiles and of MFMA blocks, but
+    // tiles of one cost, so that the workgroups of an XCD, which share operand tiles through its L2, stay in step.
+    // The compute units take 256 tiles at a time; when the
     // last r = Nt mod 256 tiles would occupy at most half of them, each of those tiles is cut into S = 2 or 4
     // slices of bm/S rows (adjacent entries, so that the slices of a tile run side by side on one XCD and share
     // the weight tile in its L2).  Group g is written by workgroup g (mod grid).
@@ -159,25 +162,27 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
                 if (desc == nullptr) continue;
                 const int Nt = mt_s[G] * NT, r = Nt % 256;
                 const int S = (r == 0 || r > 128) ? 1 : (r > 64 ? 2 : 4);
+                const int nblk = (rows + 31) >> 5;  // 32-row blocks of the group, dealt evenly to its Mg row tiles
                 for (int l = tid; l < Mg * NT; l += 256) {
                     const int mt = l % Mg, n = l / Mg;
                     const int at = mt_s[g] * NT + l;
-                    const int trows = min(bm, rows - mt * bm);
+                    const int tfirst = 32 * ((mt * nblk) / Mg);
+                    const int trows = min(32 * (((mt + 1) * nblk) / Mg), rows) - tfirst;
                     omega_tile_desc dsc;
                     dsc.g = g;
                     dsc.n0 = n * ncols;
                     dsc.pad[0] = dsc.pad[1] = dsc.pad[2] = 0;
                     if (at < Nt - r) {
-                        dsc.row0 = (mt_s[g] + mt) * bm;
+                        dsc.row0 = mt_s[g] * bm + tfirst;
                         dsc.rows = trows;
-                        dsc.xrow0 = g < E ? -1 : mt * bm;
+                        dsc.xrow0 = g < E ? -1 : tfirst;
                         desc[at] = dsc;
                     } else {
                         const int slice = bm / S;
                         for (int sl = 0; sl < S; ++sl) {
-                            dsc.row0 = (mt_s[g] + mt) * bm + sl * slice;
+                            dsc.row0 = mt_s[g] * bm + tfirst + sl * slice;
                             dsc.rows = max(0, min(slice, trows - sl * slice));  // 0: nothing to do
-                            dsc.xrow0 = g < E ? -1 : mt * bm + sl * slice;
+                            dsc.xrow0 = g < E ? -1 : tfirst + sl * slice;
                             desc[Nt - r + (at - (Nt - r)) * S + sl] = dsc;
                         }
                     }
@@ -203,8 +208,8 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
 __device__ __forceinline__ int work_item_cost(int rows)
 {
     if (rows <= 0) return 0;
-    const int nb = (((rows + 31) >> 5) + 1) >> 1;  // 32-row blocks per wave of the busier row half
-    return nb == 1 ? 5 : nb == 2 ? 9 : nb == 3 ? 12 : 16;  // sixteenths of a full tile; the loads and the fixed part do not shrink
+    const int nb = (rows + 31) >> 5;  // 32-row MFMA blocks of the item (the two waves of a SIMD share them)
+    return 2 + (14 * nb) / 8;         // sixteenths of a full tile; the loads and the fixed part do not shrink
 }
 
 struct sched_args {
@@ -256,23 +261,19 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
             for (int r = 0; r < nr; ++r) {
                 const int c = c_next;
                 c_next = (lane < 32 && r + 1 < nr) ? cost_s[(r + 1) * 32 + lane] : 0;
-                // place of the lane's entry by rising cost (costs take five values: count with ballots) and of its
-                // workgroup by falling work; lanes that stand for no workgroup keep their own place
-                int rank_c = 0;
-#pragma unroll
-                for (int v = 0; v <= 16; ++v) {
-                    if (v != 0 && v != 5 && v != 9 && v != 12 && v != 16) continue;
-                    const unsigned long long m = __ballot(c == v && lane < wpx);
-                    if (c > v) rank_c += __popcll(m);
-                    else if (c == v) rank_c += __popcll(m & ((1ull << lane) - 1));
-                }
+                // place of the lane's entry by rising cost and of its workgroup by falling work; lanes that stand for
+                // no workgroup keep their own place
                 // keys are unique (ties go to the lower lane), so a place is a count of larger keys; lane o's key is
                 // broadcast through a scalar register
                 const int key = lane < wpx ? (work << 6) | (63 - lane) : -1;
                 int rank_w = 0;
 #pragma unroll
                 for (int o = 0; o < 32; ++o) rank_w += __builtin_amdgcn_readlane(key, o) > key ? 1 : 0;
-                if (lane >= wpx) rank_c = rank_w = lane;
+                const int ckey = lane < wpx ? (c << 6) | lane : 0x7fffffff;
+                int rank_c = 0;
+#pragma unroll
+                for (int o = 0; o < 32; ++o) rank_c += __builtin_amdgcn_readlane(ckey, o) < ckey ? 1 : 0;
+                if (lane >= wpx) { rank_c = lane; rank_w = lane; }
                 // lane p receives the entry whose cost has place p, then every workgroup fetches the entry of its place
                 const int sorted = __builtin_amdgcn_ds_permute(rank_c << 2, (c << 8) | lane);
                 const int mine = __builtin_amdgcn_ds_bpermute(rank_w << 2, sorted);
