@@ -17,64 +17,53 @@
 
 #define TOK_TILE ROUTER_TOK_TILE
 
+// Phase 1 for the tokens t0.. of one workgroup: acc[i] = logit of (token tg + i*TPP, expert e1), bias not yet added.
 // EP: experts padded to a power of two; KC: k per staged chunk (larger for few experts, where one chunk in
-// flight per workgroup would otherwise leave the kernel waiting on memory latency)
-template <int EP, int KC, bool EXACT>
-__global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
-                                                     const float *__restrict__ bg, int T, int d, int E, int K,
-                                                     int renorm, int32_t *__restrict__ ids,
-                                                     float *__restrict__ wout, int32_t *__restrict__ tile_counts,
-                                                     float *__restrict__ logits_out, float *__restrict__ probs_out)
+// flight per workgroup would otherwise leave the kernel waiting on memory latency).
+// XBF: x and Wg are stored as bf16 (else fp32).  FAST_IO: rows are 16-byte aligned and d is a multiple of KC, so
+// every load is a whole 16-byte vector; rows beyond T or E are redirected to the last valid row (their sums are
+// never used), which keeps the loads free of branches - and with that really asynchronous: a load issued inside
+// a divergent branch makes the compiler wait for all earlier ones first.
+template <int EP, int KC, bool EXACT, bool XBF, bool FAST_IO>
+__device__ __forceinline__ void router_sums(const void *__restrict__ x, const void *__restrict__ Wg, int T, int d, int E,
+                                            int t0, float (*xs)[KC + 4], float (*ws)[KC + 4],
+                                            float (&acc)[TOK_TILE * EP / 256])
 {
-    constexpr int NT = TOK_TILE * EP / 256;  // tokens per thread in phase 1
+    constexpr int NT = TOK_TILE * EP / 256;  // tokens per thread
     constexpr int TPP = 256 / EP;            // tokens per pass
-    constexpr int GS = EP < 64 ? EP : 64;    // lanes that share one token in phase 2
-    constexpr int VPL = EP / GS;             // experts per lane in phase 2
-    constexpr int LDW = KC + 4;  // LDS row stride in floats: rows stay 16-byte aligned and bank-staggered
-    __shared__ __attribute__((aligned(16))) float xs[TOK_TILE][LDW];
-    __shared__ __attribute__((aligned(16))) float ws[EP][LDW];
-    __shared__ float lg[TOK_TILE][EP];
-    __shared__ int hist[EP];
-
     const int tid = threadIdx.x;
-    const int tile = blockIdx.x;
-    const int t0 = tile * TOK_TILE;
     const int e1 = tid % EP, tg = tid / EP;
-    if (tid < EP) hist[tid] = 0;
-
-    float acc[NT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) acc[i] = 0.0f;
-
     // staging: every thread carries 8 consecutive k of one token and of WCH gate rows from global memory to LDS;
-    // the next 64-k chunk is fetched into registers while the current one is being summed
+    // the next chunk is fetched into registers while the current one is being summed
     constexpr int XCH = KC / 64;
-    constexpr int WCH = (EP * (KC / 8) + 255) / 256;
-    const bool vec_ok = (d % 8 == 0) && (((uintptr_t)x | (uintptr_t)Wg) % 16 == 0);
+    constexpr int WCH = EP * (KC / 8) / 256;
+    static_assert(EP * (KC / 8) % 256 == 0, "every thread stages the same number of gate vectors");
     const int x_tt = tid >> 3, x_ks = (tid & 7) * 8;
     // raw staging registers: 8 k of bf16 = one uint4, 8 k of fp32 = two; conversion happens when they are
     // written to LDS, so the global loads stay in flight during the sums of the current chunk
     uint4 xr[XCH][2], wr[WCH][2];
-    auto load8 = [&](const void *base, bool valid, size_t row_off, int k, uint4 *out) {
+    auto load8 = [&](const void *base, int row, int rows, int k, uint4 *out) {
         out[0] = make_uint4(0, 0, 0, 0);
         out[1] = make_uint4(0, 0, 0, 0);
-        if (valid && vec_ok && k + 8 <= d) {
-            if (dtype == OMEGA_DTYPE_BF16) {
-                out[0] = *(const uint4 *)((const bf16_t *)base + row_off + k);
+        if (FAST_IO) {
+            const size_t off = (size_t)min(row, rows - 1) * d + k;
+            if (XBF) {
+                out[0] = *(const uint4 *)((const bf16_t *)base + off);
             } else {
-                out[0] = *(const uint4 *)((const float *)base + row_off + k);
-                out[1] = *(const uint4 *)((const float *)base + row_off + k + 4);
+                out[0] = *(const uint4 *)((const float *)base + off);
+                out[1] = *(const uint4 *)((const float *)base + off + 4);
             }
-        } else if (valid) {  // unaligned or ragged rows: element by element, packed into the same form
+        } else if (row < rows) {  // unaligned or ragged rows: element by element, packed into the same form
+            const size_t row_off = (size_t)row * d;
             uint32_t u[8];
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
                 u[q] = 0;
                 if (k + q < d)
-                    u[q] = dtype == OMEGA_DTYPE_BF16 ? (uint32_t)((const bf16_t *)base)[row_off + k + q]
-                                                     : __float_as_uint(((const float *)base)[row_off + k + q]);
+                    u[q] = XBF ? (uint32_t)((const bf16_t *)base)[row_off + k + q]
+                               : __float_as_uint(((const float *)base)[row_off + k + q]);
             }
-            if (dtype == OMEGA_DTYPE_BF16) {
+            if (XBF) {
                 out[0] = make_uint4(u[0] | (u[1] << 16), u[2] | (u[3] << 16), u[4] | (u[5] << 16), u[6] | (u[7] << 16));
             } else {
                 out[0] = make_uint4(u[0], u[1], u[2], u[3]);
@@ -84,7 +73,7 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
     };
     auto widen = [&](const uint4 *in, float *dst) {  // 8 floats to LDS
         float4 lo, hi;
-        if (dtype == OMEGA_DTYPE_BF16) {
+        if (XBF) {
             lo = make_float4(__uint_as_float(in[0].x << 16), __uint_as_float(in[0].x & 0xffff0000u),
                              __uint_as_float(in[0].y << 16), __uint_as_float(in[0].y & 0xffff0000u));
             hi = make_float4(__uint_as_float(in[0].z << 16), __uint_as_float(in[0].z & 0xffff0000u),
@@ -98,12 +87,11 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
     };
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int c = 0; c < XCH; ++c) load8(x, t0 + x_tt < T, (size_t)(t0 + x_tt) * d, k0 + x_ks + 64 * c, xr[c]);
+        for (int c = 0; c < XCH; ++c) load8(x, t0 + x_tt, T, k0 + x_ks + 64 * c, xr[c]);
 #pragma unroll
         for (int c = 0; c < WCH; ++c) {
             const int idx = tid + c * 256;
-            const int e = idx / (KC / 8);
-            load8(Wg, idx < EP * (KC / 8) && e < E, (size_t)e * d, k0 + (idx % (KC / 8)) * 8, wr[c]);
+            load8(Wg, idx / (KC / 8), E, k0 + (idx % (KC / 8)) * 8, wr[c]);
         }
     };
     auto stash = [&]() {
@@ -112,7 +100,7 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
 #pragma unroll
         for (int c = 0; c < WCH; ++c) {
             const int idx = tid + c * 256;
-            if (idx < EP * (KC / 8)) widen(wr[c], &ws[idx / (KC / 8)][(idx % (KC / 8)) * 8]);
+            widen(wr[c], &ws[idx / (KC / 8)][(idx % (KC / 8)) * 8]);
         }
     };
 
@@ -144,7 +132,7 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
             }                                                                          \
         }                                                                              \
     } while (0)
-        if (kend == KC) {
+        if (FAST_IO || kend == KC) {
             // whole chunk: no exit test inside, so the LDS reads of later steps are issued ahead of the sums
 #pragma unroll(NT >= 8 ? 4 : 16)
             for (int k4 = 0; k4 < KC / 4; ++k4) ROUTER_K4(k4);
@@ -154,6 +142,43 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
         }
 #undef ROUTER_K4
         __syncthreads();
+    }
+}
+
+template <int EP, int KC, bool EXACT>
+__global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
+                                                     const float *__restrict__ bg, int T, int d, int E, int K,
+                                                     int renorm, int32_t *__restrict__ ids,
+                                                     float *__restrict__ wout, int32_t *__restrict__ tile_counts,
+                                                     float *__restrict__ logits_out, float *__restrict__ probs_out)
+{
+    constexpr int NT = TOK_TILE * EP / 256;  // tokens per thread in phase 1
+    constexpr int TPP = 256 / EP;            // tokens per pass
+    constexpr int GS = EP < 64 ? EP : 64;    // lanes that share one token in phase 2
+    constexpr int VPL = EP / GS;             // experts per lane in phase 2
+    constexpr int LDW = KC + 4;  // LDS row stride in floats: rows stay 16-byte aligned and bank-staggered
+    __shared__ __attribute__((aligned(16))) float xs[TOK_TILE][LDW];
+    __shared__ __attribute__((aligned(16))) float ws[EP][LDW];
+    __shared__ float lg[TOK_TILE][EP];
+    __shared__ int hist[EP];
+
+    const int tid = threadIdx.x;
+    const int tile = blockIdx.x;
+    const int t0 = tile * TOK_TILE;
+    const int e1 = tid % EP, tg = tid / EP;
+    if (tid < EP) hist[tid] = 0;
+
+    float acc[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) acc[i] = 0.0f;
+
+    const bool fast_io = (d % KC == 0) && (((uintptr_t)x | (uintptr_t)Wg) % 16 == 0);
+    if (dtype == OMEGA_DTYPE_BF16) {
+        if (fast_io) router_sums<EP, KC, EXACT, true, true>(x, Wg, T, d, E, t0, xs, ws, acc);
+        else router_sums<EP, KC, EXACT, true, false>(x, Wg, T, d, E, t0, xs, ws, acc);
+    } else {
+        if (fast_io) router_sums<EP, KC, EXACT, false, true>(x, Wg, T, d, E, t0, xs, ws, acc);
+        else router_sums<EP, KC, EXACT, false, false>(x, Wg, T, d, E, t0, xs, ws, acc);
     }
     {
         const float b = (bg != nullptr && e1 < E) ? bg[e1] : 0.0f;
