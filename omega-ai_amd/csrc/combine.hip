@@ -9,7 +9,9 @@
 
 #define MAXK 64
 
-template <int VEC, bool BF16>
+// KU: slots whose rows are fetched together before any of them is used (all loads of a group are in flight at
+// once; slots beyond K re-read the last row and are ignored).
+template <int VEC, bool BF16, int KU>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ dst,
                                                       const float *__restrict__ w, int T, int K, int d, int Es,
                                                       const int32_t *__restrict__ tile_meta, int E, int bm,
@@ -29,18 +31,29 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         float acc[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
-        for (int j = 0; j < K; ++j) {
-            const int row = __shfl(myrow, j, 64);
-            const float wj = __shfl(myw, j, 64);
-            const float4 *src = (const float4 *)(y + (size_t)row * d + c0);
+        for (int j0 = 0; j0 < K; j0 += KU) {
+            float4 buf[KU][VEC / 4];
 #pragma unroll
-            for (int q = 0; q < VEC / 4; ++q) {
-                const float4 v4 = src[q];
-                float term;
-                term = wj * v4.x; acc[q * 4 + 0] = acc[q * 4 + 0] + term;
-                term = wj * v4.y; acc[q * 4 + 1] = acc[q * 4 + 1] + term;
-                term = wj * v4.z; acc[q * 4 + 2] = acc[q * 4 + 2] + term;
-                term = wj * v4.w; acc[q * 4 + 3] = acc[q * 4 + 3] + term;
+            for (int u = 0; u < KU; ++u) {
+                const int row = __shfl(myrow, min(j0 + u, K - 1), 64);
+                const float4 *src = (const float4 *)(y + (size_t)row * d + c0);
+#pragma unroll
+                for (int q = 0; q < VEC / 4; ++q) buf[u][q] = src[q];
+            }
+#pragma unroll
+            for (int u = 0; u < KU; ++u) {
+                if (j0 + u < K) {
+                    const float wj = __shfl(myw, j0 + u, 64);
+#pragma unroll
+                    for (int q = 0; q < VEC / 4; ++q) {
+                        const float4 v4 = buf[u][q];
+                        float term;
+                        term = wj * v4.x; acc[q * 4 + 0] = acc[q * 4 + 0] + term;
+                        term = wj * v4.y; acc[q * 4 + 1] = acc[q * 4 + 1] + term;
+                        term = wj * v4.z; acc[q * 4 + 2] = acc[q * 4 + 2] + term;
+                        term = wj * v4.w; acc[q * 4 + 3] = acc[q * 4 + 3] + term;
+                    }
+                }
             }
         }
         for (int s = 0; s < Es; ++s) {
@@ -94,12 +107,19 @@ hipError_t launch_combine(const omega_moe *m, int T, void *out, hipStream_t s)
     const bool bf = c.dtype == OMEGA_DTYPE_BF16;
     const int vec = bf ? 8 : 4;
     if (c.d % vec == 0 && ((uintptr_t)out % 16) == 0 && c.K <= MAXK) {
-        if (bf)
-            hipLaunchKernelGGL((combine_kernel<8, true>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dstp, m->w, T,
-                               c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, out);
-        else
-            hipLaunchKernelGGL((combine_kernel<4, false>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dstp, m->w, T,
-                               c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, out);
+#define COMBINE_LAUNCH(KUV)                                                                                          \
+    do {                                                                                                            \
+        if (bf)                                                                                                     \
+            hipLaunchKernelGGL((combine_kernel<8, true, KUV>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dstp, m->w, \
+                               T, c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, out);                                   \
+        else                                                                                                        \
+            hipLaunchKernelGGL((combine_kernel<4, false, KUV>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dstp, \
+                               m->w, T, c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, out);                             \
+    } while (0)
+        if (c.K <= 2) COMBINE_LAUNCH(2);
+        else if (c.K <= 4) COMBINE_LAUNCH(4);
+        else COMBINE_LAUNCH(8);
+#undef COMBINE_LAUNCH
     } else {
         if (bf)
             hipLaunchKernelGGL(combine_scalar_kernel<true>, dim3(T), dim3(256), 0, s, m->y, m->dstp, m->w, T, c.K, c.d,
