@@ -26,8 +26,8 @@ PEAK_F32_TFLOPS = 157.3
 PEAK_HBM_GBPS = 8000.0
 
 # HBM traffic per launch of the dominant kernel from the committed rocprofv3 --pmc runs
-# (profiles/experts_up_c2_mixtral_pmc.txt): FETCH_SIZE + WRITE_SIZE in bytes, scaled by the copy-kernel factor.
-TRAFFIC_BYTES = {}
+# (profiles/experts_bf16_c2_mixtral_pmc.txt): FETCH_SIZE + WRITE_SIZE in bytes, scaled by the copy-kernel factor.
+TRAFFIC_BYTES = {"c2_mixtral": 5.51e9}
 
 
 def main():
