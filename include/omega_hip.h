@@ -41,7 +41,9 @@ typedef enum {
     OMEGA_W_GATE_BIAS = 1, /* [E] always fp32  */
     OMEGA_W_W1 = 2,        /* [H,d] per expert */
     OMEGA_W_W3 = 3,        /* [H,d] per expert */
-    OMEGA_W_W2 = 4         /* [d,H] per expert */
+    OMEGA_W_W2 = 4,        /* [d,H] per expert */
+    OMEGA_W_NORM = 5       /* [d] always fp32: weight (gamma) of the RMSNorm in front of the layer, block form only
+                              (RMSLayer.gamma, J/engine/nn/layer/normalization/RMSLayer.java) */
 } omega_weight_kind;
 
 /* Constructor arguments of the layer, in the house style of
@@ -112,6 +114,20 @@ int omega_moe_get_weights(omega_moe *moe, int which, int expert, void *dst, int 
  * LlamaMLPLayer.forward(Tensor) (J/engine/nn/layer/llama/LlamaMLPLayer.java:200-217). */
 int omega_moe_forward(omega_moe *moe, const void *x_dev, int T, void *out_dev);
 
+/* Block form: out = x + layer(rmsnorm(x)), the second half of the transformer block,
+ *   getNorm2().forward(tmp1); getMlp().forward(getNorm2().getOutput()); Tensor_OP().add(getMlp().getOutput(), tmp1, tmp2)
+ * (J/engine/nn/layer/llama/LlamaTransformerBlock.java:134-136), in one call and without the two [T,d] round trips
+ * through memory of the normalised rows and of the layer output: the row statistics are taken by a small kernel,
+ * the router and the gather normalise the rows of x as they read them, the combine adds x back.
+ * rmsnorm = rmsnorm_forward_kernel2 (J/engine/nn/layer/normalization/gpu/RMSKernel.cu:185-223, the kernel
+ * RMSLayer.output launches, RMSLayer.java:230): rms = sqrtf(mean(x^2) + 1e-6f), h = (x / rms) * gamma, with the
+ * sum of squares taken lane by lane as that kernel takes it; bf16 layers round h to bf16 and round x + layer(h) once.
+ * The norm weight must have been set (omega_moe_set_weights(moe, OMEGA_W_NORM, 0, gamma, is_device)). */
+int omega_moe_forward_block(omega_moe *moe, const void *x_dev, int T, void *out_dev);
+/* rms[t] of the last omega_moe_forward_block, T floats to host (blocking).  For tests; the normalised rows
+ * themselves are visible as the gathered rows, omega_moe_get_workspace(moe, 0, ...). */
+int omega_moe_get_norm(omega_moe *moe, int T, float *rms_host);
+
 /* The four stages of forward, callable one at a time (per-stage timing and tests); they use the
  * same kernels and workspace as omega_moe_forward and must be called in this order for one T:
  *   router   x -> ids, weights, per-tile expert histogram      (gate: FullyLayer.output, FullyLayer.java:218-243;
@@ -147,7 +163,7 @@ int omega_moe_get_workspace(omega_moe *moe, int which, int T, void *host_dst);
 /* Average duration in milliseconds of the launches of one stage, measured with events on the
  * context's stream: runs `iters` back-to-back repetitions of the stage (0 router, 1 dispatch,
  * 2 experts_up, 3 experts_down, 4 combine, 5 whole forward, 6 dispatch index kernels only, 7 dispatch
- * row gather only) after `warmup` untimed ones.
+ * row gather only, 8 whole forward_block, 9 row statistics of the pre-norm only) after `warmup` untimed ones.
  * x_dev/out_dev as for forward; the stages before `stage` must have been run for this T. */
 int omega_moe_time_stage(omega_moe *moe, int stage, const void *x_dev, int T, void *out_dev, int warmup, int iters,
                          float *ms_avg);

@@ -11,8 +11,9 @@ LIB_PATH = os.path.join(_HERE, "libomega_hip.so")
 OK, ERR_INVALID_ARG, ERR_OOM, ERR_HIP, ERR_UNSUPPORTED = range(5)
 DTYPE_F32, DTYPE_BF16 = 0, 1
 ROUTER_EXACT, ROUTER_FAST = 0, 1
-W_GATE, W_GATE_BIAS, W_W1, W_W3, W_W2 = range(5)
-STAGE_ROUTER, STAGE_DISPATCH, STAGE_UP, STAGE_DOWN, STAGE_COMBINE, STAGE_FORWARD, STAGE_INDEX, STAGE_GATHER = range(8)
+W_GATE, W_GATE_BIAS, W_W1, W_W3, W_W2, W_NORM = range(6)
+(STAGE_ROUTER, STAGE_DISPATCH, STAGE_UP, STAGE_DOWN, STAGE_COMBINE, STAGE_FORWARD, STAGE_INDEX, STAGE_GATHER,
+ STAGE_FORWARD_BLOCK, STAGE_RMS) = range(10)
 
 
 class MoEConfigStruct(C.Structure):
@@ -40,6 +41,8 @@ SIGNATURES = {
     "omega_moe_set_weights": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
     "omega_moe_get_weights": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
     "omega_moe_forward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+    "omega_moe_forward_block": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+    "omega_moe_get_norm": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "omega_moe_router": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "omega_moe_dispatch": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "omega_moe_experts": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),

@@ -13,6 +13,7 @@ import numpy as np
 STREAM_X = 0
 STREAM_WG = 1
 STREAM_BG_PERM = 2
+STREAM_NORM = 3       # gamma of the RMSNorm in front of the layer (block form): 1 + 0.1 * N(0,1)
 STREAM_EXPERT0 = 16
 
 

@@ -155,10 +155,10 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 static void moe_free_workspace(omega_moe *m)
 {
     void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y,
-                    m->desc_up, m->desc_down, m->wq_up, m->wq_down};
+                    m->desc_up, m->desc_down, m->wq_up, m->wq_down, m->rms};
     for (void *p : ptrs)
         if (p) hipFree(p);
-    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr;
+    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr; m->rms = nullptr;
     m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
     m->T_cap = 0;
 }
@@ -191,6 +191,7 @@ static int moe_reserve(omega_moe *m, int T)
     m->rows_cap = (size_t)m->tiles_cap * bm;
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->ids, P * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->w, P * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->rms, (size_t)T * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_counts, (size_t)n_tok_tiles * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_base, (size_t)n_tok_tiles * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->dst, P * 4));
@@ -215,7 +216,7 @@ static int moe_reserve(omega_moe *m, int T)
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->wq_up, 0, q_up * m->n_wg * sizeof(omega_tile_desc), ctx->stream));
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->wq_down, 0, q_down * m->n_wg * sizeof(omega_tile_desc), ctx->stream));
     }
-    if (c.dtype == OMEGA_DTYPE_BF16 && c.Es > 0) {
+    if (c.Es > 0) {  // rows the shared experts read: packed copy of x (bf16), normalised copy of x (fp32 block form)
         const size_t xs_rows = (size_t)ceil_div(T, bm) * bm;
         OMEGA_HIP_CHECK(ctx, hipMalloc(&m->xs, xs_rows * c.d * m->esize));
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->xs, 0, xs_rows * c.d * m->esize, ctx->stream));
@@ -259,6 +260,7 @@ int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **ou
     };
     alloc0(&m->Wg, (size_t)c.E * c.d * m->esize);
     alloc0((void **)&m->bg, (size_t)c.E * 4);
+    alloc0((void **)&m->gamma, (size_t)c.d * 4);
     alloc0(&m->W1, wsz);
     alloc0(&m->W3, wsz);
     alloc0(&m->W2, wsz);
@@ -272,7 +274,7 @@ int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **ou
         omega_set_error(ctx, e == hipErrorOutOfMemory ? OMEGA_ERR_OOM : OMEGA_ERR_HIP, "moe_create: allocation", e,
                         __FILE__, __LINE__);
         // release whatever was allocated
-        void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta};
+        void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta, m->gamma};
         for (void *p : ptrs)
             if (p) hipFree(p);
         if (m->ev0) hipEventDestroy(m->ev0);
@@ -284,7 +286,7 @@ int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **ou
         int st = moe_reserve(m, c.T_max);
         if (st != OMEGA_OK) {
             moe_free_workspace(m);
-            void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta};
+            void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta, m->gamma};
             for (void *p : ptrs)
                 if (p) hipFree(p);
             hipEventDestroy(m->ev0);
@@ -304,7 +306,7 @@ int omega_moe_destroy(omega_moe *m)
     CTX_ENTER(ctx);
     hipStreamSynchronize(ctx->stream);
     moe_free_workspace(m);
-    void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta};
+    void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta, m->gamma};
     for (void *p : ptrs)
         if (p) hipFree(p);
     hipEventDestroy(m->ev0);
@@ -321,6 +323,7 @@ static int weight_slot(omega_moe *m, int which, int expert, void **ptr, size_t *
     switch (which) {
         case OMEGA_W_GATE: *ptr = m->Wg; *bytes = (size_t)c.E * c.d * m->esize; return OMEGA_OK;
         case OMEGA_W_GATE_BIAS: *ptr = m->bg; *bytes = (size_t)c.E * 4; return OMEGA_OK;
+        case OMEGA_W_NORM: *ptr = m->gamma; *bytes = (size_t)c.d * 4; return OMEGA_OK;
         case OMEGA_W_W1: case OMEGA_W_W3: case OMEGA_W_W2: {
             if (expert < 0 || expert >= m->G) return OMEGA_ERR_INVALID_ARG;
             unsigned char *base = (unsigned char *)(which == OMEGA_W_W1 ? m->W1 : which == OMEGA_W_W3 ? m->W3 : m->W2);
@@ -350,6 +353,7 @@ int omega_moe_set_weights(omega_moe *m, int which, int expert, const void *src, 
     if (!weight_is_packed(m, which)) {
         OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(p, src, bytes, is_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream));
         OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+        if (which == OMEGA_W_NORM) m->gamma_set = true;
         return OMEGA_OK;
     }
     const int R = which == OMEGA_W_W2 ? m->cfg.d : m->cfg.H, Kd = which == OMEGA_W_W2 ? m->cfg.H : m->cfg.d;
@@ -401,21 +405,25 @@ static int check_T(omega_moe *m, const void *x, int T, bool need_x)
     return OMEGA_OK;
 }
 
-static int stage_router(omega_moe *m, const void *x, int T)
+// block != 0: block form, out = x + layer(rmsnorm(x)); the row statistics are taken first and the normalisation
+// is applied by the router and the gather to the rows they read
+static int stage_router(omega_moe *m, const void *x, int T, int block)
 {
-    OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, nullptr, m->ctx->stream));
+    if (block) OMEGA_HIP_CHECK(m->ctx, launch_rms_stats(m, x, T, m->ctx->stream));
+    OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, nullptr, block, m->ctx->stream));
     return OMEGA_OK;
 }
-static int stage_dispatch(omega_moe *m, const void *x, int T)
+static int stage_dispatch(omega_moe *m, const void *x, int T, int block)
 {
     const int bm = moe_tile_m(m, T);
     m->bm = bm;
     m->max_m_tiles = moe_max_m_tiles(m, T, bm);
     if (m->max_m_tiles > m->tiles_cap) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: workspace too small for this T");
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));
-    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));
+    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, block, m->ctx->stream));
     return OMEGA_OK;
 }
+// x: the rows the shared experts read in fp32 layers (bf16 layers read the packed copy the gather left in xs)
 static int stage_experts(omega_moe *m, const void *x, int T, int which)
 {
     if (m->bm != moe_tile_m(m, T)) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "experts: dispatch has not run for this T");
@@ -423,9 +431,9 @@ static int stage_experts(omega_moe *m, const void *x, int T, int which)
     else OMEGA_HIP_CHECK(m->ctx, launch_experts_f32(m, x, T, which, m->ctx->stream));
     return OMEGA_OK;
 }
-static int stage_combine(omega_moe *m, int T, void *out)
+static int stage_combine(omega_moe *m, int T, void *out, const void *resid)
 {
-    OMEGA_HIP_CHECK(m->ctx, launch_combine(m, T, out, m->ctx->stream));
+    OMEGA_HIP_CHECK(m->ctx, launch_combine(m, T, out, resid, m->ctx->stream));
     return OMEGA_OK;
 }
 
@@ -440,13 +448,17 @@ static int stage_combine(omega_moe *m, int T, void *out)
         if (_st != OMEGA_OK) return _st;  \
     } while (0)
 
-int omega_moe_forward(omega_moe *m, const void *x, int T, void *out)
+static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block)
 {
-    MOE_ENTER(m);
+    omega_ctx *ctx = m->ctx;
     RUN(check_T(m, x, T, true));
     if (T == 0) return OMEGA_OK;
     if (!out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "forward: out is NULL");
+    if (block && !m->gamma_set) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "forward_block: the norm weight (OMEGA_W_NORM) has not been set");
     RUN(moe_reserve(m, T));
+    // rows the shared experts of an fp32 layer read: x itself, or its normalised copy
+    const void *xsh = (block && m->cfg.dtype == OMEGA_DTYPE_F32 && m->cfg.Es > 0) ? m->xs : x;
+    const void *resid = block ? x : nullptr;
     if (m->profiling) {
         // six events bracket the five stages; durations are read back by omega_moe_get_profile
         if (m->prof_used + 6 > m->prof_events.size()) {
@@ -458,24 +470,45 @@ int omega_moe_forward(omega_moe *m, const void *x, int T, void *out)
         }
         hipEvent_t *ev = &m->prof_events[m->prof_used];
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[0], ctx->stream));
-        RUN(stage_router(m, x, T));
+        RUN(stage_router(m, x, T, block));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[1], ctx->stream));
-        RUN(stage_dispatch(m, x, T));
+        RUN(stage_dispatch(m, x, T, block));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[2], ctx->stream));
-        RUN(stage_experts(m, x, T, 0));
+        RUN(stage_experts(m, xsh, T, 0));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[3], ctx->stream));
-        RUN(stage_experts(m, x, T, 1));
+        RUN(stage_experts(m, xsh, T, 1));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[4], ctx->stream));
-        RUN(stage_combine(m, T, out));
+        RUN(stage_combine(m, T, out, resid));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[5], ctx->stream));
         m->prof_used += 6;
         return OMEGA_OK;
     }
-    RUN(stage_router(m, x, T));
-    RUN(stage_dispatch(m, x, T));
-    RUN(stage_experts(m, x, T, 0));
-    RUN(stage_experts(m, x, T, 1));
-    RUN(stage_combine(m, T, out));
+    RUN(stage_router(m, x, T, block));
+    RUN(stage_dispatch(m, x, T, block));
+    RUN(stage_experts(m, xsh, T, 0));
+    RUN(stage_experts(m, xsh, T, 1));
+    RUN(stage_combine(m, T, out, resid));
+    return OMEGA_OK;
+}
+
+int omega_moe_forward(omega_moe *m, const void *x, int T, void *out)
+{
+    MOE_ENTER(m);
+    return forward_impl(m, x, T, out, 0);
+}
+
+int omega_moe_forward_block(omega_moe *m, const void *x, int T, void *out)
+{
+    MOE_ENTER(m);
+    return forward_impl(m, x, T, out, 1);
+}
+
+int omega_moe_get_norm(omega_moe *m, int T, float *rms_host)
+{
+    MOE_ENTER(m);
+    if (!rms_host || T < 0 || T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_norm: bad argument or no forward_block has run for this T");
+    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(rms_host, m->rms, (size_t)T * 4, hipMemcpyDeviceToHost, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
     return OMEGA_OK;
 }
 
@@ -511,7 +544,7 @@ int omega_moe_router(omega_moe *m, const void *x, int T)
     RUN(check_T(m, x, T, true));
     if (T == 0) return OMEGA_OK;
     RUN(moe_reserve(m, T));
-    return stage_router(m, x, T);
+    return stage_router(m, x, T, 0);
 }
 
 int omega_moe_dispatch(omega_moe *m, const void *x, int T)
@@ -520,7 +553,7 @@ int omega_moe_dispatch(omega_moe *m, const void *x, int T)
     RUN(check_T(m, x, T, true));
     if (T == 0) return OMEGA_OK;
     if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "dispatch: router has not run for this T");
-    return stage_dispatch(m, x, T);
+    return stage_dispatch(m, x, T, 0);
 }
 
 int omega_moe_experts_up(omega_moe *m, const void *x, int T)
@@ -554,7 +587,7 @@ int omega_moe_combine(omega_moe *m, int T, void *out)
     if (T == 0) return OMEGA_OK;
     if (!out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "combine: out is NULL");
     if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "combine: router has not run for this T");
-    return stage_combine(m, T, out);
+    return stage_combine(m, T, out, nullptr);
 }
 
 int omega_moe_get_routing(omega_moe *m, int T, int32_t *ids, float *w, int32_t *counts, int32_t *offsets, int32_t *dst,
@@ -584,7 +617,7 @@ int omega_moe_get_router_probs(omega_moe *m, const void *x, int T, float *logits
     float *dl = nullptr, *dp = nullptr;
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&dl, n * 4));
     hipError_t e = hipMalloc((void **)&dp, n * 4);
-    if (e == hipSuccess) e = launch_router(m, x, T, dl, dp, ctx->stream);
+    if (e == hipSuccess) e = launch_router(m, x, T, dl, dp, 0, ctx->stream);
     if (e == hipSuccess && logits) e = hipMemcpyAsync(logits, dl, n * 4, hipMemcpyDeviceToHost, ctx->stream);
     if (e == hipSuccess && probs) e = hipMemcpyAsync(probs, dp, n * 4, hipMemcpyDeviceToHost, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -637,32 +670,36 @@ int omega_moe_get_workspace(omega_moe *m, int which, int T, void *host_dst)
 int omega_moe_time_stage(omega_moe *m, int stage, const void *x, int T, void *out, int warmup, int iters, float *ms_avg)
 {
     MOE_ENTER(m);
-    RUN(check_T(m, x, T, stage == 0 || stage == 1 || stage == 5 || stage == 7));
+    RUN(check_T(m, x, T, stage == 0 || stage == 1 || stage == 5 || stage == 7 || stage == 8 || stage == 9));
     if ((stage == 6 || stage == 7) && m->bm == 0) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: dispatch has not run");
-    if (!ms_avg || iters <= 0 || warmup < 0 || stage < 0 || stage > 7 || T <= 0)
+    if (!ms_avg || iters <= 0 || warmup < 0 || stage < 0 || stage > 9 || T <= 0)
         OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: bad argument");
-    if ((stage == 4 || stage == 5) && !out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: out is NULL");
-    if (stage == 0 || stage == 5) RUN(moe_reserve(m, T));
+    if ((stage == 4 || stage == 5 || stage == 8) && !out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: out is NULL");
+    if (stage == 0 || stage == 5 || stage == 8 || stage == 9) RUN(moe_reserve(m, T));
     else if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: earlier stages have not run for this T");
     auto once = [&]() -> int {
         switch (stage) {
-            case 0: return stage_router(m, x, T);
-            case 1: return stage_dispatch(m, x, T);
+            case 0: return stage_router(m, x, T, 0);
+            case 1: return stage_dispatch(m, x, T, 0);
             case 2: return stage_experts(m, x, T, 0);
             case 3: return stage_experts(m, x, T, 1);
-            case 4: return stage_combine(m, T, out);
+            case 4: return stage_combine(m, T, out, nullptr);
             case 6:
                 OMEGA_HIP_CHECK(ctx, launch_dispatch_index(m, T, m->bm, ctx->stream));
                 return OMEGA_OK;
             case 7:
-                OMEGA_HIP_CHECK(ctx, launch_dispatch_gather(m, x, T, ctx->stream));
+                OMEGA_HIP_CHECK(ctx, launch_dispatch_gather(m, x, T, 0, ctx->stream));
+                return OMEGA_OK;
+            case 8: return forward_impl(m, x, T, out, 1);
+            case 9:
+                OMEGA_HIP_CHECK(ctx, launch_rms_stats(m, x, T, ctx->stream));
                 return OMEGA_OK;
             default:
-                RUN(stage_router(m, x, T));
-                RUN(stage_dispatch(m, x, T));
+                RUN(stage_router(m, x, T, 0));
+                RUN(stage_dispatch(m, x, T, 0));
                 RUN(stage_experts(m, x, T, 0));
                 RUN(stage_experts(m, x, T, 1));
-                return stage_combine(m, T, out);
+                return stage_combine(m, T, out, nullptr);
         }
     };
     for (int i = 0; i < warmup; ++i) RUN(once());

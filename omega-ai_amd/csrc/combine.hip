@@ -11,11 +11,13 @@
 
 // KU: slots whose rows are fetched together before any of them is used (all loads of a group are in flight at
 // once; slots beyond K re-read the last row and are ignored).
+// resid != nullptr (block form): the row of x is added to the fp32 sum before the output is rounded
+// (Tensor_OP().add(mlp out, tmp1, tmp2), J/engine/nn/layer/llama/LlamaTransformerBlock.java:136).
 template <int VEC, bool BF16, int KU>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ dst,
                                                       const float *__restrict__ w, int T, int K, int d, int Es,
                                                       const int32_t *__restrict__ tile_meta, int E, int bm,
-                                                      void *__restrict__ out)
+                                                      const void *__restrict__ resid, void *__restrict__ out)
 {
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -67,6 +69,20 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                 acc[q * 4 + 3] = acc[q * 4 + 3] + v4.w;
             }
         }
+        if (resid != nullptr) {
+            if (BF16) {
+                const uint4 u = *(const uint4 *)((const bf16_t *)resid + (size_t)t * d + c0);
+                const uint32_t uu[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int v = 0; v < VEC / 2; ++v) {
+                    acc[2 * v] = acc[2 * v] + __uint_as_float(uu[v] << 16);
+                    acc[2 * v + 1] = acc[2 * v + 1] + __uint_as_float(uu[v] & 0xffff0000u);
+                }
+            } else {
+                const float4 r4 = *(const float4 *)((const float *)resid + (size_t)t * d + c0);
+                acc[0] = acc[0] + r4.x; acc[1] = acc[1] + r4.y; acc[2] = acc[2] + r4.z; acc[3] = acc[3] + r4.w;
+            }
+        }
         if (BF16) {
             uint32_t pk[VEC / 2];
 #pragma unroll
@@ -86,7 +102,7 @@ template <bool BF16>
 __global__ __launch_bounds__(256) void combine_scalar_kernel(const float *__restrict__ y, const int32_t *__restrict__ dst,
                                                              const float *__restrict__ w, int T, int K, int d, int Es,
                                                              const int32_t *__restrict__ tile_meta, int E, int bm,
-                                                             void *__restrict__ out)
+                                                             const void *__restrict__ resid, void *__restrict__ out)
 {
     const int t = blockIdx.x;
     for (int c = threadIdx.x; c < d; c += 256) {
@@ -96,25 +112,27 @@ __global__ __launch_bounds__(256) void combine_scalar_kernel(const float *__rest
             acc = acc + term;
         }
         for (int s = 0; s < Es; ++s) acc = acc + y[((size_t)tile_meta[1 + E + s] * bm + t) * d + c];
+        if (resid != nullptr)
+            acc = acc + (BF16 ? bf16_to_f32(((const bf16_t *)resid)[(size_t)t * d + c]) : ((const float *)resid)[(size_t)t * d + c]);
         if (BF16) ((bf16_t *)out)[(size_t)t * d + c] = f32_to_bf16(acc);
         else ((float *)out)[(size_t)t * d + c] = acc;
     }
 }
 
-hipError_t launch_combine(const omega_moe *m, int T, void *out, hipStream_t s)
+hipError_t launch_combine(const omega_moe *m, int T, void *out, const void *resid, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
     const bool bf = c.dtype == OMEGA_DTYPE_BF16;
     const int vec = bf ? 8 : 4;
-    if (c.d % vec == 0 && ((uintptr_t)out % 16) == 0 && c.K <= MAXK) {
+    if (c.d % vec == 0 && (((uintptr_t)out | (uintptr_t)resid) % 16) == 0 && c.K <= MAXK) {
 #define COMBINE_LAUNCH(KUV)                                                                                          \
     do {                                                                                                            \
         if (bf)                                                                                                     \
             hipLaunchKernelGGL((combine_kernel<8, true, KUV>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dstp, m->w, \
-                               T, c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, out);                                   \
+                               T, c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, resid, out);                                   \
         else                                                                                                        \
             hipLaunchKernelGGL((combine_kernel<4, false, KUV>), dim3(ceil_div(T, 4)), dim3(256), 0, s, m->y, m->dstp, \
-                               m->w, T, c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, out);                             \
+                               m->w, T, c.K, c.d, c.Es, m->tile_meta, c.E, m->bm, resid, out);                             \
     } while (0)
         if (c.K <= 2) COMBINE_LAUNCH(2);
         else if (c.K <= 4) COMBINE_LAUNCH(4);
@@ -123,10 +141,10 @@ hipError_t launch_combine(const omega_moe *m, int T, void *out, hipStream_t s)
     } else {
         if (bf)
             hipLaunchKernelGGL(combine_scalar_kernel<true>, dim3(T), dim3(256), 0, s, m->y, m->dstp, m->w, T, c.K, c.d,
-                               c.Es, m->tile_meta, c.E, m->bm, out);
+                               c.Es, m->tile_meta, c.E, m->bm, resid, out);
         else
             hipLaunchKernelGGL(combine_scalar_kernel<false>, dim3(T), dim3(256), 0, s, m->y, m->dstp, m->w, T, c.K, c.d,
-                               c.Es, m->tile_meta, c.E, m->bm, out);
+                               c.Es, m->tile_meta, c.E, m->bm, resid, out);
     }
     return hipGetLastError();
 }

@@ -56,7 +56,10 @@ struct omega_moe {
     void *W1 = nullptr;   // [G,H,d]
     void *W3 = nullptr;   // [G,H,d]
     void *W2 = nullptr;   // [G,d,H]
+    float *gamma = nullptr;  // [d] weight of the RMSNorm in front of the layer (block form), fp32
+    bool gamma_set = false;
     // workspace
+    float *rms = nullptr;            // [T] row statistics of the pre-norm (block form)
     int32_t *ids = nullptr;          // [T,K]
     float *w = nullptr;              // [T,K]
     int32_t *tile_counts = nullptr;  // [n_tok_tiles,E] histogram per token tile (router)
@@ -109,12 +112,16 @@ hipError_t launch_fill_normal(void *dptr, uint64_t n, uint64_t seed, uint64_t st
                               int dtype, hipStream_t s);
 hipError_t launch_convert(void *dst, int dst_dtype, const void *src, int src_dtype, uint64_t n, hipStream_t s);
 
-hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s);
+// block != 0: the rows of x are normalised on the fly, h = (x / rms[t]) * gamma (rounded to bf16 in bf16 layers)
+hipError_t launch_rms_stats(const omega_moe *m, const void *x, int T, hipStream_t s);
+hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, int block,
+                         hipStream_t s);
 hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s);
-hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipStream_t s);
+hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, int block, hipStream_t s);
 hipError_t launch_experts_f32(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
 hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
-hipError_t launch_combine(const omega_moe *m, int T, void *out, hipStream_t s);
+// resid != nullptr: out = resid + layer output (one rounding of the fp32 sum)
+hipError_t launch_combine(const omega_moe *m, int T, void *out, const void *resid, hipStream_t s);
 hipError_t launch_pack_rows(void *dst_packed, const void *src_rowmajor, int R, int Kd, hipStream_t s);
 hipError_t launch_unpack_rows(void *dst_rowmajor, const void *src_packed, int R, int Kd, hipStream_t s);
 int experts_bf16_tile_m(const omega_moe *m, int T);
@@ -130,5 +137,14 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f)
     if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
     u += 0x7fffu + ((u >> 16) & 1u);
     return (bf16_t)(u >> 16);
+}
+// One element of the pre-norm: (x / rms) * weight with two roundings, as rmsnorm_forward_kernel2 writes it
+// (J/engine/nn/layer/normalization/gpu/RMSKernel.cu:218-222); bf16 layers store the result as bf16.
+template <bool XBF>
+__device__ __forceinline__ float norm_apply(float v, float rms, float g)
+{
+    const float n = v / rms;
+    const float h = n * g;
+    return XBF ? bf16_to_f32(f32_to_bf16(h)) : h;
 }
 #endif

@@ -121,6 +121,8 @@ public:
         upload(OMEGA_W_GATE, 0, Wg, (size_t)nExperts_ * embedDim_);
         if (bg) check(ctx_.get(), omega_moe_set_weights(moe_, OMEGA_W_GATE_BIAS, 0, bg, 0));
     }
+    // weight of the RMSNorm in front of the layer (norm2 of the block), fp32
+    void setNorm(const float *gamma) { check(ctx_.get(), omega_moe_set_weights(moe_, OMEGA_W_NORM, 0, gamma, 0)); }
     void setExpert(int g, const float *W1, const float *W3, const float *W2)
     {
         const size_t n = (size_t)hidden_ * embedDim_;
@@ -144,16 +146,16 @@ public:
     }
     void initBack() override {}
     void initParam() override {}
-    void output() override
+    void output() override { run(false); }
+    // second half of the transformer block in one call: output = input + layer(rmsnorm(input))
+    // (getNorm2().forward(tmp1); getMlp().forward(...); Tensor_OP().add(mlp out, tmp1, tmp2),
+    //  J/engine/nn/layer/llama/LlamaTransformerBlock.java:134-136); setNorm must have been called
+    void forwardBlock(Tensor &in)
     {
-        const size_t n = (size_t)number * embedDim_;
-        if (dtype_ == OMEGA_DTYPE_BF16) {
-            check(ctx_.get(), omega_hip_convert(ctx_.get(), xLow_, OMEGA_DTYPE_BF16, input->gpuData, OMEGA_DTYPE_F32, n));
-            check(ctx_.get(), omega_moe_forward(moe_, xLow_, number, outLow_));
-            check(ctx_.get(), omega_hip_convert(ctx_.get(), output_->gpuData, OMEGA_DTYPE_F32, outLow_, OMEGA_DTYPE_BF16, n));
-        } else {
-            check(ctx_.get(), omega_moe_forward(moe_, input->gpuData, number, output_->gpuData));
-        }
+        if (in.width != embedDim_ || !in.isHasGPU()) throw std::runtime_error("Error code 1:input width does not match embedDim or tensor has no device data");
+        setInput(in);
+        init();
+        run(true);
     }
     Tensor *getOutput() override { return output_.get(); }
     void forward() override
@@ -187,6 +189,18 @@ public:
     void loadModel(FILE *f) { eachParam([&](int which, int g, size_t n) { std::vector<float> h(n); if (fread(h.data(), 4, n, f) != n) throw std::runtime_error("Error code 1:checkpoint ends early"); if (which == OMEGA_W_GATE_BIAS) check(ctx_.get(), omega_moe_set_weights(moe_, which, g, h.data(), 0)); else upload(which, g, h.data(), n); }); }
 
 private:
+    void run(bool block)
+    {
+        const size_t n = (size_t)number * embedDim_;
+        auto fwd = block ? omega_moe_forward_block : omega_moe_forward;
+        if (dtype_ == OMEGA_DTYPE_BF16) {
+            check(ctx_.get(), omega_hip_convert(ctx_.get(), xLow_, OMEGA_DTYPE_BF16, input->gpuData, OMEGA_DTYPE_F32, n));
+            check(ctx_.get(), fwd(moe_, xLow_, number, outLow_));
+            check(ctx_.get(), omega_hip_convert(ctx_.get(), output_->gpuData, OMEGA_DTYPE_F32, outLow_, OMEGA_DTYPE_BF16, n));
+        } else {
+            check(ctx_.get(), fwd(moe_, input->gpuData, number, output_->gpuData));
+        }
+    }
     [[noreturn]] static void unsupported() { throw std::logic_error("MoELayer is forward-only"); }
     template <class F> void eachParam(F f)
     {

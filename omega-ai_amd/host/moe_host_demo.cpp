@@ -45,6 +45,18 @@ int main(int argc, char **argv)
         FILE *fi = fopen((dir + "/ids.bin").c_str(), "wb");
         fwrite(ids.data(), 4, ids.size(), fi);
         fclose(fi);
+        // block form (norm2 -> mlp -> residual add), when the directory holds the norm weight
+        if (FILE *fg = fopen((dir + "/gamma.bin").c_str(), "rb")) {
+            fclose(fg);
+            std::vector<float> gamma = read_f32(dir + "/gamma.bin", (size_t)d);
+            mlp.setNorm(gamma.data());
+            mlp.forwardBlock(x);
+            omega::Tensor *ob = mlp.getOutput();
+            ob->syncHost();
+            FILE *fb = fopen((dir + "/out_block.bin").c_str(), "wb");
+            fwrite(ob->data.data(), 4, ob->data.size(), fb);
+            fclose(fb);
+        }
         // round trip of the checkpoint format
         FILE *sv = fopen((dir + "/model_saved.bin").c_str(), "wb");
         mlp.saveModel(sv);

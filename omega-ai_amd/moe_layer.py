@@ -120,7 +120,7 @@ class MoELayer:
 
     # ---- parameters
     def _upload(self, which, expert, a):
-        if which == L.W_GATE_BIAS or self.dtype == "f32":
+        if which in (L.W_GATE_BIAS, L.W_NORM) or self.dtype == "f32":
             h = np.ascontiguousarray(a, np.float32)
         else:
             h = f32_to_bf16_bits(a)
@@ -132,6 +132,11 @@ class MoELayer:
         if bg is not None:
             assert self.hasBias and bg.shape == (self.nExperts,)
             self._upload(L.W_GATE_BIAS, 0, bg)
+
+    def set_norm(self, gamma):
+        """Weight of the RMSNorm in front of the layer (block form, forward_block); always fp32."""
+        assert gamma.shape == (self.embedDim,)
+        self._upload(L.W_NORM, 0, gamma)
 
     def set_expert(self, g, W1, W3, W2):
         assert W1.shape == (self.hidden, self.embedDim) and W3.shape == W1.shape
@@ -159,6 +164,12 @@ class MoELayer:
         bg = cfgmod.zipf_gate_bias(cfg, seed)
         if bg is not None:
             self._upload(L.W_GATE_BIAS, 0, bg)
+        # norm weight of the block form: 1 + 0.1 * N(0,1), drawn on the device as fp32
+        gam = DeviceBuffer(self.ctx, (self.embedDim,), "f32")
+        self.ctx.check(fill(self.ctx.handle, gam.ptr, self.embedDim, seed, cfgmod.STREAM_NORM, 1.0, 0, L.DTYPE_F32))
+        g = gam.to_numpy() * np.float32(0.1) + np.float32(1.0)
+        gam.free()
+        self.set_norm(g.astype(np.float32))
         self.ctx.sync()
 
     # ---- Layer contract
@@ -183,6 +194,21 @@ class MoELayer:
         self.init()
         self.output()
         return self.output_buf
+
+    def forward_block(self, inp):
+        """out = inp + layer(rmsnorm(inp)): norm2 -> mlp -> residual add of LlamaTransformerBlock.output
+        (J/engine/nn/layer/llama/LlamaTransformerBlock.java:134-136) in one call."""
+        self.setInput(inp)
+        self.init()
+        self.ctx.check(self.lib.omega_moe_forward_block(self.handle, self.input.ptr, self.number, self.output_buf.ptr))
+        return self.output_buf
+
+    def norm_rms(self, T=None):
+        """rms[t] of the last forward_block (host copy)."""
+        T = self.number if T is None else T
+        r = np.empty(T, np.float32)
+        self.ctx.check(self.lib.omega_moe_get_norm(self.handle, T, r.ctypes.data))
+        return r
 
     def getOutput(self):
         return self.output_buf

@@ -19,6 +19,11 @@
  *   orc_dispatch         stable argsort brute force, bijection / stability invariants (pinned)
  *   orc_swiglu_rows      fp64 cross-check, SiLU closed forms                  (pinned to tolerance; GEMM bits unpinned as above)
  *   orc_combine / orc_moe_forward   dense-MoE identity in fp64                (pinned)
+ *   orc_rmsnorm          NumPy twin written from the kernel text (bit-exact), closed forms (all-ones row,
+ *                        scale invariance), fp64 formula to 1e-6 (pinned, except the order of the five
+ *                        additions inside cooperative_groups::reduce, which is library code outside the
+ *                        reference tree: taken as the xor butterfly, "parity unpinned" at the ulp level)
+ *   orc_block_tokens / orc_block_forward   residual identity out - x == layer(rmsnorm(x)) (pinned by composition)
  *
  * Build: make -C oracle   (gcc -O2 -ffp-contract=off; no fast-math, so every float
  * operation below is a single IEEE-754 rounding in the order written).
@@ -274,8 +279,8 @@ void orc_swiglu_rows(const float *xg, int rows, const float *W1, const float *W3
 /* S7 combine: out[t,:] = sum_j w[t,j]*y[dst[t*K+j],:] in slot order (weighted sum shaped like
  * add_mul_kernel, J/engine/gpu/BaseKernel.cu:228-241), then + shared-expert rows
  * (add: J/engine/ad/op/gpu/OPKernel.cu:359-366).  yshared may be NULL; it is [Es,T,d]. */
-void orc_combine(const float *y, const int32_t *dst, const float *w, const float *yshared, int T, int K, int d,
-                 int Es, int bf16_mode, float *out)
+void orc_combine_resid(const float *y, const int32_t *dst, const float *w, const float *yshared, const float *resid,
+                       int T, int K, int d, int Es, int bf16_mode, float *out)
 {
     for (int t = 0; t < T; ++t)
         for (int c = 0; c < d; ++c) {
@@ -285,16 +290,58 @@ void orc_combine(const float *y, const int32_t *dst, const float *w, const float
                 acc = acc + term;
             }
             for (int s = 0; s < Es; ++s) acc = acc + yshared[((size_t)s * T + t) * d + c];
+            /* block form: the residual is added to the fp32 sum before the one rounding of the output
+             * (Tensor_OP().add(mlp_out, tmp1, tmp2), J/engine/nn/layer/llama/LlamaTransformerBlock.java:136;
+             * add_kernel, J/engine/ad/op/gpu/OPKernel.cu:359-366) */
+            if (resid) acc = acc + resid[(size_t)t * d + c];
             out[(size_t)t * d + c] = bf16_mode ? bf16_round(acc) : acc;
         }
+}
+
+void orc_combine(const float *y, const int32_t *dst, const float *w, const float *yshared, int T, int K, int d,
+                 int Es, int bf16_mode, float *out)
+{
+    orc_combine_resid(y, dst, w, yshared, NULL, T, K, d, Es, bf16_mode, out);
+}
+
+/* Pre-norm of the block: rmsnorm_forward_kernel2 (J/engine/nn/layer/normalization/gpu/RMSKernel.cu:185-223), the
+ * kernel RMSLayer.output runs (J/engine/nn/layer/normalization/RMSLayer.java:230 -> RMSKernel.java:232-249).
+ * One 32-lane group per row: lane l adds x[i]*x[i] for i = l, l+32, ... in index order (written
+ * `sum_squares += x[i] * x[i]`, one fused multiply-add per step under nvcc's default contraction); the 32 partial
+ * sums are combined by cooperative_groups::reduce(warp, ., plus), taken here as the xor butterfly with strides
+ * 16, 8, 4, 2, 1; rms = sqrtf(sum / C + 1e-6f); out[c] = (x[c] / rms) * weight[c].
+ * bf16 mode: the normalised row is rounded to bf16 (the activation storage type).  rms_o may be NULL. */
+void orc_rmsnorm(const float *x, const float *gamma, int T, int d, int bf16_mode, float *h, float *rms_o)
+{
+    for (int t = 0; t < T; ++t) {
+        const float *xr = x + (size_t)t * d;
+        float part[32];
+        for (int l = 0; l < 32; ++l) {
+            float s = 0.0f;
+            for (int i = l; i < d; i += 32) s = fmaf(xr[i], xr[i], s);
+            part[l] = s;
+        }
+        for (int m = 16; m >= 1; m >>= 1) {
+            float nxt[32];
+            for (int l = 0; l < 32; ++l) nxt[l] = part[l] + part[l ^ m];
+            memcpy(part, nxt, sizeof(part));
+        }
+        float rms = sqrtf(part[0] / (float)d + 1e-6f);
+        if (rms_o) rms_o[t] = rms;
+        for (int c = 0; c < d; ++c) {
+            float n = xr[c] / rms;
+            float v = n * gamma[c];
+            h[(size_t)t * d + c] = bf16_mode ? bf16_round(v) : v;
+        }
+    }
 }
 
 /* Whole layer for a subset of tokens (tok_list, n_tok) of a T-token batch whose routing
  * (ids, w over all T tokens) is already known: used to check full-size runs on a sample.
  * W1,W3,W2 hold E+Es experts back to back.  out is [n_tok, d]. */
-void orc_moe_tokens(const float *x, const int32_t *ids, const float *w, const float *W1, const float *W3,
-                    const float *W2, int d, int H, int E, int K, int Es, int bf16_mode, const int32_t *tok_list,
-                    int n_tok, float *out)
+static void moe_tokens_impl(const float *x, const float *resid, const int32_t *ids, const float *w, const float *W1,
+                            const float *W3, const float *W2, int d, int H, int E, int K, int Es, int bf16_mode,
+                            const int32_t *tok_list, int n_tok, float *out)
 {
     float *scratch = (float *)malloc(sizeof(float) * (size_t)H);
     float *yk = (float *)malloc(sizeof(float) * (size_t)d * (size_t)(K + Es));
@@ -313,6 +360,7 @@ void orc_moe_tokens(const float *x, const int32_t *ids, const float *w, const fl
                 acc = acc + term;
             }
             for (int s = 0; s < Es; ++s) acc = acc + yk[(size_t)(K + s) * d + c];
+            if (resid) acc = acc + resid[(size_t)t * d + c];
             out[(size_t)i * d + c] = bf16_mode ? bf16_round(acc) : acc;
         }
     }
@@ -320,12 +368,29 @@ void orc_moe_tokens(const float *x, const int32_t *ids, const float *w, const fl
     free(yk);
 }
 
+void orc_moe_tokens(const float *x, const int32_t *ids, const float *w, const float *W1, const float *W3,
+                    const float *W2, int d, int H, int E, int K, int Es, int bf16_mode, const int32_t *tok_list,
+                    int n_tok, float *out)
+{
+    moe_tokens_impl(x, NULL, ids, w, W1, W3, W2, d, H, E, K, Es, bf16_mode, tok_list, n_tok, out);
+}
+
+/* Block form for a subset of tokens: the layer runs on h = rmsnorm(x) (rows of h for all T tokens, as the routing
+ * ids/w were computed from them) and x is added back: out = x + layer(h)
+ * (getNorm2().forward(tmp1); getMlp().forward(norm2 out); add(mlp out, tmp1), LlamaTransformerBlock.java:134-136). */
+void orc_block_tokens(const float *x, const float *h, const int32_t *ids, const float *w, const float *W1,
+                      const float *W3, const float *W2, int d, int H, int E, int K, int Es, int bf16_mode,
+                      const int32_t *tok_list, int n_tok, float *out)
+{
+    moe_tokens_impl(h, x, ids, w, W1, W3, W2, d, H, E, K, Es, bf16_mode, tok_list, n_tok, out);
+}
+
 /* Whole layer, all tokens, through the materialised dispatch (S1..S7). Outputs every
  * intermediate the parity tests compare.  Any output pointer except `out` may be NULL. */
-void orc_moe_forward(const float *x, const float *Wg, const float *bg, const float *W1, const float *W3,
-                     const float *W2, int T, int d, int E, int K, int H, int Es, int renorm, int bf16_mode,
-                     float *logits_o, float *p_o, int32_t *ids_o, float *w_o, int32_t *counts_o,
-                     int32_t *offsets_o, int32_t *dst_o, int32_t *src_row_o, float *out)
+static void moe_forward_impl(const float *x, const float *resid, const float *Wg, const float *bg, const float *W1,
+                             const float *W3, const float *W2, int T, int d, int E, int K, int H, int Es, int renorm,
+                             int bf16_mode, float *logits_o, float *p_o, int32_t *ids_o, float *w_o,
+                             int32_t *counts_o, int32_t *offsets_o, int32_t *dst_o, int32_t *src_row_o, float *out)
 {
     int P = T * K;
     float *logits = (float *)malloc(sizeof(float) * (size_t)T * E);
@@ -352,7 +417,7 @@ void orc_moe_forward(const float *x, const float *Wg, const float *bg, const flo
     for (int s = 0; s < Es; ++s)
         orc_swiglu_rows(x, T, W1 + (size_t)(E + s) * H * d, W3 + (size_t)(E + s) * H * d,
                         W2 + (size_t)(E + s) * d * H, d, H, bf16_mode, ysh + (size_t)s * T * d, scratch);
-    orc_combine(y, dst, w, ysh, T, K, d, Es, bf16_mode, out);
+    orc_combine_resid(y, dst, w, ysh, resid, T, K, d, Es, bf16_mode, out);
 
     if (logits_o) memcpy(logits_o, logits, sizeof(float) * (size_t)T * E);
     if (p_o) memcpy(p_o, p, sizeof(float) * (size_t)T * E);
@@ -364,4 +429,26 @@ void orc_moe_forward(const float *x, const float *Wg, const float *bg, const flo
     if (src_row_o) memcpy(src_row_o, src_row, sizeof(int32_t) * (size_t)P);
     free(logits); free(p); free(ids); free(w); free(counts); free(offsets); free(dst); free(src_row);
     free(xg); free(y); free(ysh); free(scratch);
+}
+
+void orc_moe_forward(const float *x, const float *Wg, const float *bg, const float *W1, const float *W3,
+                     const float *W2, int T, int d, int E, int K, int H, int Es, int renorm, int bf16_mode,
+                     float *logits_o, float *p_o, int32_t *ids_o, float *w_o, int32_t *counts_o,
+                     int32_t *offsets_o, int32_t *dst_o, int32_t *src_row_o, float *out)
+{
+    moe_forward_impl(x, NULL, Wg, bg, W1, W3, W2, T, d, E, K, H, Es, renorm, bf16_mode, logits_o, p_o, ids_o, w_o,
+                     counts_o, offsets_o, dst_o, src_row_o, out);
+}
+
+/* Block form, all tokens: h = rmsnorm(x) (returned in h_o, [T,d]; rms in rms_o, may be NULL), the layer on h,
+ * out = x + layer(h)  (LlamaTransformerBlock.java:134-136). */
+void orc_block_forward(const float *x, const float *gamma, const float *Wg, const float *bg, const float *W1,
+                       const float *W3, const float *W2, int T, int d, int E, int K, int H, int Es, int renorm,
+                       int bf16_mode, float *h_o, float *rms_o, float *logits_o, float *p_o, int32_t *ids_o,
+                       float *w_o, int32_t *counts_o, int32_t *offsets_o, int32_t *dst_o, int32_t *src_row_o,
+                       float *out)
+{
+    orc_rmsnorm(x, gamma, T, d, bf16_mode, h_o, rms_o);
+    moe_forward_impl(h_o, x, Wg, bg, W1, W3, W2, T, d, E, K, H, Es, renorm, bf16_mode, logits_o, p_o, ids_o, w_o,
+                     counts_o, offsets_o, dst_o, src_row_o, out);
 }

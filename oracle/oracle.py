@@ -44,6 +44,10 @@ def lib():
         L.orc_combine.argtypes = [_f, _i, _f, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _f]
         L.orc_moe_tokens.argtypes = [_f, _i, _f, _f, _f, _f] + [C.c_int] * 6 + [_i, C.c_int, _f]
         L.orc_moe_forward.argtypes = [_f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8 + [_f, _f, _i, _f, _i, _i, _i, _i, _f]
+        L.orc_rmsnorm.argtypes = [_f, _f, C.c_int, C.c_int, C.c_int, _f, _f]
+        L.orc_block_tokens.argtypes = [_f, _f, _i, _f, _f, _f, _f] + [C.c_int] * 6 + [_i, C.c_int, _f]
+        L.orc_block_forward.argtypes = ([_f, _f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8
+                                        + [_f, _f, _f, _f, _i, _f, _i, _i, _i, _i, _f])
         L.orc_cpu_baseline_forward.restype = C.c_double
         L.orc_cpu_baseline_forward.argtypes = [_f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8 + [_f]
         L.orc_cpu_sgemm_tn.argtypes = [C.c_int, C.c_int, C.c_int, _f, C.c_int, _f, C.c_int, _f, C.c_int, C.c_int]
@@ -131,6 +135,42 @@ def moe_forward(x, Wg, bg, W1, W3, W2, K, renorm, Es=0, bf16=False):
              dst=np.empty(P, np.int32), src_row=np.empty(P, np.int32), out=np.empty((T, d), np.float32))
     lib().orc_moe_forward(x, Wg, _opt(bg), W1, W3, W2, T, d, E, K, H, Es, int(renorm), int(bf16), r["logits"],
                           r["p"], r["ids"], r["w"], r["counts"], r["offsets"], r["dst"], r["src_row"], r["out"])
+    return r
+
+
+def rmsnorm(x, gamma, bf16=False):
+    """Pre-norm of the block: returns (h [T,d], rms [T])."""
+    T, d = x.shape
+    h, rms = np.empty((T, d), np.float32), np.empty(T, np.float32)
+    lib().orc_rmsnorm(np.ascontiguousarray(x), np.ascontiguousarray(gamma, np.float32), T, d, int(bf16), h, rms)
+    return h, rms
+
+
+def block_tokens(x, h, ids, w, W1, W3, W2, E, Es, tokens, bf16=False):
+    """x + layer(h) for the listed tokens only (h = rmsnorm(x) for all tokens, routing given)."""
+    T, d = x.shape
+    K = ids.shape[1]
+    H = W1.shape[1]
+    tok = np.ascontiguousarray(tokens, np.int32)
+    out = np.empty((len(tok), d), np.float32)
+    lib().orc_block_tokens(x, np.ascontiguousarray(h), np.ascontiguousarray(ids), np.ascontiguousarray(w), W1, W3, W2,
+                           d, H, E, K, Es, int(bf16), tok, len(tok), out)
+    return out
+
+
+def block_forward(x, gamma, Wg, bg, W1, W3, W2, K, renorm, Es=0, bf16=False):
+    """out = x + layer(rmsnorm(x)); returns every intermediate, including h and rms."""
+    T, d = x.shape
+    E = Wg.shape[0]
+    H = W1.shape[1]
+    P = T * K
+    r = dict(h=np.empty((T, d), np.float32), rms=np.empty(T, np.float32), logits=np.empty((T, E), np.float32),
+             p=np.empty((T, E), np.float32), ids=np.empty((T, K), np.int32), w=np.empty((T, K), np.float32),
+             counts=np.empty(E, np.int32), offsets=np.empty(E + 1, np.int32), dst=np.empty(P, np.int32),
+             src_row=np.empty(P, np.int32), out=np.empty((T, d), np.float32))
+    lib().orc_block_forward(x, np.ascontiguousarray(gamma, np.float32), Wg, _opt(bg), W1, W3, W2, T, d, E, K, H, Es,
+                            int(renorm), int(bf16), r["h"], r["rms"], r["logits"], r["p"], r["ids"], r["w"],
+                            r["counts"], r["offsets"], r["dst"], r["src_row"], r["out"])
     return r
 
 

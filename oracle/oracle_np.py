@@ -154,3 +154,26 @@ def rel_l2(a, b):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
     return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
+
+
+def rmsnorm_lanes(x, gamma, bf16=False):
+    """rmsnorm_forward_kernel2 (RMSKernel.cu:185-223) written from the kernel text: 32 lanes per row, lane l adds
+    x[i]^2 for i = l, l+32, ... with one fused multiply-add per step, xor butterfly 16..1 over the lanes,
+    rms = sqrt(sum/C + 1e-6), out = (x/rms)*weight - every operation rounded to float32 as the kernel does.
+    (The fused multiply-add is emulated in float64: the product of two float32 is exact there.)"""
+    x = np.asarray(x, np.float32)
+    T, d = x.shape
+    pad = (-d) % 32
+    xp = np.concatenate([x, np.zeros((T, pad), np.float32)], axis=1).reshape(T, -1, 32)
+    s = np.zeros((T, 32), np.float32)
+    for j in range(xp.shape[1]):
+        v = xp[:, j, :].astype(np.float64)
+        s = (v * v + s.astype(np.float64)).astype(np.float32)
+    lanes = np.arange(32)
+    for m in (16, 8, 4, 2, 1):
+        s = (s + s[:, lanes ^ m]).astype(np.float32)
+    rms = np.sqrt((s[:, 0] / np.float32(d)).astype(np.float32) + np.float32(1e-6)).astype(np.float32)
+    h = ((x / rms[:, None]).astype(np.float32) * np.asarray(gamma, np.float32)[None, :]).astype(np.float32)
+    if bf16:
+        h = round_bf16(h)
+    return h, rms

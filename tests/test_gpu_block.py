@@ -1,0 +1,102 @@
+"""Block form through the C ABI: out = x + layer(rmsnorm(x)) against the oracle.
+
+Row statistics, routing of the normalised rows (ids, weights, counts, offsets, permutation) and the gathered
+normalised rows are compared bit for bit; outputs to 1e-5 (fp32) / 1e-2 (bf16) relative L2.  The plain forward of the
+same layer must be unaffected by a block call before it."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from oracle import oracle_np as N
+from tests.synth import C, make_inputs, scaled
+
+pytestmark = pytest.mark.gpu
+
+SEED = 20251
+
+
+def _gamma(d, seed):
+    return (O.fill_normal(d, seed, C.STREAM_NORM, 1.0) * np.float32(0.1) + np.float32(1.0)).astype(np.float32)
+
+
+CASES = [
+    ("c1_tiny_f32", {}),
+    ("c1_tiny_f32", dict(T=77, d=102, H=72)),                      # unaligned rows: element-wise paths
+    ("c4_finegrained", dict(T=96, d=128, H=64, E=8, K=3, Es=2, dtype="f32")),   # shared experts read the normalised rows
+    ("c2_mixtral", dict(T=300, d=256, H=384)),
+    ("c4_finegrained", dict(T=200, d=256, H=256, E=16, K=4, Es=2)),
+    ("c5_skewed", dict(T=257, d=512, H=256, E=32, K=4)),
+]
+
+
+@pytest.mark.parametrize("name,kw", CASES)
+def test_block_forward_matches_oracle(name, kw):
+    from tests import gpu_util as G
+    cfg = scaled(C.CONFIGS[name], **kw)
+    bf = cfg.dtype == "bf16"
+    inp = make_inputs(cfg, 77)
+    gamma = _gamma(cfg.d, 77)
+    layer = G.build_layer(cfg, inp)
+    with pytest.raises(RuntimeError):  # the norm weight has not been set yet
+        layer.forward_block(G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype))
+    layer.set_norm(gamma)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    out = layer.forward_block(x).to_numpy()
+    ref = O.block_forward(inp["x"], gamma, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm,
+                          cfg.Es, bf)
+    assert np.array_equal(layer.norm_rms().view(np.uint32), ref["rms"].view(np.uint32))
+    r = layer.routing()
+    G.assert_routing_bit_exact(r, ref)
+    assert np.array_equal(layer.workspace("xg", cfg.T), ref["h"][ref["src_row"]])
+    err = N.rel_l2(out, ref["out"])
+    assert err < (1e-2 if bf else 1e-5), err
+    # the same call again gives the same bits, and the plain forward is what it was
+    assert np.array_equal(layer.forward_block(x).to_numpy(), out)
+    plain = layer.forward(x).to_numpy()
+    pref = G.oracle_forward(cfg, inp)
+    G.assert_routing_bit_exact(layer.routing(), pref)
+    assert N.rel_l2(plain, pref["out"]) < (1e-2 if bf else 1e-5)
+    layer.close()
+
+
+def test_block_forward_full_size_mixtral():
+    """C2 at full size: statistics and routing of all tokens bit for bit, output on sampled tokens."""
+    from tests import gpu_util as G
+    P, L = G.P, __import__("importlib").import_module("omega-ai_amd._lib")
+    cfg = C.CONFIGS["c2_mixtral"]
+    layer = P.MoELayer(cfg.d, cfg.H, cfg.E, cfg.K, renorm=cfg.renorm, nShared=cfg.Es, bias=cfg.has_gate_bias,
+                       ctx=G.ctx(), dtype=cfg.dtype, router_mode="exact", T_max=cfg.T)
+    layer.init_synthetic(SEED, C, cfg)
+    x = P.DeviceBuffer(G.ctx(), (cfg.T, cfg.d), cfg.dtype)
+    x.fill_normal(SEED, C.STREAM_X, C.tensor_std(cfg, "x"))
+    out = layer.forward_block(x).to_numpy()
+    xh = x.to_numpy()
+    gamma = _gamma(cfg.d, SEED)
+    h, rms = O.rmsnorm(xh, gamma, True)
+    assert np.array_equal(layer.norm_rms().view(np.uint32), rms.view(np.uint32))
+    Wg = layer._download_weight(L.W_GATE, 0, (cfg.E, cfg.d))
+    ids, w = O.topk(O.softmax(O.gate(h, Wg, None)), cfg.K, cfg.renorm)
+    r = layer.routing()
+    assert np.array_equal(r["ids"], ids)
+    assert np.array_equal(r["w"].view(np.uint32), w.view(np.uint32))
+    counts, offsets, dst, src = N.dispatch_argsort(ids, cfg.E)
+    for k, v in (("counts", counts), ("offsets", offsets), ("dst", dst), ("src_row", src)):
+        assert np.array_equal(r[k], v), k
+    assert np.array_equal(layer.workspace("xg", cfg.T), h[src])
+    tok = np.unique(np.linspace(0, cfg.T - 1, 6).astype(np.int32))
+    need = sorted(set(r["ids"][tok].ravel().tolist()))
+    remap = {g: i for i, g in enumerate(need)}
+    W1 = np.stack([layer._download_weight(L.W_W1, g, (cfg.H, cfg.d)) for g in need])
+    W3 = np.stack([layer._download_weight(L.W_W3, g, (cfg.H, cfg.d)) for g in need])
+    W2 = np.stack([layer._download_weight(L.W_W2, g, (cfg.d, cfg.H)) for g in need])
+    ids_c = np.vectorize(remap.get)(r["ids"][tok]).astype(np.int32)
+    ref = O.block_tokens(np.ascontiguousarray(xh[tok]), np.ascontiguousarray(h[tok]), ids_c,
+                         np.ascontiguousarray(r["w"][tok]), W1, W3, W2, len(need), 0,
+                         np.arange(len(tok), dtype=np.int32), bf16=True)
+    assert N.rel_l2(out[tok], ref) < 1e-2
+    assert np.isfinite(out).all()
+    # residual identity on the whole batch: out - x is the layer applied to h, whose plain forward we can run
+    hbuf = P.DeviceBuffer.from_numpy(G.ctx(), h, cfg.dtype)
+    lay = layer.forward(hbuf).to_numpy()
+    assert N.rel_l2(out.astype(np.float64) - xh, lay) < 5e-2
+    layer.close()

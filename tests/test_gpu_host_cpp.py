@@ -28,6 +28,8 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
         model = np.concatenate([inp["Wg"].ravel()] + [np.concatenate([inp["W1"][g].ravel(), inp["W3"][g].ravel(),
                                                                      inp["W2"][g].ravel()]) for g in range(G)])
         model.astype("<f4").tofile(os.path.join(td, "model.bin"))
+        gamma = (O.fill_normal(cfg.d, 17, C.STREAM_NORM, 1.0) * np.float32(0.1) + np.float32(1.0)).astype(np.float32)
+        gamma.astype("<f4").tofile(os.path.join(td, "gamma.bin"))
         r = subprocess.run([DEMO, td, str(cfg.T), str(cfg.d), str(cfg.E), str(cfg.K), str(cfg.H), str(cfg.Es), "1",
                             "1" if dtype == "bf16" else "0"], capture_output=True, text=True, timeout=100)
         assert r.returncode == 0, r.stderr
@@ -35,7 +37,11 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
         out = np.fromfile(os.path.join(td, "out.bin"), "<f4").reshape(cfg.T, cfg.d)
         ids = np.fromfile(os.path.join(td, "ids.bin"), "<i4").reshape(cfg.T, cfg.K)
         saved = np.fromfile(os.path.join(td, "model_saved.bin"), "<f4")
+        out_block = np.fromfile(os.path.join(td, "out_block.bin"), "<f4").reshape(cfg.T, cfg.d)
     ref = O.moe_forward(inp["x"], inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es, bf16=dtype == "bf16")
     assert np.array_equal(ids, ref["ids"])
     assert N.rel_l2(out, ref["out"]) <= (1e-2 if dtype == "bf16" else 1e-5)
     assert np.array_equal(saved, model.astype(np.float32))      # checkpoint round trip is byte-exact
+    blk = O.block_forward(inp["x"], gamma, inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es,
+                          bf16=dtype == "bf16")
+    assert N.rel_l2(out_block, blk["out"]) <= (1e-2 if dtype == "bf16" else 1e-5)   # forwardBlock of the C++ layer

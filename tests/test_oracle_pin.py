@@ -240,3 +240,74 @@ def test_zipf_bias_shape():
     ranks = np.sort(w)[::-1]
     assert np.allclose(ranks[0] / ranks[1], 2 ** 1.2, rtol=1e-5)
     assert not np.array_equal(bg, C.zipf_gate_bias(cfg, 2))
+
+
+# ---------------------------------------------------------------- block form: pre-norm and residual
+@pytest.mark.parametrize("T,d", [(7, 128), (3, 100), (2, 33), (4, 4096)])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_rmsnorm_against_kernel_text_twin(T, d, bf16):
+    rng = np.random.default_rng(T * 1000 + d)
+    x = (rng.standard_normal((T, d)) * 3).astype(np.float32)
+    g = rng.standard_normal(d).astype(np.float32)
+    if bf16:
+        x = O.round_bf16(x)
+    h, rms = O.rmsnorm(x, g, bf16)
+    h2, rms2 = N.rmsnorm_lanes(x, g, bf16)
+    assert np.array_equal(rms.view(np.uint32), rms2.view(np.uint32))
+    assert np.array_equal(h.view(np.uint32), h2.view(np.uint32))
+    # the definition in fp64: x / sqrt(mean(x^2) + 1e-6) * g
+    x64 = x.astype(np.float64)
+    ref = x64 / np.sqrt((x64**2).mean(1, keepdims=True) + 1e-6) * g.astype(np.float64)
+    tol = 1e-2 if bf16 else 1e-6
+    assert N.rel_l2(h, ref) < tol
+
+
+def test_rmsnorm_closed_forms_and_lane_order():
+    d = 256
+    g = np.linspace(-1, 1, d).astype(np.float32)
+    # a row of ones: every lane holds d/32 exactly, the sum is exactly d, rms = sqrt(1 + 1e-6)
+    h, rms = O.rmsnorm(np.ones((1, d), np.float32), g)
+    r = np.sqrt(np.float32(1.0) + np.float32(1e-6)).astype(np.float32)
+    assert rms[0] == r
+    assert np.array_equal(h[0], (np.float32(1.0) / r * g).astype(np.float32))
+    # a row of zeros: rms = sqrt(1e-6), output exactly zero (no NaN)
+    h, rms = O.rmsnorm(np.zeros((1, d), np.float32), g)
+    assert rms[0] == np.sqrt(np.float32(1e-6)) and not h.any()
+    # doubling the row doubles rms up to the 1e-6 term
+    x = np.random.default_rng(3).standard_normal((1, d)).astype(np.float32)
+    _, r1 = O.rmsnorm(x, g)
+    _, r2 = O.rmsnorm(2 * x, g)
+    assert abs(r2[0] / r1[0] - 2) < 1e-5
+    # the order of the additions is part of the definition: a plain left-to-right sum of squares gives other bits
+    # on some rows, so a restatement that ignored the 32-lane structure would fail the twin test above
+    X = (np.random.default_rng(4).standard_normal((64, 4096)) * 3).astype(np.float32)
+    _, rms = O.rmsnorm(X, np.ones(4096, np.float32))
+    seq = np.zeros(64, np.float32)
+    for i in range(4096):
+        seq = (seq + X[:, i] * X[:, i]).astype(np.float32)
+    naive = np.sqrt((seq / np.float32(4096)).astype(np.float32) + np.float32(1e-6)).astype(np.float32)
+    assert (naive != rms).any()
+    assert np.allclose(naive, rms, rtol=1e-5)
+
+
+@pytest.mark.parametrize("name,kw", [("c1_tiny_f32", {}), ("c4_finegrained", dict(T=48, d=64, H=32, E=8, K=3, Es=2, dtype="f32")),
+                                     ("c2_mixtral", dict(T=40, d=64, H=64))])
+def test_block_is_layer_on_normalised_rows_plus_residual(name, kw):
+    cfg = scaled(C.CONFIGS[name], **kw)
+    inp = make_inputs(cfg, 31)
+    bf = cfg.dtype == "bf16"
+    gamma = O.fill_normal(cfg.d, 31, C.STREAM_NORM, 1.0) * np.float32(0.1) + np.float32(1.0)
+    blk = O.block_forward(inp["x"], gamma, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm,
+                          cfg.Es, bf)
+    h, rms = O.rmsnorm(inp["x"], gamma, bf)
+    assert np.array_equal(blk["h"], h) and np.array_equal(blk["rms"], rms)
+    lay = O.moe_forward(h, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es, bf)
+    for k in ("ids", "w", "counts", "offsets", "dst", "src_row", "logits", "p"):
+        assert np.array_equal(blk[k], lay[k]), k
+    if not bf:  # fp32: the layer output is the unrounded sum, so the residual identity is exact
+        assert np.array_equal(blk["out"], (lay["out"] + inp["x"]).astype(np.float32))
+    else:       # bf16: one rounding of (sum + x) against rounding the sum first
+        assert N.rel_l2(blk["out"], lay["out"].astype(np.float64) + inp["x"]) < 1e-2
+    tok = np.array([0, 5, cfg.T - 1], np.int32)
+    sub = O.block_tokens(inp["x"], h, blk["ids"], blk["w"], inp["W1"], inp["W3"], inp["W2"], cfg.E, cfg.Es, tok, bf)
+    assert np.array_equal(sub, blk["out"][tok])
