@@ -304,6 +304,12 @@ class MoELayer:
                 raise RuntimeError("Error code 1:checkpoint ends early")
             self._upload(which, g, np.frombuffer(buf, "<f4").reshape(shape))
 
+    def loadJson(self, weight_map, layer_index=0, scheme="omega", strict=True):
+        """Weights by name from a JSON export of a PyTorch state dict (see weights_json.py; the reference's
+        LagJsonReader + ModeLoaderlUtils.loadData route)."""
+        from . import weights_json
+        return weights_json.load_moe_weights(self, weight_map, layer_index, scheme, strict)
+
     def close(self):
         if self.output_buf is not None:
             self.output_buf.free()
