@@ -126,11 +126,21 @@ __device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, 
 // instead of their own, so the matrix cores of the next item start on data that travelled during this item's
 // epilogue.
 template <bool FUSED, int NBLK>
-__device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx, TileCtx &nx, const omega_tile_desc &dn,
-                                         const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa, const bf16_t *Wb, int &cur,
+__device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_in, TileCtx &nx, const omega_tile_desc &dn,
+                                         const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa, const bf16_t *Wb, int &cur_io,
                                          void *Cout, int N, int Kd, int wave, int lane)
 {
     constexpr int NB = NBLK > 0 ? NBLK : 1;
+    // the item's uniform fields and the ring position live in scalar registers for the whole item (the direct loads
+    // take their base address and LDS address from scalar operands)
+    TileCtx ctx = ctx_in;
+    ctx.A = uniform_ptr(ctx_in.A);
+    ctx.B0 = uniform_ptr(ctx_in.B0);
+    ctx.B1 = uniform_ptr(ctx_in.B1);
+    ctx.row0 = __builtin_amdgcn_readfirstlane(ctx_in.row0);
+    ctx.rows = __builtin_amdgcn_readfirstlane(ctx_in.rows);
+    ctx.n0 = __builtin_amdgcn_readfirstlane(ctx_in.n0);
+    int cur = __builtin_amdgcn_readfirstlane(cur_io);
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     const uint32_t lds_wave = lds0 + wave * 1024;
@@ -235,6 +245,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx,
     nx = make_ctx<FUSED>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
     for (; kt < KT; ++kt) K_STEP(true);
 #undef K_STEP
+    cur_io = cur;
 
     // ---- epilogue ----
     if (FUSED) {
@@ -273,6 +284,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx,
             for (int r = 0; r < 16; ++r) {
                 const int row = (2 * i + wm) * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
                 if (row >= ctx.rows) continue;
+                // (32 lanes x 4 bytes = one 128-byte line per store; 16-byte stores of a transposed accumulator layout
+                //  write 32-byte pieces of 32 different lines and were 8 % slower on short-K shapes)
                 float *out = (float *)Cout + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l32;
 #pragma unroll
                 for (int j = 0; j < 2; ++j) out[j * 32] = acc[i][j][r];

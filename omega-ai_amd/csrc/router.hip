@@ -16,8 +16,11 @@
 #include "common.h"
 
 #define TOK_TILE ROUTER_TOK_TILE
+#define ROUTER_EPT(EP) ((EP) >= 128 ? 4 : (EP) >= 32 ? 2 : 1)
 
-// Phase 1 for the tokens t0.. of one workgroup: acc[i] = logit of (token tg + i*TPP, expert e1), bias not yet added.
+// Phase 1 for the tokens t0.. of one workgroup: acc[x*NT + i] = logit of (token tg + i*TPP, expert e1 + x*EL), bias
+// not yet added.  A thread owns EPT experts (2 from 128 experts on: each x value read from LDS then feeds two sums,
+// which halves the LDS reads per multiply-add) and NT tokens.
 // EP: experts padded to a power of two; KC: k per staged chunk (larger for few experts, where one chunk in
 // flight per workgroup would otherwise leave the kernel waiting on memory latency).
 // XBF: x and Wg are stored as bf16 (else fp32).  FAST_IO: rows are 16-byte aligned and d is a multiple of KC, so
@@ -31,10 +34,12 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
                                             float (*xs)[KC + 4], float (*ws)[KC + 4],
                                             float (&acc)[TOK_TILE * EP / 256])
 {
-    constexpr int NT = TOK_TILE * EP / 256;  // tokens per thread
-    constexpr int TPP = 256 / EP;            // tokens per pass
+    constexpr int EPT = ROUTER_EPT(EP);           // experts per thread
+    constexpr int EL = EP / EPT;                  // threads across the experts
+    constexpr int NT = TOK_TILE * EL / 256;       // tokens per thread
+    constexpr int TPP = 256 / EL;                 // tokens per pass
     const int tid = threadIdx.x;
-    const int e1 = tid % EP, tg = tid / EP;
+    const int e1 = tid % EL, tg = tid / EL;
     // staging: every thread carries 8 consecutive k of one token and of WCH gate rows from global memory to LDS;
     // the next chunk is fetched into registers while the current one is being summed
     constexpr int XCH = KC / 64;
@@ -146,27 +151,33 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
         // FAST with a fused multiply-add (one rounding per step)
 #define ROUTER_K4(k4)                                                                  \
     do {                                                                               \
-        const float4 wv = *(const float4 *)&ws[e1][(k4) * 4];                          \
+        float4 wv[EPT];                                                                \
+        _Pragma("unroll") for (int x_ = 0; x_ < EPT; ++x_)                             \
+            wv[x_] = *(const float4 *)&ws[e1 + x_ * EL][(k4) * 4];                     \
         _Pragma("unroll") for (int i = 0; i < NT; ++i)                                 \
         {                                                                              \
             const float4 xv = *(const float4 *)&xs[tg + i * TPP][(k4) * 4];            \
-            if (EXACT) {                                                               \
-                float prod;                                                            \
-                prod = xv.x * wv.x; acc[i] = acc[i] + prod;                            \
-                prod = xv.y * wv.y; acc[i] = acc[i] + prod;                            \
-                prod = xv.z * wv.z; acc[i] = acc[i] + prod;                            \
-                prod = xv.w * wv.w; acc[i] = acc[i] + prod;                            \
-            } else {                                                                   \
-                acc[i] = fmaf(xv.x, wv.x, acc[i]);                                     \
-                acc[i] = fmaf(xv.y, wv.y, acc[i]);                                     \
-                acc[i] = fmaf(xv.z, wv.z, acc[i]);                                     \
-                acc[i] = fmaf(xv.w, wv.w, acc[i]);                                     \
+            _Pragma("unroll") for (int x_ = 0; x_ < EPT; ++x_)                         \
+            {                                                                          \
+                float &a_ = acc[x_ * NT + i];                                          \
+                if (EXACT) {                                                           \
+                    float prod;                                                        \
+                    prod = xv.x * wv[x_].x; a_ = a_ + prod;                            \
+                    prod = xv.y * wv[x_].y; a_ = a_ + prod;                            \
+                    prod = xv.z * wv[x_].z; a_ = a_ + prod;                            \
+                    prod = xv.w * wv[x_].w; a_ = a_ + prod;                            \
+                } else {                                                               \
+                    a_ = fmaf(xv.x, wv[x_].x, a_);                                     \
+                    a_ = fmaf(xv.y, wv[x_].y, a_);                                     \
+                    a_ = fmaf(xv.z, wv[x_].z, a_);                                     \
+                    a_ = fmaf(xv.w, wv[x_].w, a_);                                     \
+                }                                                                      \
             }                                                                          \
         }                                                                              \
     } while (0)
         if (FAST_IO || kend == KC) {
             // whole chunk: no exit test inside, so the LDS reads of later steps are issued ahead of the sums
-#pragma unroll(NT >= 8 ? 4 : 16)
+#pragma unroll(NT * EPT >= 8 ? 4 : 16)
             for (int k4 = 0; k4 < KC / 4; ++k4) ROUTER_K4(k4);
         } else {
             // last, partial chunk (zero-filled beyond d: a +0 product leaves every sum unchanged)
@@ -185,8 +196,9 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
                                                      float *__restrict__ wout, int32_t *__restrict__ tile_counts,
                                                      float *__restrict__ logits_out, float *__restrict__ probs_out)
 {
-    constexpr int NT = TOK_TILE * EP / 256;  // tokens per thread in phase 1
-    constexpr int TPP = 256 / EP;            // tokens per pass
+    constexpr int EPT = ROUTER_EPT(EP), EL = EP / EPT;  // phase 1: experts per thread, threads across the experts
+    constexpr int NT = TOK_TILE * EL / 256;             // tokens per thread in phase 1
+    constexpr int TPP = 256 / EL;                       // tokens per pass
     constexpr int GS = EP < 64 ? EP : 64;    // lanes that share one token in phase 2
     constexpr int VPL = EP / GS;             // experts per lane in phase 2
     constexpr int LDW = KC + 4;  // LDS row stride in floats: rows stay 16-byte aligned and bank-staggered
@@ -198,12 +210,12 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
     const int tid = threadIdx.x;
     const int tile = blockIdx.x;
     const int t0 = tile * TOK_TILE;
-    const int e1 = tid % EP, tg = tid / EP;
+    const int e1 = tid % EL, tg = tid / EL;
     if (tid < EP) hist[tid] = 0;
 
-    float acc[NT];
+    float acc[NT * EPT];
 #pragma unroll
-    for (int i = 0; i < NT; ++i) acc[i] = 0.0f;
+    for (int i = 0; i < NT * EPT; ++i) acc[i] = 0.0f;
 
     const bool fast_io = (d % KC == 0) && (((uintptr_t)x | (uintptr_t)Wg | (uintptr_t)gamma) % 16 == 0);
     if (dtype == OMEGA_DTYPE_BF16) {
@@ -213,14 +225,16 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
         if (fast_io) router_sums<EP, KC, EXACT, false, true, NORM>(x, Wg, T, d, E, t0, rms, gamma, xs, ws, acc);
         else router_sums<EP, KC, EXACT, false, false, NORM>(x, Wg, T, d, E, t0, rms, gamma, xs, ws, acc);
     }
-    {
-        const float b = (bg != nullptr && e1 < E) ? bg[e1] : 0.0f;
+#pragma unroll
+    for (int x_ = 0; x_ < EPT; ++x_) {
+        const int e = e1 + x_ * EL;
+        const float b = (bg != nullptr && e < E) ? bg[e] : 0.0f;
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
-            const float z = bg != nullptr ? acc[i] + b : acc[i];
-            lg[tg + i * TPP][e1] = z;
+            const float z = bg != nullptr ? acc[x_ * NT + i] + b : acc[x_ * NT + i];
+            lg[tg + i * TPP][e] = z;
             const int t = t0 + tg + i * TPP;
-            if (logits_out != nullptr && t < T && e1 < E) logits_out[(size_t)t * E + e1] = z;
+            if (logits_out != nullptr && t < T && e < E) logits_out[(size_t)t * E + e] = z;
         }
     }
     __syncthreads();
