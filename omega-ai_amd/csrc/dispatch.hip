@@ -261,23 +261,34 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
             for (int r = 0; r < nr; ++r) {
                 const int c = c_next;
                 c_next = (lane < 32 && r + 1 < nr) ? cost_s[(r + 1) * 32 + lane] : 0;
-                // place of the lane's entry by rising cost and of its workgroup by falling work; lanes that stand for
-                // no workgroup keep their own place
-                // keys are unique (ties go to the lower lane), so a place is a count of larger keys; lane o's key is
-                // broadcast through a scalar register
-                const int key = lane < wpx ? (work << 6) | (63 - lane) : -1;
-                int rank_w = 0;
+                int ce, src;
+                // a round whose entries all cost the same (the common case: tiles of one expert after the even split)
+                // needs no dealing - it adds the same work to every queue: each workgroup takes the entry of its place
+                const unsigned long long act = __ballot(lane < wpx);
+                const int c0 = __builtin_amdgcn_readfirstlane(c);
+                if (__ballot(lane < wpx && c == c0) == act) {
+                    ce = c;
+                    src = lane;
+                } else {
+                    // place of the lane's entry by rising cost and of its workgroup by falling work; lanes that stand
+                    // for no workgroup keep their own place
+                    // keys are unique (ties go to the lower lane), so a place is a count of larger keys; lane o's key is
+                    // broadcast through a scalar register
+                    const int key = lane < wpx ? (work << 6) | (63 - lane) : -1;
+                    int rank_w = 0;
 #pragma unroll
-                for (int o = 0; o < 32; ++o) rank_w += __builtin_amdgcn_readlane(key, o) > key ? 1 : 0;
-                const int ckey = lane < wpx ? (c << 6) | lane : 0x7fffffff;
-                int rank_c = 0;
+                    for (int o = 0; o < 32; ++o) rank_w += __builtin_amdgcn_readlane(key, o) > key ? 1 : 0;
+                    const int ckey = lane < wpx ? (c << 6) | lane : 0x7fffffff;
+                    int rank_c = 0;
 #pragma unroll
-                for (int o = 0; o < 32; ++o) rank_c += __builtin_amdgcn_readlane(ckey, o) < ckey ? 1 : 0;
-                if (lane >= wpx) { rank_c = lane; rank_w = lane; }
-                // lane p receives the entry whose cost has place p, then every workgroup fetches the entry of its place
-                const int sorted = __builtin_amdgcn_ds_permute(rank_c << 2, (c << 8) | lane);
-                const int mine = __builtin_amdgcn_ds_bpermute(rank_w << 2, sorted);
-                const int ce = mine >> 8, src = mine & 31;
+                    for (int o = 0; o < 32; ++o) rank_c += __builtin_amdgcn_readlane(ckey, o) < ckey ? 1 : 0;
+                    if (lane >= wpx) { rank_c = lane; rank_w = lane; }
+                    // lane p receives the entry whose cost has place p, then every workgroup fetches the entry of its place
+                    const int sorted = __builtin_amdgcn_ds_permute(rank_c << 2, (c << 8) | lane);
+                    const int mine = __builtin_amdgcn_ds_bpermute(rank_w << 2, sorted);
+                    ce = mine >> 8;
+                    src = mine & 31;
+                }
                 if (lane < 32) {
                     unsigned short pl = 0;
                     if (lane < wpx && ce > 0) {
