@@ -96,7 +96,7 @@ def main():
     dispatch_bytes = 2 * cfg.P * cfg.d * b + cfg.P * 12
     combine_bytes = cfg.P * cfg.d * b + cfg.T * cfg.d * b + cfg.P * 8
     gather_ms = layer.time_stage(L.STAGE_GATHER, x, cfg.T, warmup=2, iters=20)
-    # block form (out = x + layer(rmsnorm(x)), the widening next to the path): whole call and its statistics kernel
+    # block form (out = x + layer(rmsnorm(x)), the widening next to the path): whole call and its pre-norm kernel
     outb = P.DeviceBuffer(ctx, (cfg.T, cfg.d), cfg.dtype)
     block_ms = layer.time_stage(L.STAGE_FORWARD_BLOCK, x, cfg.T, out=outb, warmup=2, iters=a.steps)
     rms_ms = layer.time_stage(L.STAGE_RMS, x, cfg.T, warmup=2, iters=20)
@@ -116,7 +116,7 @@ def main():
                      "algorithmic_flops_per_launch": up_flops, "avg_launch_ms": stage_ms["experts_up"],
                      "traffic": TRAFFIC_BYTES.get(cfg.name)},
         "block_form": {"what": "out = x + layer(rmsnorm(x)) in one call (omega_moe_forward_block)", "ms_per_step": block_ms,
-                       "tokens/s": cfg.T / (block_ms * 1e-3), "rms_stats_ms": rms_ms},
+                       "tokens/s": cfg.T / (block_ms * 1e-3), "prenorm_kernel_ms": rms_ms},
         "stages": {
             "avg_ms": stage_ms, "profiled_forwards": n_prof,
             "experts_down": {"TFLOP/s": down_tflops, "frac_mfma": down_tflops / peak},

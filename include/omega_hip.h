@@ -116,9 +116,10 @@ int omega_moe_forward(omega_moe *moe, const void *x_dev, int T, void *out_dev);
 
 /* Block form: out = x + layer(rmsnorm(x)), the second half of the transformer block,
  *   getNorm2().forward(tmp1); getMlp().forward(getNorm2().getOutput()); Tensor_OP().add(getMlp().getOutput(), tmp1, tmp2)
- * (J/engine/nn/layer/llama/LlamaTransformerBlock.java:134-136), in one call and without the two [T,d] round trips
- * through memory of the normalised rows and of the layer output: the row statistics are taken by a small kernel,
- * the router and the gather normalise the rows of x as they read them, the combine adds x back.
+ * (J/engine/nn/layer/llama/LlamaTransformerBlock.java:134-136), in one call: one kernel writes the row statistics
+ * and the normalised rows h (layer dtype) that the router and the gather then read, and the combine kernel adds the
+ * row of x to its fp32 sum before the one rounding of the output, so the layer output never makes a round trip
+ * through memory on its own.
  * rmsnorm = rmsnorm_forward_kernel2 (J/engine/nn/layer/normalization/gpu/RMSKernel.cu:185-223, the kernel
  * RMSLayer.output launches, RMSLayer.java:230): rms = sqrtf(mean(x^2) + 1e-6f), h = (x / rms) * gamma, with the
  * sum of squares taken lane by lane as that kernel takes it; bf16 layers round h to bf16 and round x + layer(h) once.
@@ -163,7 +164,7 @@ int omega_moe_get_workspace(omega_moe *moe, int which, int T, void *host_dst);
 /* Average duration in milliseconds of the launches of one stage, measured with events on the
  * context's stream: runs `iters` back-to-back repetitions of the stage (0 router, 1 dispatch,
  * 2 experts_up, 3 experts_down, 4 combine, 5 whole forward, 6 dispatch index kernels only, 7 dispatch
- * row gather only, 8 whole forward_block, 9 row statistics of the pre-norm only) after `warmup` untimed ones.
+ * row gather only, 8 whole forward_block, 9 the pre-norm kernel of the block form only) after `warmup` untimed ones.
  * x_dev/out_dev as for forward; the stages before `stage` must have been run for this T. */
 int omega_moe_time_stage(omega_moe *moe, int stage, const void *x_dev, int T, void *out_dev, int warmup, int iters,
                          float *ms_avg);

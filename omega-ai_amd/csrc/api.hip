@@ -155,10 +155,10 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 static void moe_free_workspace(omega_moe *m)
 {
     void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y,
-                    m->desc_up, m->desc_down, m->wq_up, m->wq_down, m->rms};
+                    m->desc_up, m->desc_down, m->wq_up, m->wq_down, m->rms, m->hbuf};
     for (void *p : ptrs)
         if (p) hipFree(p);
-    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr; m->rms = nullptr;
+    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr; m->rms = nullptr; m->hbuf = nullptr;
     m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
     m->T_cap = 0;
 }
@@ -192,6 +192,7 @@ static int moe_reserve(omega_moe *m, int T)
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->ids, P * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->w, P * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->rms, (size_t)T * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc(&m->hbuf, (size_t)T * c.d * m->esize));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_counts, (size_t)n_tok_tiles * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_base, (size_t)n_tok_tiles * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->dst, P * 4));
@@ -216,7 +217,7 @@ static int moe_reserve(omega_moe *m, int T)
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->wq_up, 0, q_up * m->n_wg * sizeof(omega_tile_desc), ctx->stream));
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->wq_down, 0, q_down * m->n_wg * sizeof(omega_tile_desc), ctx->stream));
     }
-    if (c.Es > 0) {  // rows the shared experts read: packed copy of x (bf16), normalised copy of x (fp32 block form)
+    if (c.dtype == OMEGA_DTYPE_BF16 && c.Es > 0) {
         const size_t xs_rows = (size_t)ceil_div(T, bm) * bm;
         OMEGA_HIP_CHECK(ctx, hipMalloc(&m->xs, xs_rows * c.d * m->esize));
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->xs, 0, xs_rows * c.d * m->esize, ctx->stream));
@@ -405,22 +406,19 @@ static int check_T(omega_moe *m, const void *x, int T, bool need_x)
     return OMEGA_OK;
 }
 
-// block != 0: block form, out = x + layer(rmsnorm(x)); the row statistics are taken first and the normalisation
-// is applied by the router and the gather to the rows they read
-static int stage_router(omega_moe *m, const void *x, int T, int block)
+static int stage_router(omega_moe *m, const void *x, int T)
 {
-    if (block) OMEGA_HIP_CHECK(m->ctx, launch_rms_stats(m, x, T, m->ctx->stream));
-    OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, nullptr, block, m->ctx->stream));
+    OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, nullptr, m->ctx->stream));
     return OMEGA_OK;
 }
-static int stage_dispatch(omega_moe *m, const void *x, int T, int block)
+static int stage_dispatch(omega_moe *m, const void *x, int T)
 {
     const int bm = moe_tile_m(m, T);
     m->bm = bm;
     m->max_m_tiles = moe_max_m_tiles(m, T, bm);
     if (m->max_m_tiles > m->tiles_cap) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: workspace too small for this T");
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));
-    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, block, m->ctx->stream));
+    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));
     return OMEGA_OK;
 }
 // x: the rows the shared experts read in fp32 layers (bf16 layers read the packed copy the gather left in xs)
@@ -456,9 +454,9 @@ static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block
     if (!out) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "forward: out is NULL");
     if (block && !m->gamma_set) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "forward_block: the norm weight (OMEGA_W_NORM) has not been set");
     RUN(moe_reserve(m, T));
-    // rows the shared experts of an fp32 layer read: x itself, or its normalised copy
-    const void *xsh = (block && m->cfg.dtype == OMEGA_DTYPE_F32 && m->cfg.Es > 0) ? m->xs : x;
+    // block form: the layer runs on the normalised rows h (one small kernel writes them and rms), the combine adds x back
     const void *resid = block ? x : nullptr;
+    const void *xin = block ? m->hbuf : x;
     if (m->profiling) {
         // six events bracket the five stages; durations are read back by omega_moe_get_profile
         if (m->prof_used + 6 > m->prof_events.size()) {
@@ -470,23 +468,25 @@ static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block
         }
         hipEvent_t *ev = &m->prof_events[m->prof_used];
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[0], ctx->stream));
-        RUN(stage_router(m, x, T, block));
+        if (block) OMEGA_HIP_CHECK(ctx, launch_rmsnorm(m, x, T, m->hbuf, ctx->stream));
+        RUN(stage_router(m, xin, T));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[1], ctx->stream));
-        RUN(stage_dispatch(m, x, T, block));
+        RUN(stage_dispatch(m, xin, T));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[2], ctx->stream));
-        RUN(stage_experts(m, xsh, T, 0));
+        RUN(stage_experts(m, xin, T, 0));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[3], ctx->stream));
-        RUN(stage_experts(m, xsh, T, 1));
+        RUN(stage_experts(m, xin, T, 1));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[4], ctx->stream));
         RUN(stage_combine(m, T, out, resid));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[5], ctx->stream));
         m->prof_used += 6;
         return OMEGA_OK;
     }
-    RUN(stage_router(m, x, T, block));
-    RUN(stage_dispatch(m, x, T, block));
-    RUN(stage_experts(m, xsh, T, 0));
-    RUN(stage_experts(m, xsh, T, 1));
+    if (block) OMEGA_HIP_CHECK(ctx, launch_rmsnorm(m, x, T, m->hbuf, ctx->stream));
+    RUN(stage_router(m, xin, T));
+    RUN(stage_dispatch(m, xin, T));
+    RUN(stage_experts(m, xin, T, 0));
+    RUN(stage_experts(m, xin, T, 1));
     RUN(stage_combine(m, T, out, resid));
     return OMEGA_OK;
 }
@@ -544,7 +544,7 @@ int omega_moe_router(omega_moe *m, const void *x, int T)
     RUN(check_T(m, x, T, true));
     if (T == 0) return OMEGA_OK;
     RUN(moe_reserve(m, T));
-    return stage_router(m, x, T, 0);
+    return stage_router(m, x, T);
 }
 
 int omega_moe_dispatch(omega_moe *m, const void *x, int T)
@@ -553,7 +553,7 @@ int omega_moe_dispatch(omega_moe *m, const void *x, int T)
     RUN(check_T(m, x, T, true));
     if (T == 0) return OMEGA_OK;
     if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "dispatch: router has not run for this T");
-    return stage_dispatch(m, x, T, 0);
+    return stage_dispatch(m, x, T);
 }
 
 int omega_moe_experts_up(omega_moe *m, const void *x, int T)
@@ -617,7 +617,7 @@ int omega_moe_get_router_probs(omega_moe *m, const void *x, int T, float *logits
     float *dl = nullptr, *dp = nullptr;
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&dl, n * 4));
     hipError_t e = hipMalloc((void **)&dp, n * 4);
-    if (e == hipSuccess) e = launch_router(m, x, T, dl, dp, 0, ctx->stream);
+    if (e == hipSuccess) e = launch_router(m, x, T, dl, dp, ctx->stream);
     if (e == hipSuccess && logits) e = hipMemcpyAsync(logits, dl, n * 4, hipMemcpyDeviceToHost, ctx->stream);
     if (e == hipSuccess && probs) e = hipMemcpyAsync(probs, dp, n * 4, hipMemcpyDeviceToHost, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -679,8 +679,8 @@ int omega_moe_time_stage(omega_moe *m, int stage, const void *x, int T, void *ou
     else if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: earlier stages have not run for this T");
     auto once = [&]() -> int {
         switch (stage) {
-            case 0: return stage_router(m, x, T, 0);
-            case 1: return stage_dispatch(m, x, T, 0);
+            case 0: return stage_router(m, x, T);
+            case 1: return stage_dispatch(m, x, T);
             case 2: return stage_experts(m, x, T, 0);
             case 3: return stage_experts(m, x, T, 1);
             case 4: return stage_combine(m, T, out, nullptr);
@@ -688,15 +688,15 @@ int omega_moe_time_stage(omega_moe *m, int stage, const void *x, int T, void *ou
                 OMEGA_HIP_CHECK(ctx, launch_dispatch_index(m, T, m->bm, ctx->stream));
                 return OMEGA_OK;
             case 7:
-                OMEGA_HIP_CHECK(ctx, launch_dispatch_gather(m, x, T, 0, ctx->stream));
+                OMEGA_HIP_CHECK(ctx, launch_dispatch_gather(m, x, T, ctx->stream));
                 return OMEGA_OK;
             case 8: return forward_impl(m, x, T, out, 1);
             case 9:
-                OMEGA_HIP_CHECK(ctx, launch_rms_stats(m, x, T, ctx->stream));
+                OMEGA_HIP_CHECK(ctx, launch_rmsnorm(m, x, T, m->hbuf, ctx->stream));
                 return OMEGA_OK;
             default:
-                RUN(stage_router(m, x, T, 0));
-                RUN(stage_dispatch(m, x, T, 0));
+                RUN(stage_router(m, x, T));
+                RUN(stage_dispatch(m, x, T));
                 RUN(stage_experts(m, x, T, 0));
                 RUN(stage_experts(m, x, T, 1));
                 return stage_combine(m, T, out, nullptr);

@@ -60,6 +60,7 @@ struct omega_moe {
     bool gamma_set = false;
     // workspace
     float *rms = nullptr;            // [T] row statistics of the pre-norm (block form)
+    void *hbuf = nullptr;            // [T,d] normalised rows (block form), layer dtype
     int32_t *ids = nullptr;          // [T,K]
     float *w = nullptr;              // [T,K]
     int32_t *tile_counts = nullptr;  // [n_tok_tiles,E] histogram per token tile (router)
@@ -112,12 +113,11 @@ hipError_t launch_fill_normal(void *dptr, uint64_t n, uint64_t seed, uint64_t st
                               int dtype, hipStream_t s);
 hipError_t launch_convert(void *dst, int dst_dtype, const void *src, int src_dtype, uint64_t n, hipStream_t s);
 
-// block != 0: the rows of x are normalised on the fly, h = (x / rms[t]) * gamma (rounded to bf16 in bf16 layers)
-hipError_t launch_rms_stats(const omega_moe *m, const void *x, int T, hipStream_t s);
-hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, int block,
-                         hipStream_t s);
+// h[t,:] = (x[t,:] / rms[t]) * gamma in the layer's storage type, rms[t] into m->rms; h == nullptr: statistics only
+hipError_t launch_rmsnorm(const omega_moe *m, const void *x, int T, void *h, hipStream_t s);
+hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s);
 hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s);
-hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, int block, hipStream_t s);
+hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipStream_t s);
 hipError_t launch_experts_f32(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
 hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
 // resid != nullptr: out = resid + layer output (one rounding of the fp32 sum)

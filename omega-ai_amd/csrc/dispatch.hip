@@ -329,13 +329,10 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
 // One wave per token; 16-byte chunks; up to 8 chunks in flight per lane.  PACKED: destination rows are in the
 // packed tile image (chunk index = 4*kstep + c); when xs != nullptr, the token is also copied to row t of xs.
 // The first n_sched workgroups build the product kernels' queues instead (see schedule_queues).
-// NORM (block form): the row is normalised on its way through the registers, h = (x / rms[t]) * gamma
-// (a 16-byte chunk is 8 bf16 columns in PACKED = bf16 layers, 4 fp32 columns otherwise).
-template <bool PACKED, bool NORM>
+template <bool PACKED>
 __global__ __launch_bounds__(256) void dispatch_gather_kernel(const uint4 *__restrict__ x, const int32_t *__restrict__ dstp,
                                                               int T, int K, int chunks_per_row,
                                                               unsigned char *__restrict__ xg, unsigned char *__restrict__ xs,
-                                                              const float *__restrict__ rms, const float *__restrict__ gamma,
                                                               int n_sched, sched_args sa)
 {
     if (PACKED && (int)blockIdx.x < n_sched) {
@@ -353,33 +350,6 @@ __global__ __launch_bounds__(256) void dispatch_gather_kernel(const uint4 *__res
         for (int u = 0; u < 8; ++u) {
             const int c = c0 + u * 64 + lane;
             v[u] = c < chunks_per_row ? src[c] : uint4{0u, 0u, 0u, 0u};  // always assigned: the array stays in registers
-        }
-        if (NORM) {
-            const float r = rms[t];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int c = c0 + u * 64 + lane;
-                if (c < chunks_per_row) {
-                    if (PACKED) {
-                        const float4 g0 = *(const float4 *)(gamma + c * 8), g1 = *(const float4 *)(gamma + c * 8 + 4);
-                        const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
-                        uint32_t w4[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const float lo = norm_apply<true>(__uint_as_float(w4[q] << 16), r, g[2 * q]);
-                            const float hi = norm_apply<true>(__uint_as_float(w4[q] & 0xffff0000u), r, g[2 * q + 1]);
-                            w4[q] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
-                        }
-                        v[u] = uint4{w4[0], w4[1], w4[2], w4[3]};
-                    } else {
-                        const float4 g0 = *(const float4 *)(gamma + c * 4);
-                        v[u].x = __float_as_uint(norm_apply<false>(__uint_as_float(v[u].x), r, g0.x));
-                        v[u].y = __float_as_uint(norm_apply<false>(__uint_as_float(v[u].y), r, g0.y));
-                        v[u].z = __float_as_uint(norm_apply<false>(__uint_as_float(v[u].z), r, g0.z));
-                        v[u].w = __float_as_uint(norm_apply<false>(__uint_as_float(v[u].w), r, g0.w));
-                    }
-                }
-            }
         }
         const int nd = K + (xs != nullptr ? 1 : 0);
         for (int j = 0; j < nd; ++j) {
@@ -409,22 +379,6 @@ __global__ __launch_bounds__(256) void dispatch_gather_bytes_kernel(const unsign
     }
 }
 
-// The same for normalised fp32 rows (block form).
-__global__ __launch_bounds__(256) void dispatch_gather_norm_f32_kernel(const float *__restrict__ x,
-                                                                       const int32_t *__restrict__ dstp, int T, int K, int d,
-                                                                       const float *__restrict__ rms,
-                                                                       const float *__restrict__ gamma, float *__restrict__ xg,
-                                                                       float *__restrict__ xs)
-{
-    const int t = blockIdx.x;
-    const float r = rms[t];
-    for (int c = threadIdx.x; c < d; c += 256) {
-        const float h = norm_apply<false>(x[(size_t)t * d + c], r, gamma[c]);
-        for (int j = 0; j < K; ++j) xg[(size_t)dstp[(size_t)t * K + j] * d + c] = h;
-        if (xs != nullptr) xs[(size_t)t * d + c] = h;
-    }
-}
-
 hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
@@ -439,33 +393,18 @@ hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t 
     return hipGetLastError();
 }
 
-hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, int block, hipStream_t s)
+hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
     const size_t row_bytes = (size_t)c.d * m->esize;
-    const float *rms = block ? m->rms : nullptr, *gamma = block ? m->gamma : nullptr;
     if (c.dtype == OMEGA_DTYPE_BF16) {  // d % 256 == 0 is guaranteed at creation: rows are whole 64-byte k steps
         sched_args sa = {m->desc_up, m->desc_down, m->wq_up, m->wq_down, m->tile_meta, c.E + c.Es, m->n_wg};
-        if (block)
-            hipLaunchKernelGGL((dispatch_gather_kernel<true, true>), dim3(ceil_div(T, 4) + SCHED_WGS), dim3(256), 0, s,
-                               (const uint4 *)x, m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg,
-                               (unsigned char *)m->xs, rms, gamma, SCHED_WGS, sa);
-        else
-            hipLaunchKernelGGL((dispatch_gather_kernel<true, false>), dim3(ceil_div(T, 4) + SCHED_WGS), dim3(256), 0, s,
-                               (const uint4 *)x, m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg,
-                               (unsigned char *)m->xs, rms, gamma, SCHED_WGS, sa);
+        hipLaunchKernelGGL(dispatch_gather_kernel<true>, dim3(ceil_div(T, 4) + SCHED_WGS), dim3(256), 0, s, (const uint4 *)x,
+                           m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs, SCHED_WGS, sa);
     } else if (row_bytes % 16 == 0 && ((uintptr_t)x % 16) == 0) {
-        if (block)
-            hipLaunchKernelGGL((dispatch_gather_kernel<false, true>), dim3(ceil_div(T, 4)), dim3(256), 0, s, (const uint4 *)x,
-                               m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs, rms,
-                               gamma, 0, sched_args{});
-        else
-            hipLaunchKernelGGL((dispatch_gather_kernel<false, false>), dim3(ceil_div(T, 4)), dim3(256), 0, s, (const uint4 *)x,
-                               m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)nullptr, rms,
-                               gamma, 0, sched_args{});
-    } else if (block) {
-        hipLaunchKernelGGL(dispatch_gather_norm_f32_kernel, dim3(T), dim3(256), 0, s, (const float *)x, m->dstp, T, c.K, c.d,
-                           rms, gamma, (float *)m->xg, (float *)m->xs);
+        hipLaunchKernelGGL(dispatch_gather_kernel<false>, dim3(ceil_div(T, 4)), dim3(256), 0, s, (const uint4 *)x,
+                           m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)nullptr, 0,
+                           sched_args{});
     } else {
         hipLaunchKernelGGL(dispatch_gather_bytes_kernel, dim3(T), dim3(256), 0, s, (const unsigned char *)x, m->dstp, T,
                            c.K, row_bytes, (unsigned char *)m->xg);

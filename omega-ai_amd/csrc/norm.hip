@@ -1,22 +1,26 @@
-// Row statistics of the RMSNorm in front of the layer (block form): rms[t] = sqrtf(sum_k x[t,k]^2 / d + 1e-6f),
+// RMSNorm in front of the layer (block form): rms[t] = sqrtf(sum_k x[t,k]^2 / d + 1e-6f), h[t,k] = (x[t,k] / rms[t]) * w[k],
 // with the sum taken exactly as rmsnorm_forward_kernel2 takes it
 // (J/engine/nn/layer/normalization/gpu/RMSKernel.cu:185-223): 32 lanes per row, lane l adds x[i]*x[i] for
 // i = l, l+32, ... in index order with one fused multiply-add per step, then an xor butterfly (16, 8, 4, 2, 1) over
-// the 32 partial sums.  The normalised row (x/rms)*weight is never written: the router and the gather apply it to
-// the rows they read anyway (norm_apply in common.h), and the combine adds x back.
+// the 32 partial sums.  h is written once, in the layer's storage type (rounded to bf16 in bf16 layers), and is what
+// the router and the gather read; the residual x is added back by the combine kernel.
 //
 // One workgroup = 8 rows x 32 lanes.  The rows come in with 16-byte loads, pass through LDS as fp32 and are read
 // back lane-strided (32 consecutive floats per row and step: no bank conflicts); chunks of NORM_DC columns keep the
-// order of every lane's additions (chunk boundaries are multiples of 32).
+// order of every lane's additions (chunk boundaries are multiples of 32).  The second pass re-reads the rows (they
+// are still in L2) and writes h with 16-byte stores.
 // This file is compiled with -ffp-contract=off; the only fused operation is the explicit fmaf.
 #include "common.h"
 
 #define NORM_ROWS 8
 #define NORM_DC 2048  // columns per staged chunk: 8 rows x 2048 x 4 B = 64 KiB of LDS
 
+// h == nullptr: statistics only
 template <bool XBF>
-__global__ __launch_bounds__(256) void rms_stats_kernel(const void *__restrict__ x, int T, int d, float *__restrict__ rms)
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const void *__restrict__ x, const float *__restrict__ gamma, int T,
+                                                      int d, float *__restrict__ rms, void *__restrict__ h)
 {
+    __shared__ float rms_s[NORM_ROWS];
     __shared__ __attribute__((aligned(16))) float xs[NORM_ROWS][NORM_DC];
     const int tid = threadIdx.x;
     const int r = tid >> 5, l = tid & 31;
@@ -70,16 +74,67 @@ __global__ __launch_bounds__(256) void rms_stats_kernel(const void *__restrict__
 #pragma unroll
     for (int m = 16; m >= 1; m >>= 1) s = s + __shfl_xor(s, m, 32);
     const int t = t0 + r;
-    if (l == 0 && t < T) rms[t] = sqrtf(s / (float)d + 1e-6f);
+    const float my = sqrtf(s / (float)d + 1e-6f);
+    if (l == 0) {
+        rms_s[r] = my;
+        if (t < T) rms[t] = my;
+    }
+    if (h == nullptr) return;
+    __syncthreads();
+    // second pass: 8 consecutive columns per thread and step
+    const int per_row = (d + 7) / 8;
+    for (int i = tid; i < NORM_ROWS * per_row; i += 256) {
+        const int rr = i / per_row, cc = (i % per_row) * 8;
+        const int tt = t0 + rr;
+        if (tt >= T) continue;
+        const float rv = rms_s[rr];
+        const size_t off = (size_t)tt * d + cc;
+        float v[8], g[8];
+        const bool full = vec_ok && ((uintptr_t)h % 16 == 0) && ((uintptr_t)gamma % 16 == 0) && cc + 8 <= d;
+        if (full) {
+            const float4 g0 = *(const float4 *)(gamma + cc), g1 = *(const float4 *)(gamma + cc + 4);
+            g[0] = g0.x; g[1] = g0.y; g[2] = g0.z; g[3] = g0.w; g[4] = g1.x; g[5] = g1.y; g[6] = g1.z; g[7] = g1.w;
+            if (XBF) {
+                const uint4 u = *(const uint4 *)((const bf16_t *)x + off);
+                v[0] = __uint_as_float(u.x << 16); v[1] = __uint_as_float(u.x & 0xffff0000u);
+                v[2] = __uint_as_float(u.y << 16); v[3] = __uint_as_float(u.y & 0xffff0000u);
+                v[4] = __uint_as_float(u.z << 16); v[5] = __uint_as_float(u.z & 0xffff0000u);
+                v[6] = __uint_as_float(u.w << 16); v[7] = __uint_as_float(u.w & 0xffff0000u);
+            } else {
+                const float4 a = *(const float4 *)((const float *)x + off), b = *(const float4 *)((const float *)x + off + 4);
+                v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) v[q] = norm_apply<XBF>(v[q], rv, g[q]);
+            if (XBF) {
+                uint4 o;
+                o.x = (__float_as_uint(v[0]) >> 16) | (__float_as_uint(v[1]) & 0xffff0000u);
+                o.y = (__float_as_uint(v[2]) >> 16) | (__float_as_uint(v[3]) & 0xffff0000u);
+                o.z = (__float_as_uint(v[4]) >> 16) | (__float_as_uint(v[5]) & 0xffff0000u);
+                o.w = (__float_as_uint(v[6]) >> 16) | (__float_as_uint(v[7]) & 0xffff0000u);
+                *(uint4 *)((bf16_t *)h + off) = o;
+            } else {
+                *(float4 *)((float *)h + off) = make_float4(v[0], v[1], v[2], v[3]);
+                *(float4 *)((float *)h + off + 4) = make_float4(v[4], v[5], v[6], v[7]);
+            }
+        } else {
+            for (int q = 0; q < 8 && cc + q < d; ++q) {
+                const float xv = XBF ? bf16_to_f32(((const bf16_t *)x)[off + q]) : ((const float *)x)[off + q];
+                const float hv = norm_apply<XBF>(xv, rv, gamma[cc + q]);
+                if (XBF) ((bf16_t *)h)[off + q] = f32_to_bf16(hv);
+                else ((float *)h)[off + q] = hv;
+            }
+        }
+    }
 }
 
-hipError_t launch_rms_stats(const omega_moe *m, const void *x, int T, hipStream_t s)
+hipError_t launch_rmsnorm(const omega_moe *m, const void *x, int T, void *h, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
     const int grid = ceil_div(T, NORM_ROWS);
     if (c.dtype == OMEGA_DTYPE_BF16)
-        hipLaunchKernelGGL(rms_stats_kernel<true>, dim3(grid), dim3(256), 0, s, x, T, c.d, m->rms);
+        hipLaunchKernelGGL(rmsnorm_kernel<true>, dim3(grid), dim3(256), 0, s, x, m->gamma, T, c.d, m->rms, h);
     else
-        hipLaunchKernelGGL(rms_stats_kernel<false>, dim3(grid), dim3(256), 0, s, x, T, c.d, m->rms);
+        hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(grid), dim3(256), 0, s, x, m->gamma, T, c.d, m->rms, h);
     return hipGetLastError();
 }

@@ -27,11 +27,9 @@
 // every load is a whole 16-byte vector; rows beyond T or E are redirected to the last valid row (their sums are
 // never used), which keeps the loads free of branches - and with that really asynchronous: a load issued inside
 // a divergent branch makes the compiler wait for all earlier ones first.
-// NORM: the rows of x are normalised while they are staged, h = (x / rms[t]) * gamma[k] (block form).
-template <int EP, int KC, bool EXACT, bool XBF, bool FAST_IO, bool NORM>
+template <int EP, int KC, bool EXACT, bool XBF, bool FAST_IO>
 __device__ __forceinline__ void router_sums(const void *__restrict__ x, const void *__restrict__ Wg, int T, int d, int E,
-                                            int t0, const float *__restrict__ rms, const float *__restrict__ gamma,
-                                            float (*xs)[KC + 4], float (*ws)[KC + 4],
+                                            int t0, float (*xs)[KC + 4], float (*ws)[KC + 4],
                                             float (&acc)[TOK_TILE * EP / 256])
 {
     constexpr int EPT = ROUTER_EPT(EP);           // experts per thread
@@ -49,8 +47,6 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
     // raw staging registers: 8 k of bf16 = one uint4, 8 k of fp32 = two; conversion happens when they are
     // written to LDS, so the global loads stay in flight during the sums of the current chunk
     uint4 xr[XCH][2], wr[WCH][2];
-    float4 gr[NORM ? XCH : 1][2];  // gamma of the staged columns
-    const float my_rms = NORM ? rms[min(t0 + x_tt, T - 1)] : 1.0f;
     auto load8 = [&](const void *base, int row, int rows, int k, uint4 *out) {
         out[0] = make_uint4(0, 0, 0, 0);
         out[1] = make_uint4(0, 0, 0, 0);
@@ -97,22 +93,6 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
     auto fetch = [&](int k0) {
 #pragma unroll
         for (int c = 0; c < XCH; ++c) load8(x, t0 + x_tt, T, k0 + x_ks + 64 * c, xr[c]);
-        if (NORM) {
-#pragma unroll
-            for (int c = 0; c < XCH; ++c) {
-                const int k = k0 + x_ks + 64 * c;
-                if (FAST_IO) {
-                    gr[c][0] = *(const float4 *)(gamma + k);
-                    gr[c][1] = *(const float4 *)(gamma + k + 4);
-                } else {
-                    float g[8];
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) g[q] = k + q < d ? gamma[k + q] : 0.0f;
-                    gr[c][0] = make_float4(g[0], g[1], g[2], g[3]);
-                    gr[c][1] = make_float4(g[4], g[5], g[6], g[7]);
-                }
-            }
-        }
 #pragma unroll
         for (int c = 0; c < WCH; ++c) {
             const int idx = tid + c * 256;
@@ -121,19 +101,7 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
     };
     auto stash = [&]() {
 #pragma unroll
-        for (int c = 0; c < XCH; ++c) {
-            float *dst = &xs[x_tt][x_ks + 64 * c];
-            widen(xr[c], dst);
-            if (NORM) {
-                float4 lo = *(float4 *)dst, hi = *(float4 *)(dst + 4);
-                lo.x = norm_apply<XBF>(lo.x, my_rms, gr[c][0].x); lo.y = norm_apply<XBF>(lo.y, my_rms, gr[c][0].y);
-                lo.z = norm_apply<XBF>(lo.z, my_rms, gr[c][0].z); lo.w = norm_apply<XBF>(lo.w, my_rms, gr[c][0].w);
-                hi.x = norm_apply<XBF>(hi.x, my_rms, gr[c][1].x); hi.y = norm_apply<XBF>(hi.y, my_rms, gr[c][1].y);
-                hi.z = norm_apply<XBF>(hi.z, my_rms, gr[c][1].z); hi.w = norm_apply<XBF>(hi.w, my_rms, gr[c][1].w);
-                *(float4 *)dst = lo;
-                *(float4 *)(dst + 4) = hi;
-            }
-        }
+        for (int c = 0; c < XCH; ++c) widen(xr[c], &xs[x_tt][x_ks + 64 * c]);
 #pragma unroll
         for (int c = 0; c < WCH; ++c) {
             const int idx = tid + c * 256;
@@ -188,10 +156,9 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
     }
 }
 
-template <int EP, int KC, bool EXACT, bool NORM>
+template <int EP, int KC, bool EXACT>
 __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
-                                                     const float *__restrict__ bg, const float *__restrict__ rms,
-                                                     const float *__restrict__ gamma, int T, int d, int E, int K,
+                                                     const float *__restrict__ bg, int T, int d, int E, int K,
                                                      int renorm, int32_t *__restrict__ ids,
                                                      float *__restrict__ wout, int32_t *__restrict__ tile_counts,
                                                      float *__restrict__ logits_out, float *__restrict__ probs_out)
@@ -217,13 +184,13 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
 #pragma unroll
     for (int i = 0; i < NT * EPT; ++i) acc[i] = 0.0f;
 
-    const bool fast_io = (d % KC == 0) && (((uintptr_t)x | (uintptr_t)Wg | (uintptr_t)gamma) % 16 == 0);
+    const bool fast_io = (d % KC == 0) && (((uintptr_t)x | (uintptr_t)Wg) % 16 == 0);
     if (dtype == OMEGA_DTYPE_BF16) {
-        if (fast_io) router_sums<EP, KC, EXACT, true, true, NORM>(x, Wg, T, d, E, t0, rms, gamma, xs, ws, acc);
-        else router_sums<EP, KC, EXACT, true, false, NORM>(x, Wg, T, d, E, t0, rms, gamma, xs, ws, acc);
+        if (fast_io) router_sums<EP, KC, EXACT, true, true>(x, Wg, T, d, E, t0, xs, ws, acc);
+        else router_sums<EP, KC, EXACT, true, false>(x, Wg, T, d, E, t0, xs, ws, acc);
     } else {
-        if (fast_io) router_sums<EP, KC, EXACT, false, true, NORM>(x, Wg, T, d, E, t0, rms, gamma, xs, ws, acc);
-        else router_sums<EP, KC, EXACT, false, false, NORM>(x, Wg, T, d, E, t0, rms, gamma, xs, ws, acc);
+        if (fast_io) router_sums<EP, KC, EXACT, false, true>(x, Wg, T, d, E, t0, xs, ws, acc);
+        else router_sums<EP, KC, EXACT, false, false>(x, Wg, T, d, E, t0, xs, ws, acc);
     }
 #pragma unroll
     for (int x_ = 0; x_ < EPT; ++x_) {
@@ -311,23 +278,21 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
     for (int e = tid; e < E; e += 256) tile_counts[(size_t)tile * E + e] = hist[e];
 }
 
-hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, int block,
-                         hipStream_t s)
+hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
     const int tiles = ceil_div(T, TOK_TILE);
     const int exact = c.router_mode == OMEGA_ROUTER_EXACT;
     const float *bg = c.has_gate_bias ? m->bg : nullptr;
-#define ROUTER_LAUNCH2(EPV, KCV, EX, NM)                                                                              \
-    hipLaunchKernelGGL((router_kernel<EPV, KCV, EX, NM>), dim3(tiles), dim3(256), 0, s, x, c.dtype, m->Wg, bg,        \
-                       NM ? m->rms : nullptr, NM ? m->gamma : nullptr, T, c.d, c.E, c.K, c.renorm, m->ids, m->w,      \
-                       m->tile_counts, logits_out, probs_out)
-#define ROUTER_LAUNCH(EPV, KCV)                                        \
-    do {                                                               \
-        if (exact && block) ROUTER_LAUNCH2(EPV, KCV, true, true);      \
-        else if (exact) ROUTER_LAUNCH2(EPV, KCV, true, false);         \
-        else if (block) ROUTER_LAUNCH2(EPV, KCV, false, true);         \
-        else ROUTER_LAUNCH2(EPV, KCV, false, false);                   \
+#define ROUTER_LAUNCH(EPV, KCV)                                                                                    \
+    do {                                                                                                           \
+        if (exact)                                                                                                 \
+            hipLaunchKernelGGL((router_kernel<EPV, KCV, true>), dim3(tiles), dim3(256), 0, s, x, c.dtype, m->Wg, bg, \
+                               T, c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out, probs_out);   \
+        else                                                                                                       \
+            hipLaunchKernelGGL((router_kernel<EPV, KCV, false>), dim3(tiles), dim3(256), 0, s, x, c.dtype, m->Wg,    \
+                               bg, T, c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out,           \
+                               probs_out);                                                                         \
     } while (0)
     if (c.E <= 8) ROUTER_LAUNCH(8, 256);
     else if (c.E <= 16) ROUTER_LAUNCH(16, 256);
@@ -336,6 +301,5 @@ hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits
     else if (c.E <= 128) ROUTER_LAUNCH(128, 64);
     else ROUTER_LAUNCH(256, 64);
 #undef ROUTER_LAUNCH
-#undef ROUTER_LAUNCH2
     return hipGetLastError();
 }
