@@ -27,7 +27,7 @@ PEAK_HBM_GBPS = 8000.0
 
 # HBM traffic per launch of the dominant kernel from the committed rocprofv3 --pmc runs
 # (profiles/experts_bf16_c2_mixtral_pmc.txt): FETCH_SIZE + WRITE_SIZE in bytes, scaled by the copy-kernel factor.
-TRAFFIC_BYTES = {"c2_mixtral": 5.51e9}
+TRAFFIC_BYTES = {"c2_mixtral": 5.10e9}
 
 
 def main():
@@ -41,6 +41,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample duration")
+    ap.add_argument("--no-mfma-probe", action="store_true",
+                    help="skip the matrix-core ceiling probe (two runs of about 1 s with no memory traffic)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (convert_kernel fp32->fp32) three times, so that "
                          "FETCH_SIZE / WRITE_SIZE of a profiled run can be scaled by a kernel of known traffic")
@@ -103,6 +105,18 @@ def main():
     outb.free()
     index_ms = layer.time_stage(L.STAGE_INDEX, x, cfg.T, warmup=2, iters=20)
 
+    # what the matrix cores sustain on this device with nothing else going on: the nominal-clock rate with constant
+    # operands and the rate under the power cap with random bf16 operands (the realistic ceiling for a GEMM)
+    probe = None
+    if cfg.dtype == "bf16" and not a.no_mfma_probe:
+        import ctypes
+        v = ctypes.c_float()
+        probe = {}
+        for key, rnd in (("constant_operands_TFLOP/s", 0), ("random_operands_TFLOP/s", 1)):
+            ctx.check(ctx.lib.omega_hip_mfma_probe(ctx.handle, rnd, 400, ctypes.byref(v)))
+            probe[key] = v.value
+        probe["frac_of_random_operand_rate"] = up_tflops / probe["random_operands_TFLOP/s"]
+
     res = {
         "metric": "MoE-layer fwd tokens/s (Mixtral shape, bf16); MFMA util %; dispatch GB/s",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -114,7 +128,8 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "experts_bf16_kernel<up>: a = silu(xg W1^T) * (xg W3^T)",
                      "achieved": up_tflops, "peak": peak, "unit": "TFLOP/s", "frac": up_tflops / peak,
                      "algorithmic_flops_per_launch": up_flops, "avg_launch_ms": stage_ms["experts_up"],
-                     "traffic": TRAFFIC_BYTES.get(cfg.name)},
+                     "traffic": TRAFFIC_BYTES.get(cfg.name),
+                     "mfma_only_probe": probe},
         "block_form": {"what": "out = x + layer(rmsnorm(x)) in one call (omega_moe_forward_block)", "ms_per_step": block_ms,
                        "tokens/s": cfg.T / (block_ms * 1e-3), "prenorm_kernel_ms": rms_ms},
         "stages": {

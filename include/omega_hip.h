@@ -169,6 +169,12 @@ int omega_moe_get_workspace(omega_moe *moe, int which, int T, void *host_dst);
 int omega_moe_time_stage(omega_moe *moe, int stage, const void *x_dev, int T, void *out_dev, int warmup, int iters,
                          float *ms_avg);
 
+/* Measurement aid, no counterpart in the reference: the bf16 matrix-core rate the device sustains with no memory
+ * traffic at all (a loop of independent MFMAs on every SIMD, `launches` launches of about 2.5 ms, the first
+ * quarter untimed), in TFLOP/s.  random_operands != 0 feeds random bf16 values (realistic switching activity: the
+ * rate under the power cap), 0 feeds constants (the rate at the nominal clock). */
+int omega_hip_mfma_probe(omega_ctx *ctx, int random_operands, int launches, float *tflops);
+
 /* Per-stage timing of omega_moe_forward itself: while profiling is on, every forward records events
  * on the context's stream around its five stages (router, dispatch, experts_up, experts_down,
  * combine).  get_profile waits for the stream, returns the summed duration of each stage in

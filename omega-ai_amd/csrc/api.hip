@@ -667,6 +667,32 @@ int omega_moe_get_workspace(omega_moe *m, int which, int T, void *host_dst)
     return OMEGA_OK;
 }
 
+int omega_hip_mfma_probe(omega_ctx *ctx, int random_operands, int launches, float *tflops)
+{
+    CTX_ENTER(ctx);
+    if (!tflops || launches < 4) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "mfma_probe: bad argument");
+    float *scratch = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&scratch, 4));
+    hipError_t e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    double flop = 0.0;
+    const int warm = launches / 4;
+    if (e == hipSuccess) e = launch_mfma_probe(scratch, ctx->num_cus, random_operands, warm, ctx->stream, &flop);
+    if (e == hipSuccess) e = hipEventRecord(e0, ctx->stream);
+    if (e == hipSuccess) e = launch_mfma_probe(scratch, ctx->num_cus, random_operands, launches - warm, ctx->stream, &flop);
+    if (e == hipSuccess) e = hipEventRecord(e1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e0) hipEventDestroy(e0);
+    if (e1) hipEventDestroy(e1);
+    hipFree(scratch);
+    OMEGA_HIP_CHECK(ctx, e);
+    *tflops = (float)(flop * (launches - warm) / (ms * 1e-3) / 1e12);
+    return OMEGA_OK;
+}
+
 int omega_moe_time_stage(omega_moe *m, int stage, const void *x, int T, void *out, int warmup, int iters, float *ms_avg)
 {
     MOE_ENTER(m);

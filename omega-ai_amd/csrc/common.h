@@ -122,6 +122,8 @@ hipError_t launch_experts_f32(const omega_moe *m, const void *x, int T, int whic
 hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
 // resid != nullptr: out = resid + layer output (one rounding of the fp32 sum)
 hipError_t launch_combine(const omega_moe *m, int T, void *out, const void *resid, hipStream_t s);
+hipError_t launch_mfma_probe(float *scratch, int num_cus, int random_operands, int launches, hipStream_t s,
+                             double *flop_per_launch);
 hipError_t launch_pack_rows(void *dst_packed, const void *src_rowmajor, int R, int Kd, hipStream_t s);
 hipError_t launch_unpack_rows(void *dst_rowmajor, const void *src_packed, int R, int Kd, hipStream_t s);
 int experts_bf16_tile_m(const omega_moe *m, int T);
