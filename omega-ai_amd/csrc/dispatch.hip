@@ -143,14 +143,14 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     // its row tiles, instead of full tiles and a ragged last one: the same number of tiles and of MFMA blocks, but
     // tiles of one cost, so that the workgroups of an XCD, which share operand tiles through its L2, stay in step.
     // The compute units take 256 tiles at a time; when the
-    // last r = Nt mod 256 tiles would occupy at most half of them, each of those tiles is cut into S = 2 or 4
-    // slices of bm/S rows (adjacent entries, so that the slices of a tile run side by side on one XCD and share
+    // last r = Nt mod 256 tiles would occupy at most half of them, each of those tiles is cut into S = 256/r (2..4)
+    // slices of its 32-row blocks (adjacent entries, so that the slices of a tile run side by side on one XCD and share
     // the weight tile in its L2).  Group g is written by workgroup g (mod grid).
     if (desc_up != nullptr || desc_down != nullptr) {
         const int G = E + Es;
         if (tile == 0 && tid < 2) {
             const int Nt = mt_s[G] * (tid == 0 ? nt_up : nt_down), r = Nt % 256;
-            const int S = (r == 0 || r > 128) ? 1 : (r > 64 ? 2 : 4);
+            const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
             tile_meta[G + 2 + tid] = Nt - r + r * S;
         }
         for (int g = tile; g < G; g += gridDim.x) {
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
                 const int NT = pass == 0 ? nt_up : nt_down, ncols = pass == 0 ? ncols_up : ncols_down;
                 if (desc == nullptr) continue;
                 const int Nt = mt_s[G] * NT, r = Nt % 256;
-                const int S = (r == 0 || r > 128) ? 1 : (r > 64 ? 2 : 4);
+                const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
                 const int nblk = (rows + 31) >> 5;  // 32-row blocks of the group, dealt evenly to its Mg row tiles
                 for (int l = tid; l < Mg * NT; l += 256) {
                     const int mt = l % Mg, n = l / Mg;
@@ -178,11 +178,12 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
                         dsc.xrow0 = g < E ? -1 : tfirst;
                         desc[at] = dsc;
                     } else {
-                        const int slice = bm / S;
+                        const int tb = (trows + 31) >> 5;  // the tile's 32-row blocks, dealt evenly to the S slices
                         for (int sl = 0; sl < S; ++sl) {
-                            dsc.row0 = mt_s[g] * bm + tfirst + sl * slice;
-                            dsc.rows = max(0, min(slice, trows - sl * slice));  // 0: nothing to do
-                            dsc.xrow0 = g < E ? -1 : tfirst + sl * slice;
+                            const int sfirst = 32 * ((sl * tb) / S);
+                            dsc.row0 = mt_s[g] * bm + tfirst + sfirst;
+                            dsc.rows = max(0, min(32 * (((sl + 1) * tb) / S), trows) - sfirst);  // 0: nothing to do
+                            dsc.xrow0 = g < E ? -1 : tfirst + sfirst;
                             desc[Nt - r + (at - (Nt - r)) * S + sl] = dsc;
                         }
                     }
