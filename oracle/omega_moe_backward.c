@@ -1,0 +1,259 @@
+/*
+ * CPU oracle for the backward pass of the mixture-of-experts layer.  TEST INFRASTRUCTURE ONLY (see
+ * omega_moe_oracle.c): nothing in the shipped library links, loads or calls this file.
+ *
+ * The reference has no mixture-of-experts layer; the backward pass composes the backward steps of the primitives the
+ * forward pass is built from (paths relative to the reference checkout, J/ = src/main/java/com/omega/):
+ *   linear layer       diffW = delta^T . input (overwritten, beta = 0), diff = delta . W, diffB = column sums of delta
+ *                      (FullyLayer.diff, J/engine/nn/layer/FullyLayer.java:292-334)
+ *   SwiGLU wiring      w2 back; dh3 = d(a) * silu(h1); dh1 = silu'(h1) applied to d(a) * h3; input gradient =
+ *                      w1's + w3's (LlamaMLPLayer.diff, J/engine/nn/layer/llama/LlamaMLPLayer.java:139-158)
+ *   SiLU               diff = delta * s * (1 + x * (1 - s)), s = 1/(1+exp(-x))
+ *                      (silu_backward, J/engine/nn/layer/active/gpu/activeFunction.cu:182-190)
+ *   softmax            sum = sum_e out*delta; diff = (delta - sum) * out   (softmax_back, J/engine/gpu/SoftmaxKernel.cu:101-112)
+ * The routing (expert ids, dispatch permutation) is piecewise constant and carries no gradient; the gate weights get
+ * theirs through the combine weights: combine -> (renormalisation) -> selected probabilities -> softmax -> gate.
+ *
+ * bf16 mode (build-defined, the reference is fp32 only): x, dout and the weights arrive rounded; every sum is fp32;
+ * the row gradients that feed a matrix product are rounded to bf16 first (dy = w*dout, dh1, dh3), `a` as in the
+ * forward pass; dx is rounded once at the end; weight gradients stay fp32.
+ *
+ * Pinning status:
+ *   orc_moe_backward   torch float64 autograd of the dense formulation with the routing held fixed, and central
+ *                      finite differences of an independent float64 NumPy forward (pinned to tolerance; the
+ *                      summation order of the reference's cuBLAS products cannot be reproduced: bits "parity unpinned")
+ */
+#include <stdlib.h>
+
+#include "oracle_common.h"
+
+void orc_gate(const float *x, const float *Wg, const float *bg, int T, int d, int E, float *logits);
+void orc_softmax(const float *logits, int T, int E, float *p);
+void orc_topk(const float *p, int T, int E, int K, int renorm, int32_t *ids, float *w);
+void orc_dispatch(const int32_t *ids, int T, int K, int E, int32_t *counts, int32_t *offsets, int32_t *dst,
+                  int32_t *src_row);
+
+/* Backward of the SwiGLU expert g over `rows` rows.  xin: the rows' inputs (rows x d, row r at xin + r*d); dy: their
+ * output gradients (rows x d).  Writes dxin (rows x d) and OVERWRITES dW1,dW3 [H,d], dW2 [d,H] (zero when rows == 0).
+ * Scratch: 6*H floats. */
+static void expert_backward(const float *xin, const float *dy, int rows, const float *W1, const float *W3,
+                            const float *W2, int d, int H, int bf16_mode, float *dxin, float *dW1, float *dW3,
+                            float *dW2, float *scratch)
+{
+    float *h1 = scratch, *h3 = scratch + H, *a = scratch + 2 * H, *dh1 = scratch + 3 * H, *dh3 = scratch + 4 * H;
+    memset(dW1, 0, sizeof(float) * (size_t)H * d);
+    memset(dW3, 0, sizeof(float) * (size_t)H * d);
+    memset(dW2, 0, sizeof(float) * (size_t)H * d);
+    for (int r = 0; r < rows; ++r) {
+        const float *xr = xin + (size_t)r * d, *dyr = dy + (size_t)r * d;
+        for (int h = 0; h < H; ++h) {
+            const float *w1 = W1 + (size_t)h * d, *w3 = W3 + (size_t)h * d;
+            float a1 = 0.0f, a3 = 0.0f;
+            for (int k = 0; k < d; ++k) {
+                float p1 = xr[k] * w1[k];
+                a1 = a1 + p1;
+                float p3 = xr[k] * w3[k];
+                a3 = a3 + p3;
+            }
+            h1[h] = a1;
+            h3[h] = a3;
+            float av = silu_f(a1) * a3;
+            a[h] = bf16_mode ? bf16_round(av) : av;
+        }
+        /* w2 back: da = dy . W2 ; dW2 += dy^T a */
+        for (int h = 0; h < H; ++h) {
+            float da = 0.0f;
+            for (int c = 0; c < d; ++c) {
+                float pr = dyr[c] * W2[(size_t)c * H + h];
+                da = da + pr;
+            }
+            float sg = 1.0f / (1.0f + (float)exp(-(double)h1[h]));
+            float g3 = da * silu_f(h1[h]);
+            float tmp = da * h3[h];
+            float g1 = tmp * sg * (1.0f + h1[h] * (1.0f - sg));
+            dh3[h] = bf16_mode ? bf16_round(g3) : g3;
+            dh1[h] = bf16_mode ? bf16_round(g1) : g1;
+        }
+        for (int c = 0; c < d; ++c)
+            for (int h = 0; h < H; ++h) {
+                float pr = dyr[c] * a[h];
+                dW2[(size_t)c * H + h] = dW2[(size_t)c * H + h] + pr;
+            }
+        for (int h = 0; h < H; ++h)
+            for (int k = 0; k < d; ++k) {
+                float p1 = dh1[h] * xr[k];
+                dW1[(size_t)h * d + k] = dW1[(size_t)h * d + k] + p1;
+                float p3 = dh3[h] * xr[k];
+                dW3[(size_t)h * d + k] = dW3[(size_t)h * d + k] + p3;
+            }
+        for (int k = 0; k < d; ++k) {
+            float s1 = 0.0f, s3 = 0.0f;
+            for (int h = 0; h < H; ++h) {
+                float p1 = dh1[h] * W1[(size_t)h * d + k];
+                s1 = s1 + p1;
+                float p3 = dh3[h] * W3[(size_t)h * d + k];
+                s3 = s3 + p3;
+            }
+            dxin[(size_t)r * d + k] = s1 + s3;
+        }
+    }
+}
+
+/* Whole backward pass.  x, dout: [T,d]; weights as in orc_moe_forward (W1,W3: [E+Es,H,d], W2: [E+Es,d,H]).
+ * The forward quantities it needs are recomputed here.  Outputs (any may be NULL except dx): dx [T,d], dWg [E,d],
+ * dbg [E], dW1,dW3 [E+Es,H,d], dW2 [E+Es,d,H], dw [T,K] (gradient of the combine weights), dlogits [T,E]. */
+void orc_moe_backward(const float *x, const float *dout, const float *Wg, const float *bg, const float *W1,
+                      const float *W3, const float *W2, int T, int d, int E, int K, int H, int Es, int renorm,
+                      int bf16_mode, float *dx, float *dWg, float *dbg, float *dW1, float *dW3, float *dW2,
+                      float *dw_o, float *dlogits_o)
+{
+    const int P = T * K;
+    const size_t HD = (size_t)H * d;
+    float *logits = (float *)malloc(sizeof(float) * (size_t)T * E);
+    float *p = (float *)malloc(sizeof(float) * (size_t)T * E);
+    int32_t *ids = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
+    float *w = (float *)malloc(sizeof(float) * (size_t)P);
+    int32_t *counts = (int32_t *)malloc(sizeof(int32_t) * (size_t)E);
+    int32_t *offsets = (int32_t *)malloc(sizeof(int32_t) * (size_t)(E + 1));
+    int32_t *dst = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
+    int32_t *src_row = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
+    float *xg = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1) * d);
+    float *y = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1) * d);
+    float *dy = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1) * d);
+    float *dxg = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1) * d);
+    float *dxs = Es ? (float *)malloc(sizeof(float) * (size_t)Es * T * d) : NULL;
+    float *dw = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1));
+    float *dlog = (float *)malloc(sizeof(float) * (size_t)T * E);
+    float *scratch = (float *)malloc(sizeof(float) * (size_t)6 * H);
+    float *g1 = (float *)malloc(sizeof(float) * HD), *g3 = (float *)malloc(sizeof(float) * HD),
+          *g2 = (float *)malloc(sizeof(float) * HD);
+
+    /* forward quantities */
+    orc_gate(x, Wg, bg, T, d, E, logits);
+    orc_softmax(logits, T, E, p);
+    orc_topk(p, T, E, K, renorm, ids, w);
+    orc_dispatch(ids, T, K, E, counts, offsets, dst, src_row);
+    for (int r = 0; r < P; ++r) memcpy(xg + (size_t)r * d, x + (size_t)src_row[r] * d, sizeof(float) * (size_t)d);
+    {
+        /* y of the routed rows (needed for the gradient of the combine weights) */
+        float *a = scratch;
+        for (int e = 0; e < E; ++e)
+            for (int r = offsets[e]; r < offsets[e + 1]; ++r) {
+                const float *xr = xg + (size_t)r * d;
+                const float *w1b = W1 + (size_t)e * HD, *w3b = W3 + (size_t)e * HD, *w2b = W2 + (size_t)e * HD;
+                for (int h = 0; h < H; ++h) {
+                    float a1 = 0.0f, a3 = 0.0f;
+                    for (int k = 0; k < d; ++k) {
+                        float p1 = xr[k] * w1b[(size_t)h * d + k];
+                        a1 = a1 + p1;
+                        float p3 = xr[k] * w3b[(size_t)h * d + k];
+                        a3 = a3 + p3;
+                    }
+                    float av = silu_f(a1) * a3;
+                    a[h] = bf16_mode ? bf16_round(av) : av;
+                }
+                for (int c = 0; c < d; ++c) {
+                    float acc = 0.0f;
+                    for (int h = 0; h < H; ++h) {
+                        float pr = a[h] * w2b[(size_t)c * H + h];
+                        acc = acc + pr;
+                    }
+                    y[(size_t)r * d + c] = acc;
+                }
+            }
+    }
+
+    /* combine backward: dy[r,:] = w[t,j] * dout[t,:], dw[t,j] = dout[t,:] . y[r,:] */
+    for (int t = 0; t < T; ++t)
+        for (int j = 0; j < K; ++j) {
+            const int r = dst[(size_t)t * K + j];
+            const float wv = w[(size_t)t * K + j];
+            float acc = 0.0f;
+            for (int c = 0; c < d; ++c) {
+                float g = wv * dout[(size_t)t * d + c];
+                dy[(size_t)r * d + c] = bf16_mode ? bf16_round(g) : g;
+                float pr = dout[(size_t)t * d + c] * y[(size_t)r * d + c];
+                acc = acc + pr;
+            }
+            dw[(size_t)t * K + j] = acc;
+        }
+
+    /* experts */
+    for (int e = 0; e < E; ++e) {
+        expert_backward(xg + (size_t)offsets[e] * d, dy + (size_t)offsets[e] * d, counts[e], W1 + (size_t)e * HD,
+                        W3 + (size_t)e * HD, W2 + (size_t)e * HD, d, H, bf16_mode, dxg + (size_t)offsets[e] * d, g1,
+                        g3, g2, scratch);
+        if (dW1) memcpy(dW1 + (size_t)e * HD, g1, sizeof(float) * HD);
+        if (dW3) memcpy(dW3 + (size_t)e * HD, g3, sizeof(float) * HD);
+        if (dW2) memcpy(dW2 + (size_t)e * HD, g2, sizeof(float) * HD);
+    }
+    for (int s = 0; s < Es; ++s) {
+        const int g = E + s;
+        expert_backward(x, dout, T, W1 + (size_t)g * HD, W3 + (size_t)g * HD, W2 + (size_t)g * HD, d, H, bf16_mode,
+                        dxs + (size_t)s * T * d, g1, g3, g2, scratch);
+        if (dW1) memcpy(dW1 + (size_t)g * HD, g1, sizeof(float) * HD);
+        if (dW3) memcpy(dW3 + (size_t)g * HD, g3, sizeof(float) * HD);
+        if (dW2) memcpy(dW2 + (size_t)g * HD, g2, sizeof(float) * HD);
+    }
+
+    /* router: renormalisation, scatter to the selected experts, softmax, gate */
+    for (int t = 0; t < T; ++t) {
+        float *dl = dlog + (size_t)t * E;
+        const float *pr = p + (size_t)t * E;
+        for (int e = 0; e < E; ++e) dl[e] = 0.0f; /* holds dp first */
+        float S = 1.0f, dot = 0.0f;
+        if (renorm) {
+            S = 0.0f;
+            for (int j = 0; j < K; ++j) S += pr[ids[(size_t)t * K + j]];
+            for (int j = 0; j < K; ++j) {
+                float term = dw[(size_t)t * K + j] * w[(size_t)t * K + j];
+                dot = dot + term;
+            }
+        }
+        for (int j = 0; j < K; ++j) {
+            float g = dw[(size_t)t * K + j];
+            if (renorm) g = (g - dot) / S;
+            dl[ids[(size_t)t * K + j]] = g;
+        }
+        float sum = 0.0f;
+        for (int e = 0; e < E; ++e) sum += pr[e] * dl[e];
+        for (int e = 0; e < E; ++e) dl[e] = (dl[e] - sum) * pr[e];
+    }
+    if (dWg)
+        for (int e = 0; e < E; ++e)
+            for (int k = 0; k < d; ++k) {
+                float acc = 0.0f;
+                for (int t = 0; t < T; ++t) {
+                    float term = dlog[(size_t)t * E + e] * x[(size_t)t * d + k];
+                    acc = acc + term;
+                }
+                dWg[(size_t)e * d + k] = acc;
+            }
+    if (dbg)
+        for (int e = 0; e < E; ++e) {
+            float acc = 0.0f;
+            for (int t = 0; t < T; ++t) acc = acc + dlog[(size_t)t * E + e];
+            dbg[e] = acc;
+        }
+
+    /* input gradient: experts in slot order, shared experts, gate */
+    for (int t = 0; t < T; ++t)
+        for (int k = 0; k < d; ++k) {
+            float acc = 0.0f;
+            for (int j = 0; j < K; ++j) acc = acc + dxg[(size_t)dst[(size_t)t * K + j] * d + k];
+            for (int s = 0; s < Es; ++s) acc = acc + dxs[((size_t)s * T + t) * d + k];
+            float gsum = 0.0f;
+            for (int e = 0; e < E; ++e) {
+                float term = dlog[(size_t)t * E + e] * Wg[(size_t)e * d + k];
+                gsum = gsum + term;
+            }
+            acc = acc + gsum;
+            dx[(size_t)t * d + k] = bf16_mode ? bf16_round(acc) : acc;
+        }
+
+    if (dw_o) memcpy(dw_o, dw, sizeof(float) * (size_t)P);
+    if (dlogits_o) memcpy(dlogits_o, dlog, sizeof(float) * (size_t)T * E);
+    free(logits); free(p); free(ids); free(w); free(counts); free(offsets); free(dst); free(src_row);
+    free(xg); free(y); free(dy); free(dxg); free(dxs); free(dw); free(dlog); free(scratch);
+    free(g1); free(g3); free(g2);
+}

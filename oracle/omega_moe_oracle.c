@@ -33,6 +33,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include "oracle_common.h"
+
 /* ------------------------------------------------------------------------------------------
  * Seeded synthetic data: counter-based SplitMix64 + Box-Muller written with +,-,*,/,sqrt only,
  * so that C, NumPy and the device generator agree bit for bit.
@@ -119,17 +121,6 @@ void orc_fill_normal(float *out, uint64_t n, uint64_t seed, uint64_t stream, dou
 {
     uint64_t key = orc_stream_key(seed, stream);
     for (uint64_t j = 0; j < n; ++j) out[j] = normal_at(key, first + j, std);
-}
-
-/* Round-to-nearest-even fp32 -> bf16 -> fp32 (value stays in a float). */
-static float bf16_round(float v)
-{
-    uint32_t u;
-    memcpy(&u, &v, 4);
-    if ((u & 0x7fffffffu) > 0x7f800000u) { u |= 0x00400000u; u &= 0xffff0000u; }
-    else { u += 0x7fffu + ((u >> 16) & 1u); u &= 0xffff0000u; }
-    memcpy(&v, &u, 4);
-    return v;
 }
 
 void orc_round_bf16(float *buf, uint64_t n)
@@ -234,12 +225,6 @@ void orc_dispatch(const int32_t *ids, int T, int K, int E, int32_t *counts, int3
 void orc_gather(const float *x, const int32_t *src_row, int P, int d, float *xg)
 {
     for (int r = 0; r < P; ++r) memcpy(xg + (size_t)r * d, x + (size_t)src_row[r] * d, sizeof(float) * (size_t)d);
-}
-
-static float silu_f(float v)
-{
-    /* x / (1 + exp(-x)): J/engine/nn/layer/active/gpu/activeFunction.cu:172-179 */
-    return v / (1.0f + (float)exp(-(double)v));
 }
 
 /* S6 expert body for `rows` rows that all belong to one expert:

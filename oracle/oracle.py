@@ -48,6 +48,8 @@ def lib():
         L.orc_block_tokens.argtypes = [_f, _f, _i, _f, _f, _f, _f] + [C.c_int] * 6 + [_i, C.c_int, _f]
         L.orc_block_forward.argtypes = ([_f, _f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8
                                         + [_f, _f, _f, _f, _i, _f, _i, _i, _i, _i, _f])
+        L.orc_moe_backward.argtypes = ([_f, _f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8
+                                       + [_f, _f, C.c_void_p, _f, _f, _f, _f, _f])
         L.orc_cpu_baseline_forward.restype = C.c_double
         L.orc_cpu_baseline_forward.argtypes = [_f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8 + [_f]
         L.orc_cpu_sgemm_tn.argtypes = [C.c_int, C.c_int, C.c_int, _f, C.c_int, _f, C.c_int, _f, C.c_int, C.c_int]
@@ -171,6 +173,22 @@ def block_forward(x, gamma, Wg, bg, W1, W3, W2, K, renorm, Es=0, bf16=False):
     lib().orc_block_forward(x, np.ascontiguousarray(gamma, np.float32), Wg, _opt(bg), W1, W3, W2, T, d, E, K, H, Es,
                             int(renorm), int(bf16), r["h"], r["rms"], r["logits"], r["p"], r["ids"], r["w"],
                             r["counts"], r["offsets"], r["dst"], r["src_row"], r["out"])
+    return r
+
+
+def moe_backward(x, dout, Wg, bg, W1, W3, W2, K, renorm, Es=0, bf16=False):
+    """Backward of the whole layer for the output gradient dout [T,d]; the forward quantities are recomputed.
+    Returns dict(dx, dWg, dbg (None without bias), dW1, dW3, dW2, dw [T,K], dlogits [T,E])."""
+    T, d = x.shape
+    E = Wg.shape[0]
+    G, H = W1.shape[0], W1.shape[1]
+    r = dict(dx=np.empty((T, d), np.float32), dWg=np.empty((E, d), np.float32),
+             dbg=None if bg is None else np.empty(E, np.float32), dW1=np.empty((G, H, d), np.float32),
+             dW3=np.empty((G, H, d), np.float32), dW2=np.empty((G, d, H), np.float32),
+             dw=np.empty((T, K), np.float32), dlogits=np.empty((T, E), np.float32))
+    lib().orc_moe_backward(x, np.ascontiguousarray(dout, np.float32), Wg, _opt(bg), W1, W3, W2, T, d, E, K, H, Es,
+                           int(renorm), int(bf16), r["dx"], r["dWg"], _opt(r["dbg"]), r["dW1"], r["dW3"], r["dW2"],
+                           r["dw"], r["dlogits"])
     return r
 
 
