@@ -129,6 +129,29 @@ int omega_moe_forward_block(omega_moe *moe, const void *x_dev, int T, void *out_
  * themselves are visible as the gathered rows, omega_moe_get_workspace(moe, 0, ...). */
 int omega_moe_get_norm(omega_moe *moe, int T, float *rms_host);
 
+/* back(Tensor delta): gradients for the output gradient dout_dev [T,d] (layer dtype) of the omega_moe_forward call
+ * that ran last on this layer with the same x_dev and T (its routing and its activation buffers are reused; h1 and
+ * h3 are recomputed).  Writes the input gradient dx_dev [T,d] (layer dtype; Layer.diff) and OVERWRITES the layer's
+ * parameter gradients (diffW / diffB of every child linear layer: beta = 0 in FullyLayer.diff,
+ * J/engine/nn/layer/FullyLayer.java:292-334).  Composition: combine backward (gradient of the rows and of the
+ * combine weights) -> SwiGLU backward per expert as LlamaMLPLayer.diff
+ * (J/engine/nn/layer/llama/LlamaMLPLayer.java:139-158) with silu_backward
+ * (J/engine/nn/layer/active/gpu/activeFunction.cu:182-190) -> un-dispatch; combine weights -> renormalisation ->
+ * softmax_back (J/engine/gpu/SoftmaxKernel.cu:101-112) -> gate linear layer.  The expert ids and the permutation carry
+ * no gradient.  Asynchronous on the context's stream. */
+int omega_moe_backward(omega_moe *moe, const void *x_dev, const void *dout_dev, int T, void *dx_dev);
+/* One parameter gradient of the last omega_moe_backward, always fp32, in the layout of the weight it belongs to
+ * (which / expert as for omega_moe_set_weights; OMEGA_W_NORM has none).  Stands in for reading layer.diffW / diffB
+ * (LlamaMLPLayer.putParamterGrads, J/engine/nn/layer/llama/LlamaMLPLayer.java:285-295). */
+int omega_moe_get_grad(omega_moe *moe, int which, int expert, void *dst, int is_device);
+/* accGrad(scale): the first call after an update copies the gradients into the accumulators, later calls add
+ * scale * gradient (FullyLayer.accGrad, J/engine/nn/layer/FullyLayer.java:593-607). */
+int omega_moe_acc_grad(omega_moe *moe, float scale);
+/* update() of a layer without an updater: the accumulated gradients, if any, replace the gradients, then
+ * w -= lr * diffW, b -= lr * diffB, and the accumulators are cleared (FullyLayer.update,
+ * J/engine/nn/layer/FullyLayer.java:569-590).  The optimisers behind Updater are not part of this library. */
+int omega_moe_update(omega_moe *moe, float lr);
+
 /* The four stages of forward, callable one at a time (per-stage timing and tests); they use the
  * same kernels and workspace as omega_moe_forward and must be called in this order for one T:
  *   router   x -> ids, weights, per-tile expert histogram      (gate: FullyLayer.output, FullyLayer.java:218-243;

@@ -161,6 +161,56 @@ static void moe_free_workspace(omega_moe *m)
     m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr; m->rms = nullptr; m->hbuf = nullptr;
     m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
     m->T_cap = 0;
+    void *bw[] = {m->bw_probs, m->bw_dw, m->bw_dlogits, m->bw_dy, m->bw_h1, m->bw_h3, m->bw_dxg};
+    for (void *p : bw)
+        if (p) hipFree(p);
+    m->bw_probs = m->bw_dw = m->bw_dlogits = m->bw_dy = m->bw_h1 = m->bw_h3 = m->bw_dxg = nullptr;
+    m->bw_T_cap = 0;
+    m->bw_rows_cap = 0;
+    m->fwd_T = -1;
+}
+
+static size_t grad_block_floats(const omega_moe *m)
+{
+    const omega_moe_config &c = m->cfg;
+    return (size_t)c.E * c.d + (size_t)c.E + 3 * (size_t)m->G * c.H * c.d;
+}
+
+// Gradient buffers (once) and the workspace of the backward pass for the current forward workspace.
+static int moe_reserve_backward(omega_moe *m, int T)
+{
+    omega_ctx *ctx = m->ctx;
+    const omega_moe_config &c = m->cfg;
+    if (!m->dWg) {
+        float *blk = nullptr;
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&blk, grad_block_floats(m) * 4));
+        OMEGA_HIP_CHECK(ctx, hipMemsetAsync(blk, 0, grad_block_floats(m) * 4, ctx->stream));
+        const size_t per = (size_t)m->G * c.H * c.d;
+        m->dWg = blk;
+        m->dbg = m->dWg + (size_t)c.E * c.d;
+        m->dW1 = m->dbg + c.E;
+        m->dW3 = m->dW1 + per;
+        m->dW2 = m->dW3 + per;
+    }
+    if (m->bw_T_cap >= T && m->bw_rows_cap >= m->rows_cap) return OMEGA_OK;
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    void *bw[] = {m->bw_probs, m->bw_dw, m->bw_dlogits, m->bw_dy, m->bw_h1, m->bw_h3, m->bw_dxg};
+    for (void *p : bw)
+        if (p) hipFree(p);
+    m->bw_probs = m->bw_dw = m->bw_dlogits = m->bw_dy = m->bw_h1 = m->bw_h3 = m->bw_dxg = nullptr;
+    m->bw_T_cap = 0;
+    m->bw_rows_cap = 0;
+    const int Tc = m->T_cap;
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_probs, (size_t)Tc * c.E * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dw, (size_t)Tc * c.K * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dlogits, (size_t)Tc * c.E * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dy, m->rows_cap * c.d * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h1, m->rows_cap * c.H * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h3, m->rows_cap * c.H * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dxg, m->rows_cap * c.d * 4));
+    m->bw_T_cap = Tc;
+    m->bw_rows_cap = m->rows_cap;
+    return OMEGA_OK;
 }
 
 static int moe_tile_m(const omega_moe *m, int T)
@@ -310,6 +360,8 @@ int omega_moe_destroy(omega_moe *m)
     void *ptrs[] = {m->Wg, m->bg, m->W1, m->W3, m->W2, m->counts, m->offsets, m->tile_meta, m->gamma};
     for (void *p : ptrs)
         if (p) hipFree(p);
+    if (m->dWg) hipFree(m->dWg);
+    if (m->acc_grad) hipFree(m->acc_grad);
     hipEventDestroy(m->ev0);
     hipEventDestroy(m->ev1);
     for (hipEvent_t ev : m->prof_events) hipEventDestroy(ev);
@@ -457,6 +509,7 @@ static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block
     // block form: the layer runs on the normalised rows h (one small kernel writes them and rms), the combine adds x back
     const void *resid = block ? x : nullptr;
     const void *xin = block ? m->hbuf : x;
+    m->fwd_T = block ? -1 : T;
     if (m->profiling) {
         // six events bracket the five stages; durations are read back by omega_moe_get_profile
         if (m->prof_used + 6 > m->prof_events.size()) {
@@ -501,6 +554,81 @@ int omega_moe_forward_block(omega_moe *m, const void *x, int T, void *out)
 {
     MOE_ENTER(m);
     return forward_impl(m, x, T, out, 1);
+}
+
+int omega_moe_backward(omega_moe *m, const void *x, const void *dout, int T, void *dx)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, x, T, true));
+    if (m->cfg.dtype != OMEGA_DTYPE_F32) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "backward: fp32 layers only");
+    if (T != m->fwd_T) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "backward: no omega_moe_forward has run for this T");
+    if (T == 0) return OMEGA_OK;
+    if (!dout || !dx) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "backward: dout or dx is NULL");
+    RUN(moe_reserve_backward(m, T));
+    OMEGA_HIP_CHECK(ctx, launch_backward_f32(m, x, dout, T, dx, ctx->stream));
+    return OMEGA_OK;
+}
+
+static int grad_slot(omega_moe *m, int which, int expert, float **ptr, size_t *floats)
+{
+    const omega_moe_config &c = m->cfg;
+    const size_t per = (size_t)c.H * c.d;
+    switch (which) {
+        case OMEGA_W_GATE: *ptr = m->dWg; *floats = (size_t)c.E * c.d; return OMEGA_OK;
+        case OMEGA_W_GATE_BIAS: *ptr = m->dbg; *floats = (size_t)c.E; return OMEGA_OK;
+        case OMEGA_W_W1: case OMEGA_W_W3: case OMEGA_W_W2:
+            if (expert < 0 || expert >= m->G) return OMEGA_ERR_INVALID_ARG;
+            *ptr = (which == OMEGA_W_W1 ? m->dW1 : which == OMEGA_W_W3 ? m->dW3 : m->dW2) + per * (size_t)expert;
+            *floats = per;
+            return OMEGA_OK;
+        default: return OMEGA_ERR_INVALID_ARG;
+    }
+}
+
+int omega_moe_get_grad(omega_moe *m, int which, int expert, void *dst, int is_device)
+{
+    MOE_ENTER(m);
+    if (!m->dWg) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_grad: no backward has run");
+    float *p; size_t n;
+    if (!dst || grad_slot(m, which, expert, &p, &n) != OMEGA_OK)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_grad: bad kind, expert index or destination");
+    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(dst, p, n * 4, is_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    return OMEGA_OK;
+}
+
+int omega_moe_acc_grad(omega_moe *m, float scale)
+{
+    MOE_ENTER(m);
+    if (!m->dWg) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "acc_grad: no backward has run");
+    const size_t n = grad_block_floats(m);
+    if (!m->acc_grad) OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->acc_grad, n * 4));
+    if (!m->acc_valid) {
+        OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(m->acc_grad, m->dWg, n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        m->acc_valid = true;
+    } else {
+        OMEGA_HIP_CHECK(ctx, launch_axpy_f32(m->acc_grad, m->dWg, scale, n, ctx->stream));
+    }
+    return OMEGA_OK;
+}
+
+int omega_moe_update(omega_moe *m, float lr)
+{
+    MOE_ENTER(m);
+    if (m->cfg.dtype != OMEGA_DTYPE_F32) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "update: fp32 layers only");
+    if (!m->dWg) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "update: no backward has run");
+    const omega_moe_config &c = m->cfg;
+    if (m->acc_valid) {
+        OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(m->dWg, m->acc_grad, grad_block_floats(m) * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        m->acc_valid = false;
+    }
+    const size_t per = (size_t)m->G * c.H * c.d;
+    OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->Wg, m->dWg, -lr, (size_t)c.E * c.d, ctx->stream));
+    if (c.has_gate_bias) OMEGA_HIP_CHECK(ctx, launch_axpy_f32(m->bg, m->dbg, -lr, (size_t)c.E, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W1, m->dW1, -lr, per, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W3, m->dW3, -lr, per, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W2, m->dW2, -lr, per, ctx->stream));
+    return OMEGA_OK;
 }
 
 int omega_moe_get_norm(omega_moe *m, int T, float *rms_host)

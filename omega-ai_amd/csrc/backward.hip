@@ -1,0 +1,320 @@
+// Backward pass of the layer, fp32 layers: gradients of the input, the gate and every expert for an output gradient
+// dout [T,d], composed from the backward steps of the reference primitives the forward pass is built from:
+//   linear layer   diffW = delta^T . input (overwritten), diff = delta . W, diffB = column sums of delta
+//                  (FullyLayer.diff, J/engine/nn/layer/FullyLayer.java:292-334)
+//   SwiGLU wiring  w2 back; dh3 = d(a) * silu(h1); dh1 = silu'(h1) applied to d(a) * h3; input gradient = w1's + w3's
+//                  (LlamaMLPLayer.diff, J/engine/nn/layer/llama/LlamaMLPLayer.java:139-158)
+//   SiLU           diff = delta * s * (1 + x * (1 - s)), s = 1/(1+exp(-x))
+//                  (silu_backward, J/engine/nn/layer/active/gpu/activeFunction.cu:182-190)
+//   softmax        sum = sum_e out*delta; diff = (delta - sum) * out   (softmax_back, J/engine/gpu/SoftmaxKernel.cu:101-112)
+// The routing of the forward pass (ids, permutation, row tiles) is reused as it was left in the workspace, together
+// with the activations a and the expert outputs y; h1 and h3 are recomputed.  Expert rows keep their forward places:
+// dy, dh1, dh3 and dxg are indexed by the same physical rows as xg, a and y.
+//
+// Kernels (all plain LDS-tiled FMA code, the fp32 configuration is the parity case):
+//   bw_combine_kernel   dy[r,:] = w[t,j] * dout[t,:],  dw[t,j] = dout[t,:] . y[r,:]
+//   bw_rows_f32_kernel  row-tiled grouped products over the forward tile list (h1/h3, d(a) + SwiGLU backward, dxg)
+//   bw_wgrad_f32_kernel dW_g = A_g^T . B_g over the rows of group g
+//   bw_router_kernel    combine weights -> (renormalisation) -> selected probabilities -> softmax -> dlogits
+//   bw_dx_kernel        dx[t,:] = sum_j dxg[row(t,j),:] + shared rows + dlogits[t,:] . Wg
+#include "common.h"
+
+#define GBM 64
+#define GBN 64
+#define GBK 16
+
+__device__ __forceinline__ float block_sum_256(float v, float *red)
+{
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    const int wave = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// One workgroup per token.  Shared experts take dout rows directly (their combine weight is 1).
+__global__ __launch_bounds__(256) void bw_combine_kernel(const float *__restrict__ dout, const float *__restrict__ y,
+                                                         const int32_t *__restrict__ dstp, const float *__restrict__ w,
+                                                         int K, int d, float *__restrict__ dy, float *__restrict__ dw)
+{
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    const float *g = dout + (size_t)t * d;
+    for (int j = 0; j < K; ++j) {
+        const int r = dstp[(size_t)t * K + j];
+        const float wv = w[(size_t)t * K + j];
+        float part = 0.0f;
+        for (int c = threadIdx.x; c < d; c += 256) {
+            const float gv = g[c];
+            dy[(size_t)r * d + c] = wv * gv;
+            part = fmaf(gv, y[(size_t)r * d + c], part);
+        }
+        const float tot = block_sum_256(part, red);
+        if (threadIdx.x == 0) dw[(size_t)t * K + j] = tot;
+    }
+}
+
+// C[r, n] = sum_k A[r, k] * B_g(k, n) for the rows of one row tile (group g = the tile's expert).
+// BKN = false: B_g is [N, Kd] (k contiguous: "x W^T");  BKN = true: B_g is [Kd, N] (n contiguous: "delta W").
+// A rows: Atok + xrow0*Kd for a shared-expert tile when Atok is given, else Aphys + row0*Kd.
+// EPI 0: C1 = acc.  EPI 1: C1 += acc.  EPI 2: acc is d(a); with h1 = C1[r,n], h3 = C2[r,n] writes, in place,
+// C1 = dh1 = acc*h3 * s*(1 + h1*(1-s)) and C2 = dh3 = acc * h1*s, s = 1/(1+exp(-h1)).
+template <bool BKN, int EPI>
+__global__ __launch_bounds__(256) void bw_rows_f32_kernel(const float *__restrict__ Aphys, const float *__restrict__ Atok,
+                                                          const float *__restrict__ Bw, float *__restrict__ C1,
+                                                          float *__restrict__ C2, const omega_tile *__restrict__ tiles,
+                                                          const int32_t *__restrict__ tile_meta, int N, int Kd)
+{
+    const int mt = blockIdx.y;
+    if (mt >= tile_meta[0]) return;
+    const omega_tile tl = tiles[mt];
+    const int n0 = blockIdx.x * GBN;
+    const float *A = (Atok && tl.xrow0 >= 0) ? Atok + (size_t)tl.xrow0 * Kd : Aphys + (size_t)tl.row0 * Kd;
+    const float *B = Bw + (size_t)tl.g * N * Kd;
+
+    __shared__ float As[GBK][GBM + 4];
+    __shared__ float Bs[GBK][GBN + 4];
+    const int tid = threadIdx.x;
+    const int tx = tid % 16, ty = tid / 16;
+    float acc[4][4] = {};
+
+    for (int k0 = 0; k0 < Kd; k0 += GBK) {
+        for (int idx = tid; idx < GBM * GBK; idx += 256) {
+            const int r = idx / GBK, kk = idx % GBK;
+            const int k = k0 + kk;
+            As[kk][r] = (r < tl.rows && k < Kd) ? A[(size_t)r * Kd + k] : 0.0f;
+            if (!BKN) {
+                const int n = n0 + r;
+                Bs[kk][r] = (n < N && k < Kd) ? B[(size_t)n * Kd + k] : 0.0f;
+            }
+        }
+        if (BKN) {
+            for (int idx = tid; idx < GBN * GBK; idx += 256) {
+                const int kk = idx / GBN, nn = idx % GBN;
+                const int k = k0 + kk, n = n0 + nn;
+                Bs[kk][nn] = (n < N && k < Kd) ? B[(size_t)k * N + n] : 0.0f;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GBK; ++kk) {
+            float av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bv[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = ty * 4 + i;
+        if (r >= tl.rows) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            const size_t o = (size_t)(tl.row0 + r) * N + n;
+            if (EPI == 0) C1[o] = acc[i][j];
+            else if (EPI == 1) C1[o] = C1[o] + acc[i][j];
+            else {
+                const float h1 = C1[o], h3 = C2[o], da = acc[i][j];
+                const float sg = 1.0f / (1.0f + expf(-h1));
+                C2[o] = da * (h1 * sg);
+                C1[o] = (da * h3) * sg * (1.0f + h1 * (1.0f - sg));
+            }
+        }
+    }
+}
+
+// dW_g[m, n] = sum over the rows r of group g of A[r, m] * B[r, n]  (diffW = delta^T . input); always written, so a group
+// without rows gets zeros.  grid (ceil(N/64), ceil(M/64), groups).  Rows of group g: physical rows from
+// tile_meta[1+g]*bm, counts[g] of them for a routed expert, T for a shared one; a shared group reads token rows
+// 0..T-1 of Atok / Btok when those are given.  single_rows >= 0: one group, rows 0..single_rows-1 of Aphys / Bphys.
+__global__ __launch_bounds__(256) void bw_wgrad_f32_kernel(const float *__restrict__ Aphys, const float *__restrict__ Atok,
+                                                           const float *__restrict__ Bphys, const float *__restrict__ Btok,
+                                                           float *__restrict__ dW, const int32_t *__restrict__ tile_meta,
+                                                           const int32_t *__restrict__ counts, int E, int T, int bm,
+                                                           int M, int N, int single_rows)
+{
+    const int g = blockIdx.z;
+    int rows, row0;
+    if (single_rows >= 0) { rows = single_rows; row0 = 0; }
+    else { rows = g < E ? counts[g] : T; row0 = tile_meta[1 + g] * bm; }
+    const bool shared = single_rows < 0 && g >= E;
+    const float *A = (shared && Atok) ? Atok : Aphys + (size_t)row0 * M;
+    const float *B = (shared && Btok) ? Btok : Bphys + (size_t)row0 * N;
+    const int m0 = blockIdx.y * GBM, n0 = blockIdx.x * GBN;
+
+    __shared__ float As[GBK][GBM + 4];
+    __shared__ float Bs[GBK][GBN + 4];
+    const int tid = threadIdx.x;
+    const int tx = tid % 16, ty = tid / 16;
+    float acc[4][4] = {};
+    for (int r0 = 0; r0 < rows; r0 += GBK) {
+        for (int idx = tid; idx < GBK * GBM; idx += 256) {
+            const int rr = idx / GBM, cc = idx % GBM;
+            const int r = r0 + rr;
+            As[rr][cc] = (r < rows && m0 + cc < M) ? A[(size_t)r * M + m0 + cc] : 0.0f;
+            Bs[rr][cc] = (r < rows && n0 + cc < N) ? B[(size_t)r * N + n0 + cc] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GBK; ++kk) {
+            float av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bv[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+    float *out = dW + (size_t)g * M * N;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int mm = m0 + ty * 4 + i;
+        if (mm >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < N) out[(size_t)mm * N + n] = acc[i][j];
+        }
+    }
+}
+
+// One thread per token: dw -> gradient of the selected probabilities (through the renormalisation w = q / sum q when
+// enabled) -> softmax_back over the E experts.  Only the selected experts have a non-zero probability gradient, so
+// sum_e p_e*dp_e runs over the K slots.
+__global__ __launch_bounds__(256) void bw_router_kernel(const float *__restrict__ probs, const int32_t *__restrict__ ids,
+                                                        const float *__restrict__ w, const float *__restrict__ dw, int T,
+                                                        int E, int K, int renorm, float *__restrict__ dlogits)
+{
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= T) return;
+    const float *p = probs + (size_t)t * E;
+    const int32_t *id = ids + (size_t)t * K;
+    float S = 1.0f, dot = 0.0f;
+    if (renorm) {
+        S = 0.0f;
+        for (int j = 0; j < K; ++j) S += p[id[j]];
+        for (int j = 0; j < K; ++j) dot = fmaf(dw[(size_t)t * K + j], w[(size_t)t * K + j], dot);
+    }
+    float sum = 0.0f;
+    for (int j = 0; j < K; ++j) {
+        float g = dw[(size_t)t * K + j];
+        if (renorm) g = (g - dot) / S;
+        sum = fmaf(p[id[j]], g, sum);
+    }
+    float *dl = dlogits + (size_t)t * E;
+    for (int e = 0; e < E; ++e) dl[e] = (0.0f - sum) * p[e];
+    for (int j = 0; j < K; ++j) {
+        float g = dw[(size_t)t * K + j];
+        if (renorm) g = (g - dot) / S;
+        dl[id[j]] = (g - sum) * p[id[j]];
+    }
+}
+
+// dbg[e] = sum_t dlogits[t,e]: one workgroup per expert.
+__global__ __launch_bounds__(256) void bw_gate_bias_kernel(const float *__restrict__ dlogits, int T, int E,
+                                                           float *__restrict__ dbg)
+{
+    __shared__ float red[4];
+    const int e = blockIdx.x;
+    float part = 0.0f;
+    for (int t = threadIdx.x; t < T; t += 256) part += dlogits[(size_t)t * E + e];
+    const float tot = block_sum_256(part, red);
+    if (threadIdx.x == 0) dbg[e] = tot;
+}
+
+// One workgroup per token: dx[t,:] = sum_j dxg[row(t,j),:] (slot order) + shared-expert rows + dlogits[t,:] . Wg.
+__global__ __launch_bounds__(256) void bw_dx_kernel(const float *__restrict__ dxg, const int32_t *__restrict__ dstp,
+                                                    const float *__restrict__ dlogits, const float *__restrict__ Wg,
+                                                    const int32_t *__restrict__ tile_meta, int K, int d, int E, int Es,
+                                                    int bm, float *__restrict__ dx)
+{
+    const int t = blockIdx.x;
+    extern __shared__ float dl[];  // E floats
+    for (int e = threadIdx.x; e < E; e += 256) dl[e] = dlogits[(size_t)t * E + e];
+    __syncthreads();
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float acc = 0.0f;
+        for (int j = 0; j < K; ++j) acc += dxg[(size_t)dstp[(size_t)t * K + j] * d + c];
+        for (int s = 0; s < Es; ++s) acc += dxg[((size_t)tile_meta[1 + E + s] * bm + t) * d + c];
+        float gs = 0.0f;
+        for (int e = 0; e < E; ++e) gs = fmaf(dl[e], Wg[(size_t)e * d + c], gs);
+        dx[(size_t)t * d + c] = acc + gs;
+    }
+}
+
+// dst += scale * src (accGrad: axpy_gpu, J/engine/nn/layer/FullyLayer.java:593-607);  w -= lr * g (update without an updater,
+// FullyLayer.java:581-586)
+__global__ __launch_bounds__(256) void bw_axpy_kernel(float *__restrict__ dst, const float *__restrict__ src, float scale, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = fmaf(scale, src[i], dst[i]);
+}
+
+hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    const int grid = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    hipLaunchKernelGGL(bw_axpy_kernel, dim3(grid), dim3(256), 0, s, dst, src, scale, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_backward_f32(const omega_moe *m, const void *xv, const void *doutv, int T, void *dxv, hipStream_t s)
+{
+    const omega_moe_config &c = m->cfg;
+    const float *x = (const float *)xv, *dout = (const float *)doutv;
+    const float *xg = (const float *)m->xg, *a = (const float *)m->a;
+    const float *W1 = (const float *)m->W1, *W3 = (const float *)m->W3, *W2 = (const float *)m->W2;
+    const int G = m->G;
+    hipError_t e;
+    // probabilities of the forward pass (the router leaves ids and w as they are: same inputs, same arithmetic)
+    if ((e = launch_router(m, x, T, nullptr, m->bw_probs, s)) != hipSuccess) return e;
+    hipLaunchKernelGGL(bw_combine_kernel, dim3(T), dim3(256), 0, s, dout, m->y, m->dstp, m->w, c.K, c.d, m->bw_dy, m->bw_dw);
+    // h1, h3 (recomputed), then d(a) = dy . W2 with the SwiGLU backward in its epilogue: bw_h1 <- dh1, bw_h3 <- dh3
+    const dim3 gH(ceil_div(c.H, GBN), m->max_m_tiles), gD(ceil_div(c.d, GBN), m->max_m_tiles);
+    hipLaunchKernelGGL((bw_rows_f32_kernel<false, 0>), gH, dim3(256), 0, s, xg, x, W1, m->bw_h1, (float *)nullptr, m->tiles,
+                       m->tile_meta, c.H, c.d);
+    hipLaunchKernelGGL((bw_rows_f32_kernel<false, 0>), gH, dim3(256), 0, s, xg, x, W3, m->bw_h3, (float *)nullptr, m->tiles,
+                       m->tile_meta, c.H, c.d);
+    hipLaunchKernelGGL((bw_rows_f32_kernel<true, 2>), gH, dim3(256), 0, s, (const float *)m->bw_dy, dout, W2, m->bw_h1,
+                       m->bw_h3, m->tiles, m->tile_meta, c.H, c.d);
+    // dxg = dh1 . W1 + dh3 . W3
+    hipLaunchKernelGGL((bw_rows_f32_kernel<true, 0>), gD, dim3(256), 0, s, (const float *)m->bw_h1, (const float *)nullptr,
+                       W1, m->bw_dxg, (float *)nullptr, m->tiles, m->tile_meta, c.d, c.H);
+    hipLaunchKernelGGL((bw_rows_f32_kernel<true, 1>), gD, dim3(256), 0, s, (const float *)m->bw_h3, (const float *)nullptr,
+                       W3, m->bw_dxg, (float *)nullptr, m->tiles, m->tile_meta, c.d, c.H);
+    // weight gradients: dW2 = dy^T a [d,H]; dW1 = dh1^T xg, dW3 = dh3^T xg [H,d]
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.H, GBN), ceil_div(c.d, GBM), G), dim3(256), 0, s,
+                       (const float *)m->bw_dy, dout, a, (const float *)nullptr, m->dW2, m->tile_meta, m->counts, c.E, T,
+                       m->bm, c.d, c.H, -1);
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
+                       (const float *)m->bw_h1, (const float *)nullptr, xg, x, m->dW1, m->tile_meta, m->counts, c.E, T,
+                       m->bm, c.H, c.d, -1);
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
+                       (const float *)m->bw_h3, (const float *)nullptr, xg, x, m->dW3, m->tile_meta, m->counts, c.E, T,
+                       m->bm, c.H, c.d, -1);
+    // router and gate
+    hipLaunchKernelGGL(bw_router_kernel, dim3(ceil_div(T, 256)), dim3(256), 0, s, (const float *)m->bw_probs, m->ids, m->w,
+                       (const float *)m->bw_dw, T, c.E, c.K, c.renorm, m->bw_dlogits);
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.E, GBM), 1), dim3(256), 0, s,
+                       (const float *)m->bw_dlogits, (const float *)nullptr, x, (const float *)nullptr, m->dWg,
+                       m->tile_meta, m->counts, c.E, T, m->bm, c.E, c.d, T);
+    if (c.has_gate_bias)
+        hipLaunchKernelGGL(bw_gate_bias_kernel, dim3(c.E), dim3(256), 0, s, (const float *)m->bw_dlogits, T, c.E, m->dbg);
+    hipLaunchKernelGGL(bw_dx_kernel, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,
+                       (const float *)m->bw_dlogits, (const float *)m->Wg, m->tile_meta, c.K, c.d, c.E, c.Es, m->bm,
+                       (float *)dxv);
+    return hipGetLastError();
+}

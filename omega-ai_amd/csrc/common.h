@@ -86,6 +86,21 @@ struct omega_moe {
     size_t rows_cap = 0;             // physical rows the buffers hold: tile capacity * bm
     int tiles_cap = 0;               // entries of `tiles`
     int max_m_tiles = 0;
+    // backward pass (allocated by the first omega_moe_backward): parameter gradients, always fp32, in the layout of
+    // their weights, the accumulators of accGrad, and the workspace of the pass, indexed by physical rows like xg / a / y
+    float *dWg = nullptr, *dbg = nullptr, *dW1 = nullptr, *dW3 = nullptr, *dW2 = nullptr;
+    float *acc_grad = nullptr;       // accumulators, one block in the order dWg, dbg, dW1, dW3, dW2
+    bool acc_valid = false;          // accGrad has run since the last update
+    float *bw_probs = nullptr;       // [T,E] softmax of the gate logits
+    float *bw_dw = nullptr;          // [T,K] gradient of the combine weights
+    float *bw_dlogits = nullptr;     // [T,E]
+    float *bw_dy = nullptr;          // [rows_cap,d] gradient of the expert outputs
+    float *bw_h1 = nullptr;          // [rows_cap,H] h1, then dh1
+    float *bw_h3 = nullptr;          // [rows_cap,H] h3, then dh3
+    float *bw_dxg = nullptr;         // [rows_cap,d] gradient of the expert inputs
+    int bw_T_cap = 0;
+    size_t bw_rows_cap = 0;
+    int fwd_T = -1;                  // tokens of the last plain forward (what backward may follow), -1: none
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     // per-stage event profiling of forward calls (6 events per call), off by default
     bool profiling = false;
@@ -122,6 +137,8 @@ hipError_t launch_experts_f32(const omega_moe *m, const void *x, int T, int whic
 hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
 // resid != nullptr: out = resid + layer output (one rounding of the fp32 sum)
 hipError_t launch_combine(const omega_moe *m, int T, void *out, const void *resid, hipStream_t s);
+hipError_t launch_backward_f32(const omega_moe *m, const void *x, const void *dout, int T, void *dx, hipStream_t s);
+hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, hipStream_t s);
 hipError_t launch_mfma_probe(float *scratch, int num_cus, int random_operands, int launches, hipStream_t s,
                              double *flop_per_launch);
 hipError_t launch_pack_rows(void *dst_packed, const void *src_rowmajor, int R, int Kd, hipStream_t s);

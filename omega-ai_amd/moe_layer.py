@@ -99,7 +99,7 @@ class DeviceBuffer:
 
 
 class MoELayer:
-    """Mixture-of-experts FFN layer, forward only."""
+    """Mixture-of-experts FFN layer: forward, block form, backward and the plain update."""
 
     def __init__(self, embedDim, hidden, nExperts, topK, renorm=True, nShared=0, bias=False, ctx=None,
                  dtype="f32", router_mode="exact", T_max=0):
@@ -111,6 +111,8 @@ class MoELayer:
         self.number = 0
         self.input = None
         self.output_buf = None
+        self.diff = None
+        self.delta = None
         cfg = L.MoEConfigStruct(T_max, embedDim, nExperts, topK, hidden, nShared, int(renorm), int(bias),
                                 L.DTYPE_BF16 if dtype == "bf16" else L.DTYPE_F32,
                                 L.ROUTER_EXACT if router_mode == "exact" else L.ROUTER_FAST)
@@ -216,13 +218,43 @@ class MoELayer:
     def getLayerType(self):
         return "feed_forward"
 
-    def back(self, delta=None):
-        raise NotImplementedError("MoELayer is forward-only")
+    def initBack(self):
+        """(Re)allocates the input gradient when the batch size changes (FullyLayer.initBack,
+        J/engine/nn/layer/FullyLayer.java:130-144); the parameter gradients live in the native handle."""
+        if self.diff is None or self.diff.shape[0] != self.number:
+            if self.diff is not None:
+                self.diff.free()
+            self.diff = DeviceBuffer(self.ctx, (self.number, self.embedDim), self.dtype)
 
-    backTemp = diff = update = initBack = back
+    def back(self, delta):
+        """back(Tensor delta) = initBack -> setDelta -> diff (LlamaMLPLayer.back,
+        J/engine/nn/layer/llama/LlamaMLPLayer.java:186-199): input gradient returned, parameter gradients overwritten.
+        Must follow forward() of the same input."""
+        if self.input is None:
+            raise RuntimeError("Error code 1:back without a forward")
+        if tuple(delta.shape) != (self.number, self.embedDim):
+            raise RuntimeError("Error code 1:delta shape does not match the output")
+        self.initBack()
+        self.delta = delta
+        self.ctx.check(self.lib.omega_moe_backward(self.handle, self.input.ptr, delta.ptr, self.number, self.diff.ptr))
+        return self.diff
+
+    def grad(self, which, expert=0):
+        """Host copy of one parameter gradient (fp32), in the layout of its weight."""
+        shape = {L.W_GATE: (self.nExperts, self.embedDim), L.W_GATE_BIAS: (self.nExperts,),
+                 L.W_W1: (self.hidden, self.embedDim), L.W_W3: (self.hidden, self.embedDim),
+                 L.W_W2: (self.embedDim, self.hidden)}[which]
+        g = np.empty(shape, np.float32)
+        self.ctx.check(self.lib.omega_moe_get_grad(self.handle, which, expert, g.ctypes.data, 0))
+        return g
 
     def accGrad(self, scale):
-        raise NotImplementedError("MoELayer is forward-only")
+        self.ctx.check(self.lib.omega_moe_acc_grad(self.handle, float(scale)))
+
+    def update(self, learnRate):
+        """The update of a layer without an updater: w -= learnRate * diffW (FullyLayer.update,
+        J/engine/nn/layer/FullyLayer.java:569-590)."""
+        self.ctx.check(self.lib.omega_moe_update(self.handle, float(learnRate)))
 
     # ---- stages and introspection
     def stage(self, name, x=None, out=None):
@@ -314,6 +346,9 @@ class MoELayer:
         if self.output_buf is not None:
             self.output_buf.free()
             self.output_buf = None
+        if self.diff is not None:
+            self.diff.free()
+            self.diff = None
         if self.handle:
             self.lib.omega_moe_destroy(self.handle)
             self.handle = None

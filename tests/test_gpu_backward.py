@@ -1,0 +1,100 @@
+"""Backward pass through the C ABI against the backward oracle (which float64 autograd and finite differences pin):
+input gradient and every parameter gradient to 1e-5 (fp32) / 1e-2 (bf16) relative L2, plus accGrad / update."""
+import importlib
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from oracle import oracle_np as N
+from tests.synth import C, make_inputs, scaled
+
+pytestmark = pytest.mark.gpu
+L = importlib.import_module("omega-ai_amd._lib")
+
+
+def _setup(name, kw, seed):
+    from tests import gpu_util as G
+    cfg = scaled(C.CONFIGS[name], **kw)
+    inp = make_inputs(cfg, seed)
+    inp["Wg"] = inp["Wg"] * np.float32(8.0)   # spread the probabilities: a router gradient worth checking
+    dout = O.fill_normal(cfg.T * cfg.d, seed, 900, 1.0).reshape(cfg.T, cfg.d)
+    if cfg.dtype == "bf16":
+        dout = O.round_bf16(dout)
+    layer = G.build_layer(cfg, inp)
+    return G, cfg, inp, dout, layer
+
+
+def _check_grads(layer, cfg, ref, tol):
+    errs = {"dWg": N.rel_l2(layer.grad(L.W_GATE), ref["dWg"])}
+    if ref["dbg"] is not None:
+        errs["dbg"] = N.rel_l2(layer.grad(L.W_GATE_BIAS), ref["dbg"])
+    for g in range(cfg.E + cfg.Es):
+        for which, k in ((L.W_W1, "dW1"), (L.W_W3, "dW3"), (L.W_W2, "dW2")):
+            got = layer.grad(which, g)
+            if not ref[k][g].any():
+                assert not got.any(), (k, g)        # an expert without rows: exact zeros
+            else:
+                errs[f"{k}[{g}]"] = N.rel_l2(got, ref[k][g])
+    bad = {k: v for k, v in errs.items() if not v < tol}
+    assert not bad, bad
+
+
+CASES_F32 = [
+    ("c1_tiny_f32", {}),
+    ("c1_tiny_f32", dict(T=77, d=102, H=72)),                                   # nothing a multiple of the tiles
+    ("c1_tiny_f32", dict(T=96, d=64, H=48, E=6, K=3, renorm=False, Es=2)),      # shared experts, no renormalisation
+    ("c1_tiny_f32", dict(T=50, d=48, H=40, E=16, K=2, zipf_bias=1.2)),          # gate bias, experts without rows
+    ("c1_tiny_f32", dict(T=1, d=32, H=16, E=4, K=4)),
+]
+
+
+@pytest.mark.parametrize("name,kw", CASES_F32)
+def test_backward_fp32_matches_oracle(name, kw):
+    G, cfg, inp, dout, layer = _setup(name, kw, 31)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = G.P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    with pytest.raises(RuntimeError):      # no forward yet
+        layer.back(g)
+    out = layer.forward(x).to_numpy()
+    dx = layer.back(g).to_numpy()
+    ref = O.moe_backward(inp["x"], dout, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es)
+    assert N.rel_l2(dx, ref["dx"]) < 1e-5, N.rel_l2(dx, ref["dx"])
+    _check_grads(layer, cfg, ref, 1e-5)
+    # the forward output is untouched and a second backward gives the same bits (gradients are overwritten, not added)
+    assert np.array_equal(layer.getOutput().to_numpy(), out)
+    w1 = layer.grad(L.W_W1, 0)
+    assert np.array_equal(layer.back(g).to_numpy(), dx)
+    assert np.array_equal(layer.grad(L.W_W1, 0), w1)
+    layer.close()
+
+
+def test_acc_grad_and_update_fp32():
+    G, cfg, inp, dout, layer = _setup("c1_tiny_f32", dict(T=40, d=32, H=24, E=4, K=2, zipf_bias=1.2), 5)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g1 = G.P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    g2 = G.P.DeviceBuffer.from_numpy(G.ctx(), (0.5 * dout).astype(np.float32), cfg.dtype)
+    layer.forward(x)
+    layer.back(g1)
+    a = {k: layer.grad(w, 1) for k, w in (("W1", L.W_W1), ("W2", L.W_W2))}
+    a["Wg"], a["bg"] = layer.grad(L.W_GATE), layer.grad(L.W_GATE_BIAS)
+    layer.accGrad(1.0)                      # first call: copy
+    layer.back(g2)
+    layer.accGrad(2.0)                      # then acc += 2 * grad(0.5 dout) = 2 * grad(dout) in total
+    before = {k: layer._download_weight(w, 1, s) for k, w, s in (("W1", L.W_W1, (cfg.H, cfg.d)), ("W2", L.W_W2, (cfg.d, cfg.H)))}
+    before["Wg"] = layer._download_weight(L.W_GATE, 0, (cfg.E, cfg.d))
+    before["bg"] = layer._download_weight(L.W_GATE_BIAS, 0, (cfg.E,))
+    layer.update(0.25)
+    after = {k: layer._download_weight(w, 1, s) for k, w, s in (("W1", L.W_W1, (cfg.H, cfg.d)), ("W2", L.W_W2, (cfg.d, cfg.H)))}
+    after["Wg"] = layer._download_weight(L.W_GATE, 0, (cfg.E, cfg.d))
+    after["bg"] = layer._download_weight(L.W_GATE_BIAS, 0, (cfg.E,))
+    for k in ("W1", "W2", "Wg", "bg"):
+        want = before[k].astype(np.float64) - 0.25 * 2.0 * a[k].astype(np.float64)
+        assert N.rel_l2(after[k], want) < 1e-6, k
+    # the accumulators were cleared: the next update uses the plain gradient of the next backward
+    layer.forward(x)
+    layer.back(g1)
+    gW = layer.grad(L.W_W1, 1)
+    layer.update(1.0)
+    assert N.rel_l2(layer._download_weight(L.W_W1, 1, (cfg.H, cfg.d)), after["W1"].astype(np.float64) - gW) < 1e-6
+    layer.close()
