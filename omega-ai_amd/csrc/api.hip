@@ -152,6 +152,21 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 
 // ------------------------------------------------------------------------------------------ layer
 
+static void moe_free_backward_workspace(omega_moe *m)
+{
+    void **bw[] = {(void **)&m->bw_probs, (void **)&m->bw_dw, (void **)&m->bw_dlogits, (void **)&m->bw_dy, (void **)&m->bw_h1,
+                   (void **)&m->bw_h3, (void **)&m->bw_dxg, &m->bw_dy16, &m->bw_dys16, &m->bw_dh16, &m->bw_dyT, &m->bw_aT,
+                   &m->bw_xgT, &m->bw_dhT, (void **)&m->bw_kt0, (void **)&m->desc_da, (void **)&m->wq_da,
+                   (void **)&m->desc_w2, (void **)&m->wq_w2, (void **)&m->desc_w13, (void **)&m->wq_w13};
+    for (void **p : bw) {
+        if (*p) hipFree(*p);
+        *p = nullptr;
+    }
+    m->bw_T_cap = 0;
+    m->bw_rows_cap = 0;
+    m->bw_ksteps_cap = 0;
+}
+
 static void moe_free_workspace(omega_moe *m)
 {
     void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y,
@@ -161,19 +176,15 @@ static void moe_free_workspace(omega_moe *m)
     m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr; m->rms = nullptr; m->hbuf = nullptr;
     m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
     m->T_cap = 0;
-    void *bw[] = {m->bw_probs, m->bw_dw, m->bw_dlogits, m->bw_dy, m->bw_h1, m->bw_h3, m->bw_dxg};
-    for (void *p : bw)
-        if (p) hipFree(p);
-    m->bw_probs = m->bw_dw = m->bw_dlogits = m->bw_dy = m->bw_h1 = m->bw_h3 = m->bw_dxg = nullptr;
-    m->bw_T_cap = 0;
-    m->bw_rows_cap = 0;
+    moe_free_backward_workspace(m);
     m->fwd_T = -1;
 }
 
 static size_t grad_block_floats(const omega_moe *m)
 {
     const omega_moe_config &c = m->cfg;
-    return (size_t)c.E * c.d + (size_t)c.E + 3 * (size_t)m->G * c.H * c.d;
+    // dWg, dbg (rounded up to whole 16-byte units, so the expert gradients stay 16-byte aligned), dW13, dW2
+    return (size_t)c.E * c.d + (size_t)((c.E + 3) & ~3) + 3 * (size_t)m->G * c.H * c.d;
 }
 
 // Gradient buffers (once) and the workspace of the backward pass for the current forward workspace.
@@ -181,35 +192,75 @@ static int moe_reserve_backward(omega_moe *m, int T)
 {
     omega_ctx *ctx = m->ctx;
     const omega_moe_config &c = m->cfg;
+    const bool bf = c.dtype == OMEGA_DTYPE_BF16;
+    const size_t HD = (size_t)c.H * c.d;
     if (!m->dWg) {
         float *blk = nullptr;
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&blk, grad_block_floats(m) * 4));
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(blk, 0, grad_block_floats(m) * 4, ctx->stream));
-        const size_t per = (size_t)m->G * c.H * c.d;
         m->dWg = blk;
         m->dbg = m->dWg + (size_t)c.E * c.d;
-        m->dW1 = m->dbg + c.E;
-        m->dW3 = m->dW1 + per;
-        m->dW2 = m->dW3 + per;
+        m->dW13 = m->dbg + ((c.E + 3) & ~3);
+        m->dW2 = m->dW13 + 2 * (size_t)m->G * HD;
+    }
+    if (bf && !m->W2T) {
+        // one row group of slack behind W2T: the last 256-column tile of a width H = 128 mod 256 reads it (and drops it)
+        OMEGA_HIP_CHECK(ctx, hipMalloc(&m->W2T, ((size_t)m->G * HD + (size_t)128 * c.d) * 2));
+        OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->W2T, 0, ((size_t)m->G * HD + (size_t)128 * c.d) * 2, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, hipMalloc(&m->W13T, (size_t)m->G * 2 * HD * 2));
+        m->wT_valid = false;
+    }
+    if (bf && !m->wT_valid) {
+        // W2[g] [d,H] -> W2T[g] [H,d];  W1[g], W3[g] [H,d] -> W13T[g] [d, H | H]
+        OMEGA_HIP_CHECK(ctx, launch_transpose_images(m->W2, c.d, c.H, m->W2T, c.d / 32, 0, m->G, HD * 2, HD * 2, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, launch_transpose_images(m->W1, c.H, c.d, m->W13T, 2 * c.H / 32, 0, m->G, HD * 2, 2 * HD * 2, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, launch_transpose_images(m->W3, c.H, c.d, m->W13T, 2 * c.H / 32, c.H / 32, m->G, HD * 2, 2 * HD * 2, ctx->stream));
+        m->wT_valid = true;
     }
     if (m->bw_T_cap >= T && m->bw_rows_cap >= m->rows_cap) return OMEGA_OK;
     OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
-    void *bw[] = {m->bw_probs, m->bw_dw, m->bw_dlogits, m->bw_dy, m->bw_h1, m->bw_h3, m->bw_dxg};
-    for (void *p : bw)
-        if (p) hipFree(p);
-    m->bw_probs = m->bw_dw = m->bw_dlogits = m->bw_dy = m->bw_h1 = m->bw_h3 = m->bw_dxg = nullptr;
-    m->bw_T_cap = 0;
-    m->bw_rows_cap = 0;
+    moe_free_backward_workspace(m);
     const int Tc = m->T_cap;
+    const size_t rc = m->rows_cap;
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_probs, (size_t)Tc * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dw, (size_t)Tc * c.K * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dlogits, (size_t)Tc * c.E * 4));
-    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dy, m->rows_cap * c.d * 4));
-    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h1, m->rows_cap * c.H * 4));
-    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h3, m->rows_cap * c.H * 4));
-    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dxg, m->rows_cap * c.d * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h1, rc * c.H * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h3, rc * c.H * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dxg, rc * c.d * 4));
+    if (!bf) {
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dy, rc * c.d * 4));
+    } else {
+        const int bm = m->bm ? m->bm : 256;
+        auto alloc0 = [&](void **p, size_t bytes) -> hipError_t {
+            hipError_t e = hipMalloc(p, bytes);
+            return e != hipSuccess ? e : hipMemsetAsync(*p, 0, bytes, ctx->stream);
+        };
+        // row images: padding rows are read by the products (results dropped): keep them finite
+        OMEGA_HIP_CHECK(ctx, alloc0(&m->bw_dy16, rc * c.d * 2));
+        OMEGA_HIP_CHECK(ctx, alloc0(&m->bw_dh16, rc * 2 * c.H * 2));
+        if (c.Es > 0) OMEGA_HIP_CHECK(ctx, alloc0(&m->bw_dys16, (size_t)ceil_div(Tc, bm) * bm * c.d * 2));
+        // transposed images over k space (see bw_tables_kernel): at most 8 k steps of rounding per group; one row
+        // group of slack behind aT for the last column tile of a width H = 128 mod 256
+        m->bw_ksteps_cap = (int)(rc / 32) + 8 * m->G;
+        const size_t kb = (size_t)m->bw_ksteps_cap * 64;  // bytes of one image row
+        OMEGA_HIP_CHECK(ctx, alloc0(&m->bw_dyT, (size_t)c.d * kb));
+        OMEGA_HIP_CHECK(ctx, alloc0(&m->bw_aT, (size_t)(c.H + 128) * kb));
+        OMEGA_HIP_CHECK(ctx, alloc0(&m->bw_xgT, (size_t)c.d * kb));
+        OMEGA_HIP_CHECK(ctx, alloc0(&m->bw_dhT, (size_t)2 * c.H * kb));
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_kt0, (size_t)(m->G + 1) * 4));
+        const int nH = ceil_div(c.H, 256);
+        const size_t n_da = (size_t)m->tiles_cap * nH + OMEGA_TAIL_EXTRA;
+        const size_t n_w2 = (size_t)m->G * (c.d / 256) * nH, n_w13 = (size_t)m->G * (2 * c.H / 256) * (c.d / 256);
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_da, n_da * sizeof(omega_tile_desc)));
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_w2, n_w2 * sizeof(omega_tile_desc)));
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_w13, n_w13 * sizeof(omega_tile_desc)));
+        OMEGA_HIP_CHECK(ctx, alloc0((void **)&m->wq_da, (n_da / m->n_wg + 2) * m->n_wg * sizeof(omega_tile_desc)));
+        OMEGA_HIP_CHECK(ctx, alloc0((void **)&m->wq_w2, (n_w2 / m->n_wg + 2) * m->n_wg * sizeof(omega_tile_desc)));
+        OMEGA_HIP_CHECK(ctx, alloc0((void **)&m->wq_w13, (n_w13 / m->n_wg + 2) * m->n_wg * sizeof(omega_tile_desc)));
+    }
     m->bw_T_cap = Tc;
-    m->bw_rows_cap = m->rows_cap;
+    m->bw_rows_cap = rc;
     return OMEGA_OK;
 }
 
@@ -317,7 +368,7 @@ int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **ou
     alloc0(&m->W2, wsz);
     alloc0((void **)&m->counts, (size_t)c.E * 4);
     alloc0((void **)&m->offsets, (size_t)(c.E + 1) * 4);
-    alloc0((void **)&m->tile_meta, (size_t)(m->G + 4) * 4);
+    alloc0((void **)&m->tile_meta, (size_t)(m->G + 8) * 4);
     if (e == hipSuccess) e = hipEventCreate(&m->ev0);
     if (e == hipSuccess) e = hipEventCreate(&m->ev1);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -362,6 +413,8 @@ int omega_moe_destroy(omega_moe *m)
         if (p) hipFree(p);
     if (m->dWg) hipFree(m->dWg);
     if (m->acc_grad) hipFree(m->acc_grad);
+    if (m->W2T) hipFree(m->W2T);
+    if (m->W13T) hipFree(m->W13T);
     hipEventDestroy(m->ev0);
     hipEventDestroy(m->ev1);
     for (hipEvent_t ev : m->prof_events) hipEventDestroy(ev);
@@ -410,6 +463,7 @@ int omega_moe_set_weights(omega_moe *m, int which, int expert, const void *src, 
         return OMEGA_OK;
     }
     const int R = which == OMEGA_W_W2 ? m->cfg.d : m->cfg.H, Kd = which == OMEGA_W_W2 ? m->cfg.H : m->cfg.d;
+    m->wT_valid = false;  // the transposed copies of the backward pass are rebuilt by the next backward
     void *stage = nullptr;
     if (!is_device) {
         OMEGA_HIP_CHECK(ctx, hipMalloc(&stage, bytes));
@@ -560,12 +614,12 @@ int omega_moe_backward(omega_moe *m, const void *x, const void *dout, int T, voi
 {
     MOE_ENTER(m);
     RUN(check_T(m, x, T, true));
-    if (m->cfg.dtype != OMEGA_DTYPE_F32) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "backward: fp32 layers only");
     if (T != m->fwd_T) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "backward: no omega_moe_forward has run for this T");
     if (T == 0) return OMEGA_OK;
     if (!dout || !dx) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "backward: dout or dx is NULL");
     RUN(moe_reserve_backward(m, T));
-    OMEGA_HIP_CHECK(ctx, launch_backward_f32(m, x, dout, T, dx, ctx->stream));
+    if (m->cfg.dtype == OMEGA_DTYPE_BF16) OMEGA_HIP_CHECK(ctx, launch_backward_bf16(m, x, dout, T, dx, ctx->stream));
+    else OMEGA_HIP_CHECK(ctx, launch_backward_f32(m, x, dout, T, dx, ctx->stream));
     return OMEGA_OK;
 }
 
@@ -578,7 +632,8 @@ static int grad_slot(omega_moe *m, int which, int expert, float **ptr, size_t *f
         case OMEGA_W_GATE_BIAS: *ptr = m->dbg; *floats = (size_t)c.E; return OMEGA_OK;
         case OMEGA_W_W1: case OMEGA_W_W3: case OMEGA_W_W2:
             if (expert < 0 || expert >= m->G) return OMEGA_ERR_INVALID_ARG;
-            *ptr = (which == OMEGA_W_W1 ? m->dW1 : which == OMEGA_W_W3 ? m->dW3 : m->dW2) + per * (size_t)expert;
+            *ptr = which == OMEGA_W_W2 ? m->dW2 + per * (size_t)expert
+                                       : m->dW13 + per * (2 * (size_t)expert + (which == OMEGA_W_W3 ? 1 : 0));
             *floats = per;
             return OMEGA_OK;
         default: return OMEGA_ERR_INVALID_ARG;
@@ -622,12 +677,14 @@ int omega_moe_update(omega_moe *m, float lr)
         OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(m->dWg, m->acc_grad, grad_block_floats(m) * 4, hipMemcpyDeviceToDevice, ctx->stream));
         m->acc_valid = false;
     }
-    const size_t per = (size_t)m->G * c.H * c.d;
+    const size_t per = (size_t)c.H * c.d;
     OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->Wg, m->dWg, -lr, (size_t)c.E * c.d, ctx->stream));
     if (c.has_gate_bias) OMEGA_HIP_CHECK(ctx, launch_axpy_f32(m->bg, m->dbg, -lr, (size_t)c.E, ctx->stream));
-    OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W1, m->dW1, -lr, per, ctx->stream));
-    OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W3, m->dW3, -lr, per, ctx->stream));
-    OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W2, m->dW2, -lr, per, ctx->stream));
+    for (int g = 0; g < m->G; ++g) {
+        OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W1 + per * g, m->dW13 + per * 2 * g, -lr, per, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W3 + per * g, m->dW13 + per * (2 * g + 1), -lr, per, ctx->stream));
+    }
+    OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W2, m->dW2, -lr, per * m->G, ctx->stream));
     return OMEGA_OK;
 }
 

@@ -18,6 +18,7 @@
 //   bw_router_kernel    combine weights -> (renormalisation) -> selected probabilities -> softmax -> dlogits
 //   bw_dx_kernel        dx[t,:] = sum_j dxg[row(t,j),:] + shared rows + dlogits[t,:] . Wg
 #include "common.h"
+#include "pack.h"
 
 #define GBM 64
 #define GBN 64
@@ -137,9 +138,12 @@ __global__ __launch_bounds__(256) void bw_rows_f32_kernel(const float *__restric
 // without rows gets zeros.  grid (ceil(N/64), ceil(M/64), groups).  Rows of group g: physical rows from
 // tile_meta[1+g]*bm, counts[g] of them for a routed expert, T for a shared one; a shared group reads token rows
 // 0..T-1 of Atok / Btok when those are given.  single_rows >= 0: one group, rows 0..single_rows-1 of Aphys / Bphys.
+// gstride: floats between the outputs of consecutive groups.  BBF: B holds bf16 (single-group use only).
+template <bool BBF>
 __global__ __launch_bounds__(256) void bw_wgrad_f32_kernel(const float *__restrict__ Aphys, const float *__restrict__ Atok,
                                                            const float *__restrict__ Bphys, const float *__restrict__ Btok,
-                                                           float *__restrict__ dW, const int32_t *__restrict__ tile_meta,
+                                                           float *__restrict__ dW, size_t gstride,
+                                                           const int32_t *__restrict__ tile_meta,
                                                            const int32_t *__restrict__ counts, int E, int T, int bm,
                                                            int M, int N, int single_rows)
 {
@@ -162,7 +166,9 @@ __global__ __launch_bounds__(256) void bw_wgrad_f32_kernel(const float *__restri
             const int rr = idx / GBM, cc = idx % GBM;
             const int r = r0 + rr;
             As[rr][cc] = (r < rows && m0 + cc < M) ? A[(size_t)r * M + m0 + cc] : 0.0f;
-            Bs[rr][cc] = (r < rows && n0 + cc < N) ? B[(size_t)r * N + n0 + cc] : 0.0f;
+            Bs[rr][cc] = (r < rows && n0 + cc < N)
+                             ? (BBF ? bf16_to_f32(((const bf16_t *)B)[(size_t)r * N + n0 + cc]) : B[(size_t)r * N + n0 + cc])
+                             : 0.0f;
         }
         __syncthreads();
 #pragma unroll
@@ -179,7 +185,7 @@ __global__ __launch_bounds__(256) void bw_wgrad_f32_kernel(const float *__restri
         }
         __syncthreads();
     }
-    float *out = dW + (size_t)g * M * N;
+    float *out = dW + (size_t)g * gstride;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int mm = m0 + ty * 4 + i;
@@ -237,10 +243,12 @@ __global__ __launch_bounds__(256) void bw_gate_bias_kernel(const float *__restri
 }
 
 // One workgroup per token: dx[t,:] = sum_j dxg[row(t,j),:] (slot order) + shared-expert rows + dlogits[t,:] . Wg.
+// XBF: Wg and dx are bf16 (one rounding of the fp32 sum).
+template <bool XBF>
 __global__ __launch_bounds__(256) void bw_dx_kernel(const float *__restrict__ dxg, const int32_t *__restrict__ dstp,
-                                                    const float *__restrict__ dlogits, const float *__restrict__ Wg,
+                                                    const float *__restrict__ dlogits, const void *__restrict__ Wg,
                                                     const int32_t *__restrict__ tile_meta, int K, int d, int E, int Es,
-                                                    int bm, float *__restrict__ dx)
+                                                    int bm, void *__restrict__ dx)
 {
     const int t = blockIdx.x;
     extern __shared__ float dl[];  // E floats
@@ -251,8 +259,10 @@ __global__ __launch_bounds__(256) void bw_dx_kernel(const float *__restrict__ dx
         for (int j = 0; j < K; ++j) acc += dxg[(size_t)dstp[(size_t)t * K + j] * d + c];
         for (int s = 0; s < Es; ++s) acc += dxg[((size_t)tile_meta[1 + E + s] * bm + t) * d + c];
         float gs = 0.0f;
-        for (int e = 0; e < E; ++e) gs = fmaf(dl[e], Wg[(size_t)e * d + c], gs);
-        dx[(size_t)t * d + c] = acc + gs;
+        for (int e = 0; e < E; ++e)
+            gs = fmaf(dl[e], XBF ? bf16_to_f32(((const bf16_t *)Wg)[(size_t)e * d + c]) : ((const float *)Wg)[(size_t)e * d + c], gs);
+        if (XBF) ((bf16_t *)dx)[(size_t)t * d + c] = f32_to_bf16(acc + gs);
+        else ((float *)dx)[(size_t)t * d + c] = acc + gs;
     }
 }
 
@@ -296,25 +306,121 @@ hipError_t launch_backward_f32(const omega_moe *m, const void *xv, const void *d
     hipLaunchKernelGGL((bw_rows_f32_kernel<true, 1>), gD, dim3(256), 0, s, (const float *)m->bw_h3, (const float *)nullptr,
                        W3, m->bw_dxg, (float *)nullptr, m->tiles, m->tile_meta, c.d, c.H);
     // weight gradients: dW2 = dy^T a [d,H]; dW1 = dh1^T xg, dW3 = dh3^T xg [H,d]
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.H, GBN), ceil_div(c.d, GBM), G), dim3(256), 0, s,
-                       (const float *)m->bw_dy, dout, a, (const float *)nullptr, m->dW2, m->tile_meta, m->counts, c.E, T,
+    const size_t HD = (size_t)c.H * c.d;
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel<false>, dim3(ceil_div(c.H, GBN), ceil_div(c.d, GBM), G), dim3(256), 0, s,
+                       (const float *)m->bw_dy, dout, a, (const float *)nullptr, m->dW2, HD, m->tile_meta, m->counts, c.E, T,
                        m->bm, c.d, c.H, -1);
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
-                       (const float *)m->bw_h1, (const float *)nullptr, xg, x, m->dW1, m->tile_meta, m->counts, c.E, T,
-                       m->bm, c.H, c.d, -1);
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
-                       (const float *)m->bw_h3, (const float *)nullptr, xg, x, m->dW3, m->tile_meta, m->counts, c.E, T,
-                       m->bm, c.H, c.d, -1);
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel<false>, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
+                       (const float *)m->bw_h1, (const float *)nullptr, xg, x, m->dW13, 2 * HD, m->tile_meta, m->counts, c.E,
+                       T, m->bm, c.H, c.d, -1);
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel<false>, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
+                       (const float *)m->bw_h3, (const float *)nullptr, xg, x, m->dW13 + HD, 2 * HD, m->tile_meta, m->counts,
+                       c.E, T, m->bm, c.H, c.d, -1);
     // router and gate
     hipLaunchKernelGGL(bw_router_kernel, dim3(ceil_div(T, 256)), dim3(256), 0, s, (const float *)m->bw_probs, m->ids, m->w,
                        (const float *)m->bw_dw, T, c.E, c.K, c.renorm, m->bw_dlogits);
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.E, GBM), 1), dim3(256), 0, s,
-                       (const float *)m->bw_dlogits, (const float *)nullptr, x, (const float *)nullptr, m->dWg,
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel<false>, dim3(ceil_div(c.d, GBN), ceil_div(c.E, GBM), 1), dim3(256), 0, s,
+                       (const float *)m->bw_dlogits, (const float *)nullptr, x, (const float *)nullptr, m->dWg, (size_t)0,
                        m->tile_meta, m->counts, c.E, T, m->bm, c.E, c.d, T);
     if (c.has_gate_bias)
         hipLaunchKernelGGL(bw_gate_bias_kernel, dim3(c.E), dim3(256), 0, s, (const float *)m->bw_dlogits, T, c.E, m->dbg);
-    hipLaunchKernelGGL(bw_dx_kernel, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,
-                       (const float *)m->bw_dlogits, (const float *)m->Wg, m->tile_meta, c.K, c.d, c.E, c.Es, m->bm,
-                       (float *)dxv);
+    hipLaunchKernelGGL(bw_dx_kernel<false>, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,
+                       (const float *)m->bw_dlogits, (const void *)m->Wg, m->tile_meta, c.K, c.d, c.E, c.Es, m->bm, dxv);
+    return hipGetLastError();
+}
+
+
+// ------------------------------------------------------------------------------------------ bf16 layers
+// One workgroup per token: dy rows (bf16, packed tile image) and dw; with shared experts also the packed copy of dout
+// their products read.
+__global__ __launch_bounds__(256) void bw_combine_bf16_kernel(const uint4 *__restrict__ dout, const float *__restrict__ y,
+                                                              const int32_t *__restrict__ dstp, const float *__restrict__ w,
+                                                              int K, int d, unsigned char *__restrict__ dy16,
+                                                              unsigned char *__restrict__ dys16, float *__restrict__ dw)
+{
+    __shared__ float red[4];
+    const int t = blockIdx.x, nch = d >> 3, KT = d >> 5;
+    for (int j = 0; j < K; ++j) {
+        const int r = dstp[(size_t)t * K + j];
+        const float wv = w[(size_t)t * K + j];
+        float part = 0.0f;
+        for (int ch = threadIdx.x; ch < nch; ch += 256) {
+            const uint4 u = dout[(size_t)t * nch + ch];
+            const uint32_t uw[4] = {u.x, u.y, u.z, u.w};
+            const float4 y0 = *(const float4 *)(y + (size_t)r * d + ch * 8), y1 = *(const float4 *)(y + (size_t)r * d + ch * 8 + 4);
+            const float yv[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
+            uint32_t ow[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float g0 = __uint_as_float(uw[q] << 16), g1 = __uint_as_float(uw[q] & 0xffff0000u);
+                part = fmaf(g0, yv[2 * q], part);
+                part = fmaf(g1, yv[2 * q + 1], part);
+                ow[q] = (uint32_t)f32_to_bf16(wv * g0) | ((uint32_t)f32_to_bf16(wv * g1) << 16);
+            }
+            *(uint4 *)(dy16 + pk_chunk_off(r, ch >> 2, ch & 3, KT)) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+        }
+        const float tot = block_sum_256(part, red);
+        if (threadIdx.x == 0) dw[(size_t)t * K + j] = tot;
+    }
+    if (dys16 != nullptr)
+        for (int ch = threadIdx.x; ch < nch; ch += 256)
+            *(uint4 *)(dys16 + pk_chunk_off(t, ch >> 2, ch & 3, KT)) = dout[(size_t)t * nch + ch];
+}
+
+// The weight gradients of a group without rows are zero; the product kernels have no items for it.
+__global__ __launch_bounds__(256) void bw_zero_empty_kernel(const int32_t *__restrict__ counts, int E, int T,
+                                                            float *__restrict__ dW13, float *__restrict__ dW2, size_t HD)
+{
+    const int g = blockIdx.x;
+    if ((g < E ? counts[g] : T) > 0) return;
+    float4 *p13 = (float4 *)(dW13 + (size_t)g * 2 * HD), *p2 = (float4 *)(dW2 + (size_t)g * HD);
+    const float4 z = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (size_t i = (size_t)blockIdx.y * 256 + threadIdx.x; i < HD / 4; i += (size_t)gridDim.y * 256) {
+        p13[i] = z;
+        p13[HD / 4 + i] = z;
+        p2[i] = z;
+    }
+}
+
+hipError_t launch_backward_bf16(const omega_moe *m, const void *x, const void *dout, int T, void *dx, hipStream_t s)
+{
+    const omega_moe_config &c = m->cfg;
+    const int G = m->G;
+    const size_t HD = (size_t)c.H * c.d;
+    hipError_t e;
+#define STEP(expr) if ((e = (expr)) != hipSuccess) return e
+    STEP(launch_router(m, x, T, nullptr, m->bw_probs, s));
+    STEP(launch_backward_tables(m, T, s));
+    hipLaunchKernelGGL(bw_combine_bf16_kernel, dim3(T), dim3(256), 0, s, (const uint4 *)dout, (const float *)m->y, m->dstp, m->w,
+                       c.K, c.d, (unsigned char *)m->bw_dy16, (unsigned char *)m->bw_dys16, m->bw_dw);
+    STEP(hipGetLastError());
+    // h1, h3 (recomputed) as block records; d(a) = dy . W2 with the SwiGLU backward in its epilogue -> dh1 | dh3;
+    // dxg = dh1 . W1 + dh3 . W3 as one product over the 2H columns of dh
+    STEP(launch_product_bf16(m, MODE_UPRAW, m->xg, m->xs, m->W1, m->W3, m->bw_h1, m->bw_h3, nullptr, m->wq_up, c.H, c.d, s));
+    STEP(launch_product_bf16(m, MODE_DA, m->bw_dy16, m->bw_dys16, m->W2T, nullptr, m->bw_dh16, m->bw_h1, m->bw_h3, m->wq_da,
+                             c.H, c.d, s));
+    STEP(launch_product_bf16(m, MODE_DOWN, m->bw_dh16, nullptr, m->W13T, nullptr, m->bw_dxg, nullptr, nullptr, m->wq_down, c.d,
+                             2 * c.H, s));
+    // weight gradients: the experts' rows become the K axis of transposed images
+    STEP(launch_transpose_groups(m, m->bw_dy16, m->bw_dys16, c.d, m->bw_dyT, T, s));
+    STEP(launch_transpose_groups(m, m->a, nullptr, c.H, m->bw_aT, T, s));
+    STEP(launch_transpose_groups(m, m->xg, m->xs, c.d, m->bw_xgT, T, s));
+    STEP(launch_transpose_groups(m, m->bw_dh16, nullptr, 2 * c.H, m->bw_dhT, T, s));
+    STEP(launch_product_bf16(m, MODE_WGRAD, m->bw_dyT, nullptr, m->bw_aT, nullptr, m->dW2, nullptr, nullptr, m->wq_w2, c.H,
+                             m->bw_ksteps_cap * 32, s));
+    STEP(launch_product_bf16(m, MODE_WGRAD, m->bw_dhT, nullptr, m->bw_xgT, nullptr, m->dW13, nullptr, nullptr, m->wq_w13, c.d,
+                             m->bw_ksteps_cap * 32, s));
+    hipLaunchKernelGGL(bw_zero_empty_kernel, dim3(G, 32), dim3(256), 0, s, m->counts, c.E, T, m->dW13, m->dW2, HD);
+    // router and gate
+    hipLaunchKernelGGL(bw_router_kernel, dim3(ceil_div(T, 256)), dim3(256), 0, s, (const float *)m->bw_probs, m->ids, m->w,
+                       (const float *)m->bw_dw, T, c.E, c.K, c.renorm, m->bw_dlogits);
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel<true>, dim3(ceil_div(c.d, GBN), ceil_div(c.E, GBM), 1), dim3(256), 0, s,
+                       (const float *)m->bw_dlogits, (const float *)nullptr, (const float *)x, (const float *)nullptr, m->dWg,
+                       (size_t)0, m->tile_meta, m->counts, c.E, T, m->bm, c.E, c.d, T);
+    if (c.has_gate_bias)
+        hipLaunchKernelGGL(bw_gate_bias_kernel, dim3(c.E), dim3(256), 0, s, (const float *)m->bw_dlogits, T, c.E, m->dbg);
+    hipLaunchKernelGGL(bw_dx_kernel<true>, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,
+                       (const float *)m->bw_dlogits, (const void *)m->Wg, m->tile_meta, c.K, c.d, c.E, c.Es, m->bm, dx);
+#undef STEP
     return hipGetLastError();
 }

@@ -40,7 +40,9 @@ struct __attribute__((aligned(16))) omega_tile {
 struct __attribute__((aligned(32))) omega_tile_desc {
     int32_t g, row0, rows, xrow0;  // as omega_tile
     int32_t n0;                    // first output column of the tile
-    int32_t pad[3];
+    // weight-gradient items only (zero otherwise): row groups (128 rows) of the two operand tiles in their transposed
+    // images and the first k step of the expert's rows there; xrow0 then holds the item's number of k steps
+    int32_t a_rg, b_rg, kt0;
 };
 
 struct omega_moe {
@@ -88,8 +90,9 @@ struct omega_moe {
     int max_m_tiles = 0;
     // backward pass (allocated by the first omega_moe_backward): parameter gradients, always fp32, in the layout of
     // their weights, the accumulators of accGrad, and the workspace of the pass, indexed by physical rows like xg / a / y
-    float *dWg = nullptr, *dbg = nullptr, *dW1 = nullptr, *dW3 = nullptr, *dW2 = nullptr;
-    float *acc_grad = nullptr;       // accumulators, one block in the order dWg, dbg, dW1, dW3, dW2
+    // (dW13: [G][2][H,d], the gradients of W1 and W3 of an expert back to back)
+    float *dWg = nullptr, *dbg = nullptr, *dW13 = nullptr, *dW2 = nullptr;
+    float *acc_grad = nullptr;       // accumulators, one block in the order dWg, dbg, dW13, dW2
     bool acc_valid = false;          // accGrad has run since the last update
     float *bw_probs = nullptr;       // [T,E] softmax of the gate logits
     float *bw_dw = nullptr;          // [T,K] gradient of the combine weights
@@ -98,6 +101,19 @@ struct omega_moe {
     float *bw_h1 = nullptr;          // [rows_cap,H] h1, then dh1
     float *bw_h3 = nullptr;          // [rows_cap,H] h3, then dh3
     float *bw_dxg = nullptr;         // [rows_cap,d] gradient of the expert inputs
+    // bf16 layers: the products of the pass run on the matrix-core kernel of the forward pass (see experts_bf16.hip)
+    void *bw_dy16 = nullptr;         // [rows_cap,d] packed bf16: dy
+    void *bw_dys16 = nullptr;        // [ceil(T/bm)*bm,d] packed bf16 copy of dout (rows of the shared experts)
+    void *bw_dh16 = nullptr;         // [rows_cap,2H] packed bf16: dh1 | dh3  (bw_h1 / bw_h3 hold the h1 / h3 block records)
+    void *bw_dyT = nullptr, *bw_aT = nullptr, *bw_xgT = nullptr, *bw_dhT = nullptr;  // transposed packed images over k space
+    int32_t *bw_kt0 = nullptr;       // [G+1] first k step of each group in k space
+    int bw_ksteps_cap = 0;           // k steps the transposed images are laid out for
+    omega_tile_desc *desc_da = nullptr, *wq_da = nullptr;    // d(a) product: 256-column tiles over H
+    omega_tile_desc *desc_w2 = nullptr, *wq_w2 = nullptr;    // dW2 = dy^T a
+    omega_tile_desc *desc_w13 = nullptr, *wq_w13 = nullptr;  // dW1 | dW3 = dh^T xg
+    void *W2T = nullptr;             // [G][H,d] packed: transposed W2 (+ one row group of slack)
+    void *W13T = nullptr;            // [G][d,2H] packed: W1^T | W3^T
+    bool wT_valid = false;           // the transposed copies match the weights
     int bw_T_cap = 0;
     size_t bw_rows_cap = 0;
     int fwd_T = -1;                  // tokens of the last plain forward (what backward may follow), -1: none
@@ -138,6 +154,16 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
 // resid != nullptr: out = resid + layer output (one rounding of the fp32 sum)
 hipError_t launch_combine(const omega_moe *m, int T, void *out, const void *resid, hipStream_t s);
 hipError_t launch_backward_f32(const omega_moe *m, const void *x, const void *dout, int T, void *dx, hipStream_t s);
+hipError_t launch_backward_bf16(const omega_moe *m, const void *x, const void *dout, int T, void *dx, hipStream_t s);
+hipError_t launch_backward_tables(const omega_moe *m, int T, hipStream_t s);
+hipError_t launch_transpose_groups(const omega_moe *m, const void *src, const void *src_alt, int cols, void *dst, int T,
+                                   hipStream_t s);
+hipError_t launch_transpose_images(const void *src, int R, int cols, void *dst, int KTd, int k0, int n, size_t src_stride,
+                                   size_t dst_stride, hipStream_t s);
+// products of the matrix-core kernel (experts_bf16.hip describes each)
+enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4 };
+hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, const void *Aalt, const void *Wa, const void *Wb,
+                               void *Cout, void *Aux1, void *Aux2, const omega_tile_desc *wq, int N, int Kd, hipStream_t s);
 hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, hipStream_t s);
 hipError_t launch_mfma_probe(float *scratch, int num_cus, int random_operands, int launches, hipStream_t s,
                              double *flop_per_launch);

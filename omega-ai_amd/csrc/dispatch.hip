@@ -52,6 +52,50 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(const int32_t *__res
     }
 }
 
+// The work items of group g in one product's table (see the comment in dispatch_rank_kernel): NT column tiles of
+// ncols columns, Mg row tiles starting at row tile mt0; the launch has total_mt row tiles in all.  All 256 threads.
+__device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ desc, int NT, int ncols, int g, int rows,
+                                                  int Mg, int mt0, int total_mt, int bm, bool shared)
+{
+    if (desc == nullptr) return;
+    const int Nt = total_mt * NT, r = Nt % 256;
+    const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
+    const int nblk = (rows + 31) >> 5;  // 32-row blocks of the group, dealt evenly to its Mg row tiles
+    for (int l = threadIdx.x; l < Mg * NT; l += 256) {
+        const int mt = l % Mg, n = l / Mg;
+        const int at = mt0 * NT + l;
+        const int tfirst = 32 * ((mt * nblk) / Mg);
+        const int trows = min(32 * (((mt + 1) * nblk) / Mg), rows) - tfirst;
+        omega_tile_desc dsc;
+        dsc.g = g;
+        dsc.n0 = n * ncols;
+        dsc.a_rg = dsc.b_rg = dsc.kt0 = 0;
+        if (at < Nt - r) {
+            dsc.row0 = mt0 * bm + tfirst;
+            dsc.rows = trows;
+            dsc.xrow0 = shared ? tfirst : -1;
+            desc[at] = dsc;
+        } else {
+            const int tb = (trows + 31) >> 5;  // the tile's 32-row blocks, dealt evenly to the S slices
+            for (int sl = 0; sl < S; ++sl) {
+                const int sfirst = 32 * ((sl * tb) / S);
+                dsc.row0 = mt0 * bm + tfirst + sfirst;
+                dsc.rows = max(0, min(32 * (((sl + 1) * tb) / S), trows) - sfirst);  // 0: nothing to do
+                dsc.xrow0 = shared ? tfirst + sfirst : -1;
+                desc[Nt - r + (at - (Nt - r)) * S + sl] = dsc;
+            }
+        }
+    }
+}
+
+// entries of a table whose launch has total_mt row tiles and NT column tiles (with the last tiles sliced)
+__device__ __forceinline__ int table_entries(int total_mt, int NT)
+{
+    const int Nt = total_mt * NT, r = Nt % 256;
+    const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
+    return Nt - r + r * S;
+}
+
 // MAXE: experts are limited to 256 per layer by the router kernels.
 #define MAXE 256
 __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__restrict__ ids,
@@ -148,47 +192,12 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     // the weight tile in its L2).  Group g is written by workgroup g (mod grid).
     if (desc_up != nullptr || desc_down != nullptr) {
         const int G = E + Es;
-        if (tile == 0 && tid < 2) {
-            const int Nt = mt_s[G] * (tid == 0 ? nt_up : nt_down), r = Nt % 256;
-            const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
-            tile_meta[G + 2 + tid] = Nt - r + r * S;
-        }
+        if (tile == 0 && tid < 2) tile_meta[G + 2 + tid] = table_entries(mt_s[G], tid == 0 ? nt_up : nt_down);
         for (int g = tile; g < G; g += gridDim.x) {
             const int rows = g < E ? off_s[g + 1] - off_s[g] : T;
             const int Mg = mt_s[g + 1] - mt_s[g];
-            for (int pass = 0; pass < 2; ++pass) {
-                omega_tile_desc *desc = pass == 0 ? desc_up : desc_down;
-                const int NT = pass == 0 ? nt_up : nt_down, ncols = pass == 0 ? ncols_up : ncols_down;
-                if (desc == nullptr) continue;
-                const int Nt = mt_s[G] * NT, r = Nt % 256;
-                const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
-                const int nblk = (rows + 31) >> 5;  // 32-row blocks of the group, dealt evenly to its Mg row tiles
-                for (int l = tid; l < Mg * NT; l += 256) {
-                    const int mt = l % Mg, n = l / Mg;
-                    const int at = mt_s[g] * NT + l;
-                    const int tfirst = 32 * ((mt * nblk) / Mg);
-                    const int trows = min(32 * (((mt + 1) * nblk) / Mg), rows) - tfirst;
-                    omega_tile_desc dsc;
-                    dsc.g = g;
-                    dsc.n0 = n * ncols;
-                    dsc.pad[0] = dsc.pad[1] = dsc.pad[2] = 0;
-                    if (at < Nt - r) {
-                        dsc.row0 = mt_s[g] * bm + tfirst;
-                        dsc.rows = trows;
-                        dsc.xrow0 = g < E ? -1 : tfirst;
-                        desc[at] = dsc;
-                    } else {
-                        const int tb = (trows + 31) >> 5;  // the tile's 32-row blocks, dealt evenly to the S slices
-                        for (int sl = 0; sl < S; ++sl) {
-                            const int sfirst = 32 * ((sl * tb) / S);
-                            dsc.row0 = mt_s[g] * bm + tfirst + sfirst;
-                            dsc.rows = max(0, min(32 * (((sl + 1) * tb) / S), trows) - sfirst);  // 0: nothing to do
-                            dsc.xrow0 = g < E ? -1 : tfirst + sfirst;
-                            desc[Nt - r + (at - (Nt - r)) * S + sl] = dsc;
-                        }
-                    }
-                }
-            }
+            write_group_items(desc_up, nt_up, ncols_up, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E);
+            write_group_items(desc_down, nt_down, ncols_down, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E);
         }
     }
 }
@@ -213,11 +222,14 @@ __device__ __forceinline__ int work_item_cost(int rows)
     return 2 + (14 * nb) / 8;         // sixteenths of a full tile; the loads and the fixed part do not shrink
 }
 
+// up to three tables per launch: table p is scheduled by workgroups 8p .. 8p+7
 struct sched_args {
-    const omega_tile_desc *desc_up, *desc_down;
-    omega_tile_desc *wq_up, *wq_down;
+    const omega_tile_desc *desc[3];
+    omega_tile_desc *wq[3];
+    int total_slot[3];  // index in tile_meta of the table's number of entries
+    int kcost[3];       // 0: an item costs by its rows; 1: by its k steps (weight-gradient items, all 256 rows high)
     const int32_t *tile_meta;
-    int G, n_wg;
+    int n_wg;
 };
 
 __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
@@ -226,10 +238,11 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
     __shared__ unsigned short place_s[SCHED_RC * 32];  // [round][workgroup j] = 0x8000 | (queue slot - len0) << 5 | source lane
     __shared__ int len0_s[32];
     const int pass = which >> 3, x = which & 7, tid = threadIdx.x, lane = tid & 63;
-    const omega_tile_desc *desc = pass == 0 ? a.desc_up : a.desc_down;
-    omega_tile_desc *wq = pass == 0 ? a.wq_up : a.wq_down;
+    const omega_tile_desc *desc = pass == 0 ? a.desc[0] : pass == 1 ? a.desc[1] : a.desc[2];
+    omega_tile_desc *wq = pass == 0 ? a.wq[0] : pass == 1 ? a.wq[1] : a.wq[2];
+    const int kcost = pass == 0 ? a.kcost[0] : pass == 1 ? a.kcost[1] : a.kcost[2];
     const int n_wg = a.n_wg, wpx = n_wg >> 3;
-    const int total = a.tile_meta[a.G + 2 + pass];
+    const int total = a.tile_meta[pass == 0 ? a.total_slot[0] : pass == 1 ? a.total_slot[1] : a.total_slot[2]];
     const int rounds = (total + n_wg - 1) / n_wg;
     // entry of (round r, place i of this XCD), or -1
     auto entry = [&](int r, int i) {
@@ -247,12 +260,12 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
             for (int u = 0; u < 4; ++u) {
                 const int idx = i0 + u * 256 + tid;
                 const int L = idx < nr * 32 ? entry(r0 + (idx >> 5), idx & 31) : -1;
-                rows[u] = L >= 0 ? desc[L].rows : 0;
+                rows[u] = L >= 0 ? (kcost ? -desc[L].xrow0 : desc[L].rows) : 0;
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int idx = i0 + u * 256 + tid;
-                if (idx < nr * 32) cost_s[idx] = (unsigned char)work_item_cost(rows[u]);
+                if (idx < nr * 32) cost_s[idx] = (unsigned char)(rows[u] < 0 ? min(255, 2 + (-rows[u]) / 8) : work_item_cost(rows[u]));
             }
         }
         if (tid < 32) len0_s[tid] = len;
@@ -399,7 +412,9 @@ hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipS
     const omega_moe_config &c = m->cfg;
     const size_t row_bytes = (size_t)c.d * m->esize;
     if (c.dtype == OMEGA_DTYPE_BF16) {  // d % 256 == 0 is guaranteed at creation: rows are whole 64-byte k steps
-        sched_args sa = {m->desc_up, m->desc_down, m->wq_up, m->wq_down, m->tile_meta, c.E + c.Es, m->n_wg};
+        const int G = c.E + c.Es;
+        sched_args sa = {{m->desc_up, m->desc_down, nullptr}, {m->wq_up, m->wq_down, nullptr}, {G + 2, G + 3, 0}, {0, 0, 0},
+                         m->tile_meta, m->n_wg};
         hipLaunchKernelGGL(dispatch_gather_kernel<true>, dim3(ceil_div(T, 4) + SCHED_WGS), dim3(256), 0, s, (const uint4 *)x,
                            m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs, SCHED_WGS, sa);
     } else if (row_bytes % 16 == 0 && ((uintptr_t)x % 16) == 0) {
@@ -442,5 +457,185 @@ hipError_t launch_unpack_rows(void *dst_rowmajor, const void *src_packed, int R,
     const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
     hipLaunchKernelGGL(pack_rows_kernel, dim3(grid), dim3(256), 0, s, (unsigned char *)src_packed, (uint4 *)dst_rowmajor, R,
                        Kd / 8, 0);
+    return hipGetLastError();
+}
+
+
+// ---- work-item tables of the backward products (bf16 layers) ----
+// k space of the weight gradients: the experts' rows, expert after expert, each expert's share rounded up to 64 rows
+// and to at least 192 (a product item must be longer than the load ring of the product kernel); kt0[g] = first k step
+// (32 rows) of group g, kt0[G] = all of them.  Empty groups take no space and get no items.
+__device__ __forceinline__ int kspace_steps(int rows) { return rows > 0 ? max((rows + 63) / 64 * 2, 6) : 0; }
+
+// One workgroup per group g: the items of the d(a) product (256-column tiles over H, table as the forward ones), the
+// group's place in k space, and its items of the two weight-gradient products (all 256 x 256 tiles of dW_g, column
+// tile by column tile; descriptor: row0 = g*M + first row, xrow0 = k steps, a_rg / b_rg = operand row groups).
+__global__ __launch_bounds__(256) void bw_tables_kernel(int32_t *__restrict__ tile_meta, const int32_t *__restrict__ counts,
+                                                        int E, int Es, int T, int bm, omega_tile_desc *__restrict__ desc_da,
+                                                        int nt_da, int32_t *__restrict__ kt0,
+                                                        omega_tile_desc *__restrict__ desc_w2, int M2, int NT2,
+                                                        omega_tile_desc *__restrict__ desc_w13, int M13, int NT13)
+{
+    __shared__ int red_k[4], red_n[4];
+    const int G = E + Es, g = blockIdx.x, tid = threadIdx.x;
+    const int rows = g < E ? counts[g] : T;
+    const int mt0 = tile_meta[1 + g], Mg = tile_meta[2 + g] - mt0, total_mt = tile_meta[1 + G];
+    write_group_items(desc_da, nt_da, 256, g, rows, Mg, mt0, total_mt, bm, g >= E);
+    if (g == 0 && tid == 0) tile_meta[G + 4] = table_entries(total_mt, nt_da);
+    // k steps and non-empty groups before g
+    int ks = 0, ne = 0;
+    for (int q = tid; q < g; q += 256) {
+        const int r = q < E ? counts[q] : T;
+        ks += kspace_steps(r);
+        ne += r > 0 ? 1 : 0;
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        ks += __shfl_xor(ks, m, 64);
+        ne += __shfl_xor(ne, m, 64);
+    }
+    if ((tid & 63) == 0) { red_k[tid >> 6] = ks; red_n[tid >> 6] = ne; }
+    __syncthreads();
+    ks = red_k[0] + red_k[1] + red_k[2] + red_k[3];
+    ne = red_n[0] + red_n[1] + red_n[2] + red_n[3];
+    const int my_ks = kspace_steps(rows);
+    if (tid == 0) {
+        kt0[g] = ks;
+        if (g == G - 1) {
+            kt0[G] = ks + my_ks;
+            const int ne_all = ne + (rows > 0 ? 1 : 0);
+            tile_meta[G + 5] = ne_all * (M2 / 256) * NT2;
+            tile_meta[G + 6] = ne_all * (M13 / 256) * NT13;
+        }
+    }
+    if (rows <= 0) return;
+    for (int pass = 0; pass < 2; ++pass) {
+        omega_tile_desc *desc = pass == 0 ? desc_w2 : desc_w13;
+        const int M = pass == 0 ? M2 : M13, MT = M / 256, NT = pass == 0 ? NT2 : NT13;
+        for (int l = tid; l < MT * NT; l += 256) {
+            const int mi = l % MT, n = l / MT;
+            omega_tile_desc dsc;
+            dsc.g = g;
+            dsc.row0 = g * M + mi * 256;
+            dsc.rows = 256;
+            dsc.xrow0 = my_ks;
+            dsc.n0 = n * 256;
+            dsc.a_rg = mi * 2;
+            dsc.b_rg = n * 2;
+            dsc.kt0 = ks;
+            desc[(size_t)ne * MT * NT + l] = dsc;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void bw_sched_kernel(sched_args sa) { schedule_queues(sa, blockIdx.x); }
+
+hipError_t launch_backward_tables(const omega_moe *m, int T, hipStream_t s)
+{
+    const omega_moe_config &c = m->cfg;
+    const int G = c.E + c.Es;
+    hipLaunchKernelGGL(bw_tables_kernel, dim3(G), dim3(256), 0, s, m->tile_meta, m->counts, c.E, c.Es, T, m->bm, m->desc_da,
+                       ceil_div(c.H, 256), m->bw_kt0, m->desc_w2, c.d, ceil_div(c.H, 256), m->desc_w13, 2 * c.H, c.d / 256);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    sched_args sa = {{m->desc_da, m->desc_w2, m->desc_w13}, {m->wq_da, m->wq_w2, m->wq_w13}, {G + 4, G + 5, G + 6}, {0, 1, 1},
+                     m->tile_meta, m->n_wg};
+    hipLaunchKernelGGL(bw_sched_kernel, dim3(24), dim3(256), 0, s, sa);
+    return hipGetLastError();
+}
+
+// ---- transposed packed images ----
+// dst[c][32*k0 + (r - r0)] = src[r][c] for the rows r0 .. r0+nr-1 of a source image (KTs k steps wide, all its
+// 32*KTs columns), zero for the next rows up to the end of the range's 32*ksteps places.  One workgroup moves
+// 64 rows x 64 columns through LDS.  by_group != 0: the row ranges are the experts' (grid.y covers k space, the
+// workgroup looks its group up in kt0; r0 = first physical row of the group, or row 0 of src_alt for a shared expert
+// when src_alt is given); by_group == 0: one range (r0 = 0, nr rows, k0) per z, images src + z*src_stride ->
+// dst + z*dst_stride.
+__global__ __launch_bounds__(256) void transpose_packed_kernel(const unsigned char *__restrict__ src,
+                                                               const unsigned char *__restrict__ src_alt, int KTs,
+                                                               unsigned char *__restrict__ dst, int KTd, int by_group,
+                                                               const int32_t *__restrict__ kt0,
+                                                               const int32_t *__restrict__ tile_meta,
+                                                               const int32_t *__restrict__ counts, int E, int G, int T, int bm,
+                                                               int nr_single, int k0_single, size_t src_stride, size_t dst_stride)
+{
+    __shared__ uint16_t tile[64][64 + 8];
+    const int tid = threadIdx.x;
+    const int c0 = blockIdx.x * 64;  // source columns = destination rows
+    int r0, nr, kd0, rb;             // rb: first row of this workgroup within the range
+    const unsigned char *sp = src;
+    if (by_group) {
+        const int kb = blockIdx.y * 2;  // first k step of this workgroup
+        if (kb >= kt0[G]) return;
+        int lo = 0, hi = G;             // last group with kt0[g] <= kb (empty groups share their successor's kt0)
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (kt0[mid] <= kb) lo = mid; else hi = mid;
+        }
+        int g = lo;
+        while (g + 1 < G && kt0[g + 1] <= kb) ++g;
+        nr = g < E ? counts[g] : T;
+        r0 = tile_meta[1 + g] * bm;
+        if (g >= E && src_alt != nullptr) { sp = src_alt; r0 = 0; }
+        kd0 = kb;
+        rb = (kb - kt0[g]) * 32;
+    } else {
+        sp = src + blockIdx.z * src_stride;
+        dst += blockIdx.z * dst_stride;
+        r0 = 0;
+        nr = nr_single;
+        rb = blockIdx.y * 64;
+        if (rb >= nr) return;
+        kd0 = k0_single + blockIdx.y * 2;
+    }
+    // load: 64 rows x 8 chunks of 8 columns
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int idx = tid + u * 256;
+        const int rr = idx >> 3, ch = idx & 7;
+        uint4 v = {0u, 0u, 0u, 0u};
+        if (rb + rr < nr) {
+            const int c = c0 + ch * 8;
+            v = *(const uint4 *)(sp + pk_chunk_off(r0 + rb + rr, c >> 5, (c & 31) >> 3, KTs));
+        }
+        *(uint4 *)&tile[rr][ch * 8] = v;
+    }
+    __syncthreads();
+    // store: 64 destination rows x 8 chunks of 8 k places
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int idx = tid + u * 256;
+        const int cc = idx & 63, kc = idx >> 6;  // destination row c0 + cc, k places kc*8 .. kc*8+7 of the 64
+        uint16_t e[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) e[q] = tile[kc * 8 + q][cc];
+        uint4 v;
+        v.x = e[0] | ((uint32_t)e[1] << 16);
+        v.y = e[2] | ((uint32_t)e[3] << 16);
+        v.z = e[4] | ((uint32_t)e[5] << 16);
+        v.w = e[6] | ((uint32_t)e[7] << 16);
+        *(uint4 *)(dst + pk_chunk_off(c0 + cc, kd0 + (kc >> 2), kc & 3, KTd)) = v;
+    }
+}
+
+// activations: rows of the experts -> k space (ksteps_cap = k steps the destination image is laid out for)
+hipError_t launch_transpose_groups(const omega_moe *m, const void *src, const void *src_alt, int cols, void *dst, int T,
+                                   hipStream_t s)
+{
+    const omega_moe_config &c = m->cfg;
+    hipLaunchKernelGGL(transpose_packed_kernel, dim3(cols / 64, m->bw_ksteps_cap / 2), dim3(256), 0, s,
+                       (const unsigned char *)src, (const unsigned char *)src_alt, cols / 32, (unsigned char *)dst,
+                       m->bw_ksteps_cap, 1, m->bw_kt0, m->tile_meta, m->counts, c.E, c.E + c.Es, T, m->bm, 0, 0, (size_t)0,
+                       (size_t)0);
+    return hipGetLastError();
+}
+
+// weights: n images of R rows x cols columns -> images of cols rows, written at k step k0 of KTd
+hipError_t launch_transpose_images(const void *src, int R, int cols, void *dst, int KTd, int k0, int n, size_t src_stride,
+                                   size_t dst_stride, hipStream_t s)
+{
+    hipLaunchKernelGGL(transpose_packed_kernel, dim3(cols / 64, R / 64, n), dim3(256), 0, s, (const unsigned char *)src,
+                       (const unsigned char *)nullptr, cols / 32, (unsigned char *)dst, KTd, 0, (const int32_t *)nullptr,
+                       (const int32_t *)nullptr, (const int32_t *)nullptr, 0, 0, 0, 0, R, k0, src_stride, dst_stride);
     return hipGetLastError();
 }

@@ -28,8 +28,25 @@
 // tiles in its L2, and so that all queues hold the same amount of work.  The ring of LDS stages runs on from one
 // item to the next: the last steps of an item already fetch the first steps of the next, so a workgroup pays
 // the load latency once per launch, not once per tile.
+//
+// The backward pass of bf16 layers runs on the same kernel (MODE below): every product of it is brought into the
+// "both operands K-contiguous" form by keeping transposed packed copies of the weights and by transposing the
+// activations for the weight gradients, so the matrix-core pipeline is the one above and only the epilogues differ.
 #include "common.h"
 #include "pack.h"
+
+// What one instantiation of the product kernel computes (tile shape, operand order, epilogue):
+//   UP     tile 256 x (128 of Wa + 128 of Wb), silu(h1)*h3 -> packed bf16 a
+//   DOWN   tile 256 x 256, fp32 row-major output
+//   UPRAW  as UP, but h1 and h3 are stored as they sit in the accumulators (Cout = h1, Aux1 = h3): one 4 KiB record
+//          per 32x32 MFMA block, [row block][column block][register 0..15][lane 0..63]
+//   DA     tile 256 x 256 of d(a) = dy . W2 (B = packed W2^T); the epilogue reads the h1/h3 records of its blocks
+//          (Aux1, Aux2), applies the SwiGLU backward and writes dh1 | dh3 as one packed bf16 image with 2N columns
+//   WGRAD  tile 256 x 256 of dW = A^T . B over the rows of one expert: both operands are transposed packed images
+//          whose K axis is the experts' rows; the item names its operand row groups, first k step and k steps
+//          (a_rg, b_rg, kt0, xrow0); fp32 row-major output, row0 = expert * M + first row
+#define FUSED_TILE(M) ((M) == MODE_UP || (M) == MODE_UPRAW)
+#define SWAPPED(M) ((M) != MODE_DOWN && (M) != MODE_WGRAD)
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -71,6 +88,7 @@ struct TileCtx {
     const unsigned char *A, *B0, *B1;
     uint32_t a_off0, a_off1;  // this lane's byte offsets of its two A blocks within a k step
     int row0, rows, n0;
+    int kt;                   // k steps of the item
 };
 
 __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char *p)
@@ -80,18 +98,31 @@ __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char 
     return (const unsigned char *)(((uint64_t)hi << 32) | lo);
 }
 
-template <bool FUSED>
+template <int MODE>
 __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa,
                                             const bf16_t *Wb, int N, int Kd, int wave, int lane)
 {
+    constexpr bool FUSED = FUSED_TILE(MODE);
     TileCtx c;
     const int KT = Kd / BK;
     const size_t rg_bytes = (size_t)KT * 8192;  // a packed row group (128 rows) occupies KT * 8 KiB
     c.row0 = d.row0;
     c.rows = d.rows;
     c.n0 = d.n0;
-    c.A = uniform_ptr((FUSED && d.xrow0 >= 0) ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
-                                              : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes);
+    if (MODE == MODE_WGRAD) {
+        const size_t k0 = (size_t)d.kt0 * 8192;
+        c.kt = d.xrow0;
+        c.A = uniform_ptr((const unsigned char *)Axg + (size_t)d.a_rg * rg_bytes + k0);
+        c.B0 = uniform_ptr((const unsigned char *)Wa + (size_t)d.b_rg * rg_bytes + k0);
+        c.B1 = uniform_ptr(c.B0 + rg_bytes);
+        c.a_off0 = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
+        c.a_off1 = (uint32_t)KT * 8192u + c.a_off0;
+        return c;
+    }
+    c.kt = KT;
+    c.A = uniform_ptr((MODE != MODE_DOWN && Ax != nullptr && d.xrow0 >= 0)
+                          ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
+                          : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes);
     const size_t wrg = (size_t)d.g * (N >> 7) + (d.n0 >> 7);  // row group of the weight tile
     c.B0 = uniform_ptr((const unsigned char *)Wa + wrg * rg_bytes);
     c.B1 = uniform_ptr(FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : c.B0 + rg_bytes);
@@ -125,11 +156,12 @@ __device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, 
 // visible has been passed.  The last NSTAGE steps issue the first loads of the next item (dn, if it has rows)
 // instead of their own, so the matrix cores of the next item start on data that travelled during this item's
 // epilogue.
-template <bool FUSED, int NBLK>
+template <int MODE, int NBLK>
 __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_in, TileCtx &nx, const omega_tile_desc &dn,
                                          const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa, const bf16_t *Wb, int &cur_io,
-                                         void *Cout, int N, int Kd, int wave, int lane)
+                                         void *Cout, void *Aux1, void *Aux2, int N, int Kd, int wave, int lane)
 {
+    constexpr bool FUSED = FUSED_TILE(MODE), SWAP = SWAPPED(MODE);
     constexpr int NB = NBLK > 0 ? NBLK : 1;
     // the item's uniform fields and the ring position live in scalar registers for the whole item (the direct loads
     // take their base address and LDS address from scalar operands)
@@ -145,7 +177,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     const uint32_t lds_wave = lds0 + wave * 1024;
     const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
-    const int KT = Kd / BK;
+    const int KT = MODE == MODE_WGRAD ? __builtin_amdgcn_readfirstlane(ctx_in.kt) : Kd / BK;
     const bool has_next = dn.rows > 0;
 
 // load n of virtual k step v: steps beyond this item's last belong to the next item
@@ -187,8 +219,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     do {                                                                                                    \
         if ((i) < NBLK) {                                                                                   \
             _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                    \
-                acc[i][j] = FUSED ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(BF[j], AF[i], acc[i][j], 0, 0, 0) \
-                                  : __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0); \
+                acc[i][j] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(BF[j], AF[i], acc[i][j], 0, 0, 0) \
+                                 : __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0); \
         }                                                                                                   \
     } while (0)
 
@@ -242,13 +274,13 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 
     int kt = 0;
     for (; kt < KT - NSTAGE; ++kt) K_STEP(false);
-    nx = make_ctx<FUSED>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
+    nx = make_ctx<MODE>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
     for (; kt < KT; ++kt) K_STEP(true);
 #undef K_STEP
     cur_io = cur;
 
     // ---- epilogue ----
-    if (FUSED) {
+    if (MODE == MODE_UP) {
         // lane: row l32 of block i; register r -> column 8*(r/4) + 4*lhi + r%4 of the wave's 32 columns, which are
         // one k step of the packed `a` (K dimension = N): chunk r/4, bytes lhi*8 .. lhi*8+7
         const int KTa = N / BK;
@@ -276,6 +308,56 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
                 }
             }
         }
+    } else if (MODE == MODE_UPRAW) {
+        // the accumulators as they are, one record per 32x32 block (whole blocks: rows past the item's last are
+        // never read back as valid)
+        const size_t cb = (size_t)(ctx.n0 >> 5) + wn, ncb = (size_t)(N >> 5);
+#pragma unroll
+        for (int i = 0; i < NBLK; ++i) {
+            const size_t rb = (size_t)(ctx.row0 >> 5) + 2 * i + wm;
+            float *o1 = (float *)Cout + (rb * ncb + cb) * 1024 + lane, *o3 = (float *)Aux1 + (rb * ncb + cb) * 1024 + lane;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                o1[r * 64] = acc[i][0][r];
+                o3[r * 64] = acc[i][1][r];
+            }
+        }
+    } else if (MODE == MODE_DA) {
+        // acc = d(a) of (row l32 of block i, columns 8*(r/4) + 4*lhi + r%4 of column block j); h1, h3 of the same
+        // elements come from their records.  dh3 = da * silu(h1); dh1 = da*h3 * s*(1 + h1*(1-s)), s = sigmoid(h1)
+        // (silu_backward, J/engine/nn/layer/active/gpu/activeFunction.cu:182-190).  Output: packed image with 2N
+        // columns, dh1 in k steps 0..N/32-1, dh3 behind them.
+        const int ncb = N >> 5, KTa = 2 * ncb;
+#pragma unroll
+        for (int i = 0; i < NBLK; ++i) {
+            const int row = (2 * i + wm) * 32 + l32;
+            const size_t rb = (size_t)(ctx.row0 >> 5) + 2 * i + wm;
+            const int prow = ctx.row0 + row;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int cb = (ctx.n0 >> 5) + wn * 2 + j;
+                if (cb >= ncb) continue;  // last column tile of a width that is not a multiple of 256
+                const float *p1 = (const float *)Aux1 + (rb * ncb + cb) * 1024 + lane;
+                const float *p3 = (const float *)Aux2 + (rb * ncb + cb) * 1024 + lane;
+                float g1[16], g3[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float h1 = p1[r * 64], h3 = p3[r * 64], da = acc[i][j][r];
+                    const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-h1));
+                    g3[r] = da * (h1 * sg);
+                    g1[r] = (da * h3) * sg * (1.0f + h1 * (1.0f - sg));
+                }
+                if (row < ctx.rows) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const uint2 o1 = {pack_bf16x2(g1[t * 4], g1[t * 4 + 1]), pack_bf16x2(g1[t * 4 + 2], g1[t * 4 + 3])};
+                        const uint2 o3 = {pack_bf16x2(g3[t * 4], g3[t * 4 + 1]), pack_bf16x2(g3[t * 4 + 2], g3[t * 4 + 3])};
+                        *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, cb, t, KTa) + lhi * 8) = o1;
+                        *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, ncb + cb, t, KTa) + lhi * 8) = o3;
+                    }
+                }
+            }
+        }
     } else {
         // lane: column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4
 #pragma unroll
@@ -288,7 +370,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
                 //  write 32-byte pieces of 32 different lines and were 8 % slower on short-K shapes)
                 float *out = (float *)Cout + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l32;
 #pragma unroll
-                for (int j = 0; j < 2; ++j) out[j * 32] = acc[i][j][r];
+                for (int j = 0; j < 2; ++j)
+                    if (MODE == MODE_DOWN || ctx.n0 + wn * 64 + j * 32 < N) out[j * 32] = acc[i][j][r];
             }
         }
     }
@@ -298,11 +381,11 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 }
 
 // Persistent: one workgroup per compute unit walks its queue of work items (built by the dispatch stage).
-template <bool FUSED>
+template <int MODE>
 __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
                                                                    const bf16_t *__restrict__ Wa, const bf16_t *__restrict__ Wb,
-                                                                   void *__restrict__ Cout, const omega_tile_desc *__restrict__ wq,
-                                                                   int N, int Kd)
+                                                                   void *__restrict__ Cout, void *Aux1, void *Aux2,
+                                                                   const omega_tile_desc *__restrict__ wq, int N, int Kd)
 {
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -311,7 +394,7 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
 
     omega_tile_desc d = wq[wg];
     if (d.rows <= 0) return;
-    TileCtx cur_ctx = make_ctx<FUSED>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
+    TileCtx cur_ctx = make_ctx<MODE>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
     {
         // first item: k steps 0..NSTAGE-2 and the first half of step NSTAGE-1 into stages 0..NSTAGE-1
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -332,13 +415,16 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
         const omega_tile_desc dn = wq[(size_t)q * n_wg + wg];
         // 32-row blocks alternate between the two row halves of the workgroup: block b belongs to waves with wm = b % 2
         const int nblk = max(0, min(4, (((cur_ctx.rows + 31) >> 5) + 1 - (wave >> 2)) >> 1));
+#define RUN_TILE(NBLK) \
+    run_tile<MODE, NBLK>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, Aux1, Aux2, N, Kd, wave, lane)
         switch (nblk) {
-            case 4: run_tile<FUSED, 4>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
-            case 3: run_tile<FUSED, 3>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
-            case 2: run_tile<FUSED, 2>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
-            case 1: run_tile<FUSED, 1>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
-            default: run_tile<FUSED, 0>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, N, Kd, wave, lane); break;
+            case 4: RUN_TILE(4); break;
+            case 3: RUN_TILE(3); break;
+            case 2: RUN_TILE(2); break;
+            case 1: RUN_TILE(1); break;
+            default: RUN_TILE(0); break;
         }
+#undef RUN_TILE
         if (dn.rows <= 0) break;
         cur_ctx = nx;
     }
@@ -346,11 +432,14 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
 
 hipError_t experts_bf16_init(void)
 {
-    hipError_t e = hipFuncSetAttribute((const void *)experts_bf16_kernel<true>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-    if (e != hipSuccess) return e;
-    return hipFuncSetAttribute((const void *)experts_bf16_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                               SMEM_BYTES);
+    const void *fns[] = {(const void *)experts_bf16_kernel<MODE_UP>, (const void *)experts_bf16_kernel<MODE_DOWN>,
+                         (const void *)experts_bf16_kernel<MODE_UPRAW>, (const void *)experts_bf16_kernel<MODE_DA>,
+                         (const void *)experts_bf16_kernel<MODE_WGRAD>};
+    for (const void *f : fns) {
+        hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s)
@@ -361,12 +450,33 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
     // the ring must be shorter than an item: K >= (NSTAGE + 1) * BK (guaranteed at creation: d, H >= 256)
     if ((which == 0 ? c.d : c.H) < (NSTAGE + 1) * BK) return hipErrorInvalidValue;
     if (which == 0) {
-        hipLaunchKernelGGL(experts_bf16_kernel<true>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
-                           (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, m->wq_up, c.H, c.d);
+        hipLaunchKernelGGL(experts_bf16_kernel<MODE_UP>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
+                           (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
+                           (void *)nullptr, m->wq_up, c.H, c.d);
     } else {
-        hipLaunchKernelGGL(experts_bf16_kernel<false>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
-                           (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y, m->wq_down,
-                           c.d, c.H);
+        hipLaunchKernelGGL(experts_bf16_kernel<MODE_DOWN>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
+                           (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y,
+                           (void *)nullptr, (void *)nullptr, m->wq_down, c.d, c.H);
     }
+    return hipGetLastError();
+}
+
+// One product of the backward pass on the same kernel; `mode` as the enum above, operands and outputs as its comment says.
+hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, const void *Aalt, const void *Wa, const void *Wb,
+                               void *Cout, void *Aux1, void *Aux2, const omega_tile_desc *wq, int N, int Kd, hipStream_t s)
+{
+    if (Kd < (NSTAGE + 1) * BK) return hipErrorInvalidValue;
+#define LAUNCH(MODE)                                                                                                   \
+    hipLaunchKernelGGL(experts_bf16_kernel<MODE>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)A,      \
+                       (const bf16_t *)Aalt, (const bf16_t *)Wa, (const bf16_t *)Wb, Cout, Aux1, Aux2, wq, N, Kd)
+    switch (mode) {
+        case MODE_UP: LAUNCH(MODE_UP); break;
+        case MODE_DOWN: LAUNCH(MODE_DOWN); break;
+        case MODE_UPRAW: LAUNCH(MODE_UPRAW); break;
+        case MODE_DA: LAUNCH(MODE_DA); break;
+        case MODE_WGRAD: LAUNCH(MODE_WGRAD); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef LAUNCH
     return hipGetLastError();
 }

@@ -98,3 +98,41 @@ def test_acc_grad_and_update_fp32():
     layer.update(1.0)
     assert N.rel_l2(layer._download_weight(L.W_W1, 1, (cfg.H, cfg.d)), after["W1"].astype(np.float64) - gW) < 1e-6
     layer.close()
+
+
+CASES_BF16 = [
+    ("c2_mixtral", dict(T=300, d=256, H=384)),                          # H = 128 mod 256: ragged last column tile
+    ("c4_finegrained", dict(T=200, d=256, H=256, E=16, K=4, Es=2)),     # experts far below one k-space minimum, shared experts
+    ("c5_skewed", dict(T=257, d=512, H=256, E=32, K=4)),                # gate bias, experts without rows
+    ("c2_mixtral", dict(T=1200, d=256, H=512, E=4, K=2)),               # several row tiles per expert
+    ("c2_mixtral", dict(T=1, d=256, H=256, E=8, K=2)),
+]
+
+
+@pytest.mark.parametrize("name,kw", CASES_BF16)
+def test_backward_bf16_matches_oracle(name, kw):
+    G, cfg, inp, dout, layer = _setup(name, kw, 47)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = G.P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    out = layer.forward(x).to_numpy()
+    dx = layer.back(g).to_numpy()
+    ref = O.moe_backward(inp["x"], dout, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es,
+                         bf16=True)
+    assert N.rel_l2(dx, ref["dx"]) < 1e-2, N.rel_l2(dx, ref["dx"])
+    _check_grads(layer, cfg, ref, 1e-2)
+    # forward output and routing untouched; a second backward gives the same bits; a forward after it still matches
+    assert np.array_equal(layer.getOutput().to_numpy(), out)
+    w2 = layer.grad(L.W_W2, 0)
+    assert np.array_equal(layer.back(g).to_numpy(), dx)
+    assert np.array_equal(layer.grad(L.W_W2, 0), w2)
+    assert np.array_equal(layer.forward(x).to_numpy(), out)
+    # new weights invalidate the transposed copies the pass keeps: gradients follow the new weights
+    W2n = O.round_bf16(inp["W2"][0] * np.float32(0.5))
+    layer.set_expert(0, inp["W1"][0], inp["W3"][0], W2n)
+    inp["W2"][0] = W2n
+    layer.forward(x)
+    dx2 = layer.back(g).to_numpy()
+    ref2 = O.moe_backward(inp["x"], dout, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es,
+                          bf16=True)
+    assert N.rel_l2(dx2, ref2["dx"]) < 1e-2
+    layer.close()
