@@ -181,7 +181,8 @@ int omega_moe_get_routing(omega_moe *moe, int T, int32_t *ids, float *w, int32_t
 int omega_moe_get_router_probs(omega_moe *moe, const void *x_dev, int T, float *logits, float *probs);
 /* Host copy (blocking) of a workspace buffer of the last call, rows in logical order (row dst[p] of pair p,
  * then T rows per shared expert), row-major: which = 0 xg [T*K,d] (layer dtype), 1 a [T*K+Es*T,H] (layer
- * dtype), 2 y [T*K+Es*T,d] fp32.  For tests. */
+ * dtype), 2 y [T*K+Es*T,d] fp32; after omega_moe_backward of a bf16 layer also 3 dh1|dh3 [T*K+Es*T,2H] bf16, and for
+ * any layer 4 dlogits [T,E] fp32.  For tests. */
 int omega_moe_get_workspace(omega_moe *moe, int which, int T, void *host_dst);
 
 /* Average duration in milliseconds of the launches of one stage, measured with events on the
@@ -191,6 +192,11 @@ int omega_moe_get_workspace(omega_moe *moe, int which, int T, void *host_dst);
  * x_dev/out_dev as for forward; the stages before `stage` must have been run for this T. */
 int omega_moe_time_stage(omega_moe *moe, int stage, const void *x_dev, int T, void *out_dev, int warmup, int iters,
                          float *ms_avg);
+
+/* Average duration in milliseconds of omega_moe_backward, measured like omega_moe_time_stage; the forward pass for
+ * x_dev and T must have run. */
+int omega_moe_time_backward(omega_moe *moe, const void *x_dev, const void *dout_dev, int T, void *dx_dev, int warmup,
+                            int iters, float *ms_avg);
 
 /* Measurement aid, no counterpart in the reference: the bf16 matrix-core rate the device sustains with no memory
  * traffic at all (a loop of independent MFMAs on every SIMD, `launches` launches of about 2.5 ms, the first

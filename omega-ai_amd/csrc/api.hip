@@ -154,7 +154,7 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 
 static void moe_free_backward_workspace(omega_moe *m)
 {
-    void **bw[] = {(void **)&m->bw_probs, (void **)&m->bw_dw, (void **)&m->bw_dlogits, (void **)&m->bw_dy, (void **)&m->bw_h1,
+    void **bw[] = {(void **)&m->bw_probs, (void **)&m->bw_dw, (void **)&m->bw_dlogits, (void **)&m->bw_gpart, (void **)&m->bw_dy, (void **)&m->bw_h1,
                    (void **)&m->bw_h3, (void **)&m->bw_dxg, &m->bw_dy16, &m->bw_dys16, &m->bw_dh16, &m->bw_dyT, &m->bw_aT,
                    &m->bw_xgT, &m->bw_dhT, (void **)&m->bw_kt0, (void **)&m->desc_da, (void **)&m->wq_da,
                    (void **)&m->desc_w2, (void **)&m->wq_w2, (void **)&m->desc_w13, (void **)&m->wq_w13};
@@ -225,6 +225,7 @@ static int moe_reserve_backward(omega_moe *m, int T)
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_probs, (size_t)Tc * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dw, (size_t)Tc * c.K * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dlogits, (size_t)Tc * c.E * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_gpart, (size_t)32 * c.E * c.d * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h1, rc * c.H * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h3, rc * c.H * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dxg, rc * c.d * 4));
@@ -623,6 +624,26 @@ int omega_moe_backward(omega_moe *m, const void *x, const void *dout, int T, voi
     return OMEGA_OK;
 }
 
+int omega_moe_time_backward(omega_moe *m, const void *x, const void *dout, int T, void *dx, int warmup, int iters, float *ms_avg)
+{
+    MOE_ENTER(m);
+    RUN(check_T(m, x, T, true));
+    if (T <= 0 || T != m->fwd_T) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_backward: no omega_moe_forward has run for this T");
+    if (!dout || !dx || !ms_avg || iters <= 0 || warmup < 0) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_backward: bad argument");
+    RUN(moe_reserve_backward(m, T));
+    const bool bf = m->cfg.dtype == OMEGA_DTYPE_BF16;
+    for (int i = 0; i < warmup + iters; ++i) {
+        if (i == warmup) OMEGA_HIP_CHECK(ctx, hipEventRecord(m->ev0, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, bf ? launch_backward_bf16(m, x, dout, T, dx, ctx->stream) : launch_backward_f32(m, x, dout, T, dx, ctx->stream));
+    }
+    OMEGA_HIP_CHECK(ctx, hipEventRecord(m->ev1, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipEventSynchronize(m->ev1));
+    float ms = 0.0f;
+    OMEGA_HIP_CHECK(ctx, hipEventElapsedTime(&ms, m->ev0, m->ev1));
+    *ms_avg = ms / (float)iters;
+    return OMEGA_OK;
+}
+
 static int grad_slot(omega_moe *m, int which, int expert, float **ptr, size_t *floats)
 {
     const omega_moe_config &c = m->cfg;
@@ -817,14 +838,21 @@ int omega_moe_get_router_probs(omega_moe *m, const void *x, int T, float *logits
 int omega_moe_get_workspace(omega_moe *m, int which, int T, void *host_dst)
 {
     MOE_ENTER(m);
-    if (!host_dst || which < 0 || which > 2 || T <= 0 || T > m->T_cap || m->bm == 0)
+    if (!host_dst || which < 0 || which > 4 || T <= 0 || T > m->T_cap || m->bm == 0)
         OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_workspace: bad selector, T, or no dispatch has run");
     const omega_moe_config &c = m->cfg;
+    if (which >= 3 && (T > m->bw_T_cap || (which == 3 && !m->bw_dh16)))
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_workspace: no backward has run (selector 3: of a bf16 layer)");
+    if (which == 4) {
+        OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(host_dst, m->bw_dlogits, (size_t)T * c.E * 4, hipMemcpyDeviceToHost, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+        return OMEGA_OK;
+    }
     const int G = c.E + c.Es, bm = m->bm;
-    const int cols = which == 1 ? c.H : c.d;
+    const int cols = which == 1 ? c.H : which == 3 ? 2 * c.H : c.d;
     const size_t es = which == 2 ? 4 : m->esize;
     const bool packed = c.dtype == OMEGA_DTYPE_BF16 && which != 2;
-    const void *src = which == 0 ? m->xg : which == 1 ? m->a : (const void *)m->y;
+    const void *src = which == 0 ? m->xg : which == 1 ? m->a : which == 3 ? m->bw_dh16 : (const void *)m->y;
     const size_t bytes = m->rows_cap * cols * es;
     std::vector<int32_t> meta(G + 2), off(c.E + 1);
     OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(meta.data(), m->tile_meta, meta.size() * 4, hipMemcpyDeviceToHost, ctx->stream));

@@ -138,8 +138,7 @@ __global__ __launch_bounds__(256) void bw_rows_f32_kernel(const float *__restric
 // without rows gets zeros.  grid (ceil(N/64), ceil(M/64), groups).  Rows of group g: physical rows from
 // tile_meta[1+g]*bm, counts[g] of them for a routed expert, T for a shared one; a shared group reads token rows
 // 0..T-1 of Atok / Btok when those are given.  single_rows >= 0: one group, rows 0..single_rows-1 of Aphys / Bphys.
-// gstride: floats between the outputs of consecutive groups.  BBF: B holds bf16 (single-group use only).
-template <bool BBF>
+// gstride: floats between the outputs of consecutive groups.
 __global__ __launch_bounds__(256) void bw_wgrad_f32_kernel(const float *__restrict__ Aphys, const float *__restrict__ Atok,
                                                            const float *__restrict__ Bphys, const float *__restrict__ Btok,
                                                            float *__restrict__ dW, size_t gstride,
@@ -166,9 +165,7 @@ __global__ __launch_bounds__(256) void bw_wgrad_f32_kernel(const float *__restri
             const int rr = idx / GBM, cc = idx % GBM;
             const int r = r0 + rr;
             As[rr][cc] = (r < rows && m0 + cc < M) ? A[(size_t)r * M + m0 + cc] : 0.0f;
-            Bs[rr][cc] = (r < rows && n0 + cc < N)
-                             ? (BBF ? bf16_to_f32(((const bf16_t *)B)[(size_t)r * N + n0 + cc]) : B[(size_t)r * N + n0 + cc])
-                             : 0.0f;
+            Bs[rr][cc] = (r < rows && n0 + cc < N) ? B[(size_t)r * N + n0 + cc] : 0.0f;
         }
         __syncthreads();
 #pragma unroll
@@ -228,6 +225,71 @@ __global__ __launch_bounds__(256) void bw_router_kernel(const float *__restrict_
         if (renorm) g = (g - dot) / S;
         dl[id[j]] = (g - sum) * p[id[j]];
     }
+}
+
+// Gate weight gradient dWg[e,k] = sum_t dlogits[t,e] * x[t,k] (diffW = delta^T . input) in two steps, both with a fixed
+// order of additions: partial sums over slices of the tokens, then their sum.  Workgroup (column chunk of 256, token
+// slice, expert chunk of 32): a thread owns one column and up to 32 experts; the slice's dlogits pass through LDS.
+#define GW_EC 32
+template <bool XBF>
+__global__ __launch_bounds__(256) void bw_gate_partial_kernel(const float *__restrict__ dlogits, const void *__restrict__ x,
+                                                              int T, int d, int E, int tslice, float *__restrict__ part)
+{
+    __shared__ float dl[64][GW_EC];
+    const int k = blockIdx.x * 256 + threadIdx.x, e0 = blockIdx.z * GW_EC;
+    const int t0 = blockIdx.y * tslice, t1 = min(T, t0 + tslice);
+    float acc[GW_EC];
+#pragma unroll
+    for (int e = 0; e < GW_EC; ++e) acc[e] = 0.0f;
+    for (int tb = t0; tb < t1; tb += 64) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < 64 * GW_EC; i += 256) {
+            const int tt = tb + i / GW_EC, e = e0 + i % GW_EC;
+            dl[i / GW_EC][i % GW_EC] = (tt < t1 && e < E) ? dlogits[(size_t)tt * E + e] : 0.0f;
+        }
+        __syncthreads();
+        if (k < d) {
+            const int n = min(64, t1 - tb);
+            for (int tt = 0; tt < n; ++tt) {
+                const float xv = XBF ? bf16_to_f32(((const bf16_t *)x)[(size_t)(tb + tt) * d + k])
+                                     : ((const float *)x)[(size_t)(tb + tt) * d + k];
+#pragma unroll
+                for (int e = 0; e < GW_EC; ++e) acc[e] = fmaf(dl[tt][e], xv, acc[e]);
+            }
+        }
+    }
+    if (k < d)
+#pragma unroll
+        for (int e = 0; e < GW_EC; ++e)
+            if (e0 + e < E) part[((size_t)blockIdx.y * E + e0 + e) * d + k] = acc[e];
+}
+
+__global__ __launch_bounds__(256) void bw_gate_reduce_kernel(const float *__restrict__ part, int nslices, size_t n,
+                                                             float *__restrict__ dWg)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.0f;
+    for (int q = 0; q < nslices; ++q) s += part[(size_t)q * n + i];
+    dWg[i] = s;
+}
+
+#define GW_SLICES 32
+static hipError_t launch_gate_wgrad(const omega_moe *m, const void *x, int T, hipStream_t s)
+{
+    const omega_moe_config &c = m->cfg;
+    const int tslice = ceil_div(ceil_div(T, GW_SLICES), 64) * 64, nsl = ceil_div(T, tslice);
+    const dim3 grid(ceil_div(c.d, 256), nsl, ceil_div(c.E, GW_EC));
+    if (c.dtype == OMEGA_DTYPE_BF16)
+        hipLaunchKernelGGL(bw_gate_partial_kernel<true>, grid, dim3(256), 0, s, (const float *)m->bw_dlogits, x, T, c.d, c.E,
+                           tslice, m->bw_gpart);
+    else
+        hipLaunchKernelGGL(bw_gate_partial_kernel<false>, grid, dim3(256), 0, s, (const float *)m->bw_dlogits, x, T, c.d, c.E,
+                           tslice, m->bw_gpart);
+    const size_t n = (size_t)c.E * c.d;
+    hipLaunchKernelGGL(bw_gate_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const float *)m->bw_gpart, nsl,
+                       n, m->dWg);
+    return hipGetLastError();
 }
 
 // dbg[e] = sum_t dlogits[t,e]: one workgroup per expert.
@@ -307,21 +369,19 @@ hipError_t launch_backward_f32(const omega_moe *m, const void *xv, const void *d
                        W3, m->bw_dxg, (float *)nullptr, m->tiles, m->tile_meta, c.d, c.H);
     // weight gradients: dW2 = dy^T a [d,H]; dW1 = dh1^T xg, dW3 = dh3^T xg [H,d]
     const size_t HD = (size_t)c.H * c.d;
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel<false>, dim3(ceil_div(c.H, GBN), ceil_div(c.d, GBM), G), dim3(256), 0, s,
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.H, GBN), ceil_div(c.d, GBM), G), dim3(256), 0, s,
                        (const float *)m->bw_dy, dout, a, (const float *)nullptr, m->dW2, HD, m->tile_meta, m->counts, c.E, T,
                        m->bm, c.d, c.H, -1);
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel<false>, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
                        (const float *)m->bw_h1, (const float *)nullptr, xg, x, m->dW13, 2 * HD, m->tile_meta, m->counts, c.E,
                        T, m->bm, c.H, c.d, -1);
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel<false>, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
+    hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
                        (const float *)m->bw_h3, (const float *)nullptr, xg, x, m->dW13 + HD, 2 * HD, m->tile_meta, m->counts,
                        c.E, T, m->bm, c.H, c.d, -1);
     // router and gate
     hipLaunchKernelGGL(bw_router_kernel, dim3(ceil_div(T, 256)), dim3(256), 0, s, (const float *)m->bw_probs, m->ids, m->w,
                        (const float *)m->bw_dw, T, c.E, c.K, c.renorm, m->bw_dlogits);
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel<false>, dim3(ceil_div(c.d, GBN), ceil_div(c.E, GBM), 1), dim3(256), 0, s,
-                       (const float *)m->bw_dlogits, (const float *)nullptr, x, (const float *)nullptr, m->dWg, (size_t)0,
-                       m->tile_meta, m->counts, c.E, T, m->bm, c.E, c.d, T);
+    if ((e = launch_gate_wgrad(m, x, T, s)) != hipSuccess) return e;
     if (c.has_gate_bias)
         hipLaunchKernelGGL(bw_gate_bias_kernel, dim3(c.E), dim3(256), 0, s, (const float *)m->bw_dlogits, T, c.E, m->dbg);
     hipLaunchKernelGGL(bw_dx_kernel<false>, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,
@@ -414,9 +474,7 @@ hipError_t launch_backward_bf16(const omega_moe *m, const void *x, const void *d
     // router and gate
     hipLaunchKernelGGL(bw_router_kernel, dim3(ceil_div(T, 256)), dim3(256), 0, s, (const float *)m->bw_probs, m->ids, m->w,
                        (const float *)m->bw_dw, T, c.E, c.K, c.renorm, m->bw_dlogits);
-    hipLaunchKernelGGL(bw_wgrad_f32_kernel<true>, dim3(ceil_div(c.d, GBN), ceil_div(c.E, GBM), 1), dim3(256), 0, s,
-                       (const float *)m->bw_dlogits, (const float *)nullptr, (const float *)x, (const float *)nullptr, m->dWg,
-                       (size_t)0, m->tile_meta, m->counts, c.E, T, m->bm, c.E, c.d, T);
+    STEP(launch_gate_wgrad(m, x, T, s));
     if (c.has_gate_bias)
         hipLaunchKernelGGL(bw_gate_bias_kernel, dim3(c.E), dim3(256), 0, s, (const float *)m->bw_dlogits, T, c.E, m->dbg);
     hipLaunchKernelGGL(bw_dx_kernel<true>, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,

@@ -97,6 +97,7 @@ struct omega_moe {
     float *bw_probs = nullptr;       // [T,E] softmax of the gate logits
     float *bw_dw = nullptr;          // [T,K] gradient of the combine weights
     float *bw_dlogits = nullptr;     // [T,E]
+    float *bw_gpart = nullptr;       // [32][E,d] partial sums of the gate weight gradient over token slices
     float *bw_dy = nullptr;          // [rows_cap,d] gradient of the expert outputs
     float *bw_h1 = nullptr;          // [rows_cap,H] h1, then dh1
     float *bw_h3 = nullptr;          // [rows_cap,H] h3, then dh3

@@ -271,6 +271,11 @@ class MoELayer:
                                                      out.ptr if out is not None else None, warmup, iters, C.byref(ms)))
         return ms.value
 
+    def time_backward(self, x, dout, T, dx, warmup=2, iters=10):
+        ms = C.c_float()
+        self.ctx.check(self.lib.omega_moe_time_backward(self.handle, x.ptr, dout.ptr, T, dx.ptr, warmup, iters, C.byref(ms)))
+        return ms.value
+
     def set_profiling(self, on):
         self.ctx.check(self.lib.omega_moe_set_profiling(self.handle, int(on)))
 
@@ -299,11 +304,13 @@ class MoELayer:
 
     def workspace(self, which, T):
         """Host copy of a workspace buffer in logical row order: 'xg' [T*K,d], 'a' [T*K+Es*T,H],
-        'y' [T*K+Es*T,d] (fp32 values)."""
-        idx = {"xg": 0, "a": 1, "y": 2}[which]
+        'y' [T*K+Es*T,d] (fp32 values); after back() also 'dh' [T*K+Es*T,2H] (dh1 | dh3, bf16 layers) and
+        'dlogits' [T,E]."""
+        idx = {"xg": 0, "a": 1, "y": 2, "dh": 3, "dlogits": 4}[which]
         P, R = T * self.topK, T * self.topK + self.nShared * T
-        shape = {"xg": (P, self.embedDim), "a": (R, self.hidden), "y": (R, self.embedDim)}[which]
-        raw_bf16 = self.dtype == "bf16" and which != "y"
+        shape = {"xg": (P, self.embedDim), "a": (R, self.hidden), "y": (R, self.embedDim),
+                 "dh": (R, 2 * self.hidden), "dlogits": (T, self.nExperts)}[which]
+        raw_bf16 = self.dtype == "bf16" and which not in ("y", "dlogits")
         h = np.zeros(shape, np.uint16 if raw_bf16 else np.float32)
         self.ctx.check(self.lib.omega_moe_get_workspace(self.handle, idx, T, h.ctypes.data))
         return bf16_bits_to_f32(h) if raw_bf16 else h

@@ -22,6 +22,8 @@
  *   orc_moe_backward   torch float64 autograd of the dense formulation with the routing held fixed, and central
  *                      finite differences of an independent float64 NumPy forward (pinned to tolerance; the
  *                      summation order of the reference's cuBLAS products cannot be reproduced: bits "parity unpinned")
+ *   orc_moe_backward_routed   the same code path with the routing passed in: equals orc_moe_backward on the same tokens
+ *                      when given its routing (pinned by that identity)
  */
 #include <stdlib.h>
 
@@ -99,24 +101,22 @@ static void expert_backward(const float *xin, const float *dy, int rows, const f
     }
 }
 
-/* Whole backward pass.  x, dout: [T,d]; weights as in orc_moe_forward (W1,W3: [E+Es,H,d], W2: [E+Es,d,H]).
- * The forward quantities it needs are recomputed here.  Outputs (any may be NULL except dx): dx [T,d], dWg [E,d],
- * dbg [E], dW1,dW3 [E+Es,H,d], dW2 [E+Es,d,H], dw [T,K] (gradient of the combine weights), dlogits [T,E]. */
-void orc_moe_backward(const float *x, const float *dout, const float *Wg, const float *bg, const float *W1,
-                      const float *W3, const float *W2, int T, int d, int E, int K, int H, int Es, int renorm,
-                      int bf16_mode, float *dx, float *dWg, float *dbg, float *dW1, float *dW3, float *dW2,
-                      float *dw_o, float *dlogits_o)
+/* The pass for a given routing.  p [T,E]: softmax of the gate logits; ids [T,K]: selected experts as the gate numbers
+ * them (0..E-1); wid [T,K]: the same experts as indices into W1/W3/W2, which hold Ew routed experts followed by Es
+ * shared ones (wid == ids and Ew == E for a whole layer; a test that checks a few tokens of a large batch passes only
+ * the experts those tokens use); w [T,K]: combine weights.  Outputs as orc_moe_backward (dWg, dbg sum over the T
+ * tokens given). */
+static void backward_core(const float *x, const float *dout, const float *Wg, const float *p, const int32_t *ids,
+                          const int32_t *wid, const float *w, const float *W1, const float *W3, const float *W2, int T,
+                          int d, int E, int Ew, int K, int H, int Es, int renorm, int bf16_mode, float *dx, float *dWg,
+                          float *dbg, float *dW1, float *dW3, float *dW2, float *dw_o, float *dlogits_o)
 {
     const int P = T * K;
     const size_t HD = (size_t)H * d;
-    float *logits = (float *)malloc(sizeof(float) * (size_t)T * E);
-    float *p = (float *)malloc(sizeof(float) * (size_t)T * E);
-    int32_t *ids = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
-    float *w = (float *)malloc(sizeof(float) * (size_t)P);
-    int32_t *counts = (int32_t *)malloc(sizeof(int32_t) * (size_t)E);
-    int32_t *offsets = (int32_t *)malloc(sizeof(int32_t) * (size_t)(E + 1));
-    int32_t *dst = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
-    int32_t *src_row = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
+    int32_t *counts = (int32_t *)malloc(sizeof(int32_t) * (size_t)Ew);
+    int32_t *offsets = (int32_t *)malloc(sizeof(int32_t) * (size_t)(Ew + 1));
+    int32_t *dst = (int32_t *)malloc(sizeof(int32_t) * (size_t)(P ? P : 1));
+    int32_t *src_row = (int32_t *)malloc(sizeof(int32_t) * (size_t)(P ? P : 1));
     float *xg = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1) * d);
     float *y = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1) * d);
     float *dy = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1) * d);
@@ -128,16 +128,12 @@ void orc_moe_backward(const float *x, const float *dout, const float *Wg, const 
     float *g1 = (float *)malloc(sizeof(float) * HD), *g3 = (float *)malloc(sizeof(float) * HD),
           *g2 = (float *)malloc(sizeof(float) * HD);
 
-    /* forward quantities */
-    orc_gate(x, Wg, bg, T, d, E, logits);
-    orc_softmax(logits, T, E, p);
-    orc_topk(p, T, E, K, renorm, ids, w);
-    orc_dispatch(ids, T, K, E, counts, offsets, dst, src_row);
+    orc_dispatch(wid, T, K, Ew, counts, offsets, dst, src_row);
     for (int r = 0; r < P; ++r) memcpy(xg + (size_t)r * d, x + (size_t)src_row[r] * d, sizeof(float) * (size_t)d);
     {
         /* y of the routed rows (needed for the gradient of the combine weights) */
         float *a = scratch;
-        for (int e = 0; e < E; ++e)
+        for (int e = 0; e < Ew; ++e)
             for (int r = offsets[e]; r < offsets[e + 1]; ++r) {
                 const float *xr = xg + (size_t)r * d;
                 const float *w1b = W1 + (size_t)e * HD, *w3b = W3 + (size_t)e * HD, *w2b = W2 + (size_t)e * HD;
@@ -179,7 +175,7 @@ void orc_moe_backward(const float *x, const float *dout, const float *Wg, const 
         }
 
     /* experts */
-    for (int e = 0; e < E; ++e) {
+    for (int e = 0; e < Ew; ++e) {
         expert_backward(xg + (size_t)offsets[e] * d, dy + (size_t)offsets[e] * d, counts[e], W1 + (size_t)e * HD,
                         W3 + (size_t)e * HD, W2 + (size_t)e * HD, d, H, bf16_mode, dxg + (size_t)offsets[e] * d, g1,
                         g3, g2, scratch);
@@ -188,7 +184,7 @@ void orc_moe_backward(const float *x, const float *dout, const float *Wg, const 
         if (dW2) memcpy(dW2 + (size_t)e * HD, g2, sizeof(float) * HD);
     }
     for (int s = 0; s < Es; ++s) {
-        const int g = E + s;
+        const int g = Ew + s;
         expert_backward(x, dout, T, W1 + (size_t)g * HD, W3 + (size_t)g * HD, W2 + (size_t)g * HD, d, H, bf16_mode,
                         dxs + (size_t)s * T * d, g1, g3, g2, scratch);
         if (dW1) memcpy(dW1 + (size_t)g * HD, g1, sizeof(float) * HD);
@@ -253,7 +249,38 @@ void orc_moe_backward(const float *x, const float *dout, const float *Wg, const 
 
     if (dw_o) memcpy(dw_o, dw, sizeof(float) * (size_t)P);
     if (dlogits_o) memcpy(dlogits_o, dlog, sizeof(float) * (size_t)T * E);
-    free(logits); free(p); free(ids); free(w); free(counts); free(offsets); free(dst); free(src_row);
+    free(counts); free(offsets); free(dst); free(src_row);
     free(xg); free(y); free(dy); free(dxg); free(dxs); free(dw); free(dlog); free(scratch);
     free(g1); free(g3); free(g2);
+}
+
+/* Whole backward pass.  x, dout: [T,d]; weights as in orc_moe_forward (W1,W3: [E+Es,H,d], W2: [E+Es,d,H]).
+ * The forward quantities it needs are recomputed here.  Outputs (any may be NULL except dx): dx [T,d], dWg [E,d],
+ * dbg [E], dW1,dW3 [E+Es,H,d], dW2 [E+Es,d,H], dw [T,K] (gradient of the combine weights), dlogits [T,E]. */
+void orc_moe_backward(const float *x, const float *dout, const float *Wg, const float *bg, const float *W1,
+                      const float *W3, const float *W2, int T, int d, int E, int K, int H, int Es, int renorm,
+                      int bf16_mode, float *dx, float *dWg, float *dbg, float *dW1, float *dW3, float *dW2,
+                      float *dw_o, float *dlogits_o)
+{
+    const int P = T * K;
+    float *logits = (float *)malloc(sizeof(float) * (size_t)T * E);
+    float *p = (float *)malloc(sizeof(float) * (size_t)T * E);
+    int32_t *ids = (int32_t *)malloc(sizeof(int32_t) * (size_t)(P ? P : 1));
+    float *w = (float *)malloc(sizeof(float) * (size_t)(P ? P : 1));
+    orc_gate(x, Wg, bg, T, d, E, logits);
+    orc_softmax(logits, T, E, p);
+    orc_topk(p, T, E, K, renorm, ids, w);
+    backward_core(x, dout, Wg, p, ids, ids, w, W1, W3, W2, T, d, E, E, K, H, Es, renorm, bf16_mode, dx, dWg, dbg, dW1,
+                  dW3, dW2, dw_o, dlogits_o);
+    free(logits); free(p); free(ids); free(w);
+}
+
+/* The pass for a few tokens of a larger batch whose routing is known (see backward_core for p, ids, wid, w, Ew). */
+void orc_moe_backward_routed(const float *x, const float *dout, const float *Wg, const float *p, const int32_t *ids,
+                             const int32_t *wid, const float *w, const float *W1, const float *W3, const float *W2,
+                             int T, int d, int E, int Ew, int K, int H, int Es, int renorm, int bf16_mode, float *dx,
+                             float *dw_o, float *dlogits_o)
+{
+    backward_core(x, dout, Wg, p, ids, wid, w, W1, W3, W2, T, d, E, Ew, K, H, Es, renorm, bf16_mode, dx, NULL, NULL,
+                  NULL, NULL, NULL, dw_o, dlogits_o);
 }

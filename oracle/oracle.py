@@ -50,6 +50,7 @@ def lib():
                                         + [_f, _f, _f, _f, _i, _f, _i, _i, _i, _i, _f])
         L.orc_moe_backward.argtypes = ([_f, _f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8
                                        + [_f, _f, C.c_void_p, _f, _f, _f, _f, _f])
+        L.orc_moe_backward_routed.argtypes = ([_f, _f, _f, _f, _i, _i, _f, _f, _f, _f] + [C.c_int] * 9 + [_f, _f, _f])
         L.orc_cpu_baseline_forward.restype = C.c_double
         L.orc_cpu_baseline_forward.argtypes = [_f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8 + [_f]
         L.orc_cpu_sgemm_tn.argtypes = [C.c_int, C.c_int, C.c_int, _f, C.c_int, _f, C.c_int, _f, C.c_int, C.c_int]
@@ -189,6 +190,20 @@ def moe_backward(x, dout, Wg, bg, W1, W3, W2, K, renorm, Es=0, bf16=False):
     lib().orc_moe_backward(x, np.ascontiguousarray(dout, np.float32), Wg, _opt(bg), W1, W3, W2, T, d, E, K, H, Es,
                            int(renorm), int(bf16), r["dx"], r["dWg"], _opt(r["dbg"]), r["dW1"], r["dW3"], r["dW2"],
                            r["dw"], r["dlogits"])
+    return r
+
+
+def moe_backward_routed(x, dout, Wg, p, ids, wid, w, W1, W3, W2, Es, renorm, bf16=False):
+    """Backward for a few tokens of a larger batch with their routing given: p [n,E] gate probabilities, ids [n,K]
+    experts as the gate numbers them, wid [n,K] the same experts as indices into W1/W3/W2 (Ew routed experts, then Es
+    shared), w [n,K].  Returns dict(dx, dw, dlogits)."""
+    n, d = x.shape
+    E, K, H, Ew = p.shape[1], ids.shape[1], W1.shape[1], W1.shape[0] - Es
+    r = dict(dx=np.empty((n, d), np.float32), dw=np.empty((n, K), np.float32), dlogits=np.empty((n, E), np.float32))
+    c = np.ascontiguousarray
+    lib().orc_moe_backward_routed(c(x, np.float32), c(dout, np.float32), c(Wg, np.float32), c(p, np.float32),
+                                  c(ids, np.int32), c(wid, np.int32), c(w, np.float32), c(W1), c(W3), c(W2), n, d, E, Ew, K,
+                                  H, Es, int(renorm), int(bf16), r["dx"], r["dw"], r["dlogits"])
     return r
 
 

@@ -136,3 +136,75 @@ def test_backward_bf16_matches_oracle(name, kw):
                           bf16=True)
     assert N.rel_l2(dx2, ref2["dx"]) < 1e-2
     layer.close()
+
+
+def test_backward_full_size_mixtral():
+    """C2 at full size.  Rows of a token depend on that token only: input gradient and dlogits of sampled tokens against
+    the oracle (with the experts those tokens use).  Weight gradients of every expert through bilinear probes:
+    u^T dW v = sum_r (delta_r . u)(input_r . v) over the expert's rows, with delta and input taken from the workspace
+    (dy is recomputed on the host from dout, the combine weights and the permutation)."""
+    from tests import gpu_util as G
+    P = G.P
+    cfg = C.CONFIGS["c2_mixtral"]
+    T, d, H, E, K = cfg.T, cfg.d, cfg.H, cfg.E, cfg.K
+    layer = P.MoELayer(d, H, E, K, renorm=cfg.renorm, nShared=cfg.Es, bias=cfg.has_gate_bias, ctx=G.ctx(), dtype=cfg.dtype,
+                       router_mode="exact", T_max=T)
+    layer.init_synthetic(77, C, cfg)
+    x = P.DeviceBuffer(G.ctx(), (T, d), cfg.dtype)
+    x.fill_normal(77, C.STREAM_X, C.tensor_std(cfg, "x"))
+    g = P.DeviceBuffer(G.ctx(), (T, d), cfg.dtype)
+    g.fill_normal(77, 900, 1.0)
+    layer.forward(x)
+    dx = layer.back(g).to_numpy()
+    assert np.isfinite(dx).all()
+    xh, gh = x.to_numpy(), g.to_numpy()
+    r = layer.routing()
+    Wg = layer._download_weight(L.W_GATE, 0, (E, d))
+    p = O.softmax(O.gate(xh, Wg, None))
+    # ---- sampled tokens against the oracle
+    tok = np.unique(np.linspace(0, T - 1, 5).astype(np.int64))
+    need = sorted(set(r["ids"][tok].ravel().tolist()))
+    remap = {e: i for i, e in enumerate(need)}
+    wid = np.vectorize(remap.get)(r["ids"][tok]).astype(np.int32)
+    W1 = np.stack([layer._download_weight(L.W_W1, e, (H, d)) for e in need])
+    W3 = np.stack([layer._download_weight(L.W_W3, e, (H, d)) for e in need])
+    W2 = np.stack([layer._download_weight(L.W_W2, e, (d, H)) for e in need])
+    ref = O.moe_backward_routed(xh[tok], gh[tok], Wg, p[tok], r["ids"][tok], wid, r["w"][tok], W1, W3, W2, 0, cfg.renorm,
+                                bf16=True)
+    del W1, W3, W2
+    assert N.rel_l2(dx[tok], ref["dx"]) < 1e-2, N.rel_l2(dx[tok], ref["dx"])
+    dlog = layer.workspace("dlogits", T)
+    assert N.rel_l2(dlog[tok], ref["dlogits"]) < 1e-2
+    # ---- gate weight gradient: all tokens
+    rng = np.random.default_rng(5)
+    u, v = rng.standard_normal((4, E)), rng.standard_normal((4, d))
+    dWg = layer.grad(L.W_GATE).astype(np.float64)
+    want = np.array([((dlog @ u[i]) * (xh @ v[i])).sum() for i in range(4)])
+    got = np.array([u[i] @ dWg @ v[i] for i in range(4)])
+    assert N.rel_l2(got, want) < 1e-3, (got, want)
+    # ---- expert weight gradients: every expert, all its rows
+    a = layer.workspace("a", T)            # [P,H]
+    xg = layer.workspace("xg", T)          # [P,d]
+    dh = layer.workspace("dh", T)          # [P,2H]
+    dy = np.empty((T * K, d), np.float32)  # dy[dst[p]] = bf16(w[p] * dout[t])
+    wflat = r["w"].reshape(-1)
+    dy[r["dst"]] = O.round_bf16(wflat[:, None] * np.repeat(gh, K, axis=0))
+    off = r["offsets"]
+    ud, vH = rng.standard_normal(d), rng.standard_normal(H)
+    uH, vd = rng.standard_normal(H), rng.standard_normal(d)
+    got2, want2, got1, want1, got3, want3 = [], [], [], [], [], []
+    for e in range(E):
+        rows = slice(off[e], off[e + 1])
+        dW2 = layer.grad(L.W_W2, e)
+        got2.append(ud @ (dW2.astype(np.float64) @ vH))
+        want2.append(((dy[rows].astype(np.float64) @ ud) * (a[rows].astype(np.float64) @ vH)).sum())
+        xv = xg[rows].astype(np.float64) @ vd
+        dW1 = layer.grad(L.W_W1, e)
+        got1.append(uH @ (dW1.astype(np.float64) @ vd))
+        want1.append(((dh[rows, :H].astype(np.float64) @ uH) * xv).sum())
+        dW3 = layer.grad(L.W_W3, e)
+        got3.append(uH @ (dW3.astype(np.float64) @ vd))
+        want3.append(((dh[rows, H:].astype(np.float64) @ uH) * xv).sum())
+    for gt, wt, nm in ((got2, want2, "dW2"), (got1, want1, "dW1"), (got3, want3, "dW3")):
+        assert N.rel_l2(np.array(gt), np.array(wt)) < 1e-3, (nm, gt, wt)
+    layer.close()

@@ -152,3 +152,21 @@ def test_backward_bf16_mode_close_to_float64():
     for k in ("dx", "dWg", "dW1", "dW3", "dW2"):
         assert N.rel_l2(got[k], ref[k]) < 1e-2, (k, N.rel_l2(got[k], ref[k]))
     assert np.array_equal(got["dx"], O.round_bf16(got["dx"]))
+
+
+def test_backward_routed_equals_full_on_a_token_subset():
+    # input gradient, dw and dlogits of a token depend on that token only: a subset with compacted expert indices
+    # reproduces the rows of the full pass bit for bit
+    cfg, inp, dout = _case("c1_tiny_f32", 21, T=30, d=16, H=12, E=6, K=2, Es=1)
+    fwd = O.moe_forward(inp["x"], inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es)
+    full = O.moe_backward(inp["x"], dout, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es)
+    tok = np.array([3, 4, 17, 29])
+    need = sorted(set(fwd["ids"][tok].ravel().tolist()))
+    remap = {g: i for i, g in enumerate(need)}
+    wid = np.vectorize(remap.get)(fwd["ids"][tok]).astype(np.int32)
+    sel = need + [cfg.E + s for s in range(cfg.Es)]
+    got = O.moe_backward_routed(inp["x"][tok], dout[tok], inp["Wg"], fwd["p"][tok], fwd["ids"][tok], wid, fwd["w"][tok],
+                                inp["W1"][sel], inp["W3"][sel], inp["W2"][sel], cfg.Es, cfg.renorm)
+    assert np.array_equal(got["dx"], full["dx"][tok])
+    assert np.array_equal(got["dw"], full["dw"][tok])
+    assert np.array_equal(got["dlogits"], full["dlogits"][tok])
