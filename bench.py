@@ -43,6 +43,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample duration")
     ap.add_argument("--no-mfma-probe", action="store_true",
                     help="skip the matrix-core ceiling probe (two runs of about 1 s with no memory traffic)")
+    ap.add_argument("--no-backward", action="store_true", help="skip the backward-pass figures")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (convert_kernel fp32->fp32) three times, so that "
                          "FETCH_SIZE / WRITE_SIZE of a profiled run can be scaled by a kernel of known traffic")
@@ -117,6 +118,30 @@ def main():
             probe[key] = v.value
         probe["frac_of_random_operand_rate"] = up_tflops / probe["random_operands_TFLOP/s"]
 
+    # backward pass (the widening behind the path): after a plain forward (h1 / h3 recomputed) and in training mode
+    # (the forward pass keeps them); algorithmic work = input and weight gradients of the three products, 12*d*H per row
+    backward = None
+    if not a.no_backward:
+        gbuf = P.DeviceBuffer(ctx, (cfg.T, cfg.d), cfg.dtype)
+        gbuf.fill_normal(a.seed, 900, 1.0)
+        dxb = P.DeviceBuffer(ctx, (cfg.T, cfg.d), cfg.dtype)
+        outf = layer.forward(x)
+        bw_ms = layer.time_backward(x, gbuf, cfg.T, dxb, warmup=2, iters=max(3, a.steps // 2))
+        layer.set_training(True)
+        fwd_train_ms = layer.time_stage(L.STAGE_FORWARD, x, cfg.T, out=outf, warmup=2, iters=max(3, a.steps // 2))
+        layer.forward(x)
+        bw_train_ms = layer.time_backward(x, gbuf, cfg.T, dxb, warmup=2, iters=max(3, a.steps // 2))
+        layer.set_training(False)
+        bw_flops = 12.0 * cfg.d * cfg.H * rows
+        backward = {"what": "omega_moe_backward: dx and all parameter gradients (fp32) for one dout",
+                    "ms": bw_ms, "algorithmic_TFLOP/s": bw_flops / (bw_ms * 1e-3) / 1e12,
+                    "training_mode": {"forward_ms": fwd_train_ms, "backward_ms": bw_train_ms,
+                                      "algorithmic_TFLOP/s": bw_flops / (bw_train_ms * 1e-3) / 1e12,
+                                      "frac_mfma": bw_flops / (bw_train_ms * 1e-3) / 1e12 / peak,
+                                      "fwd+bwd_tokens/s": cfg.T / ((fwd_train_ms + bw_train_ms) * 1e-3)}}
+        gbuf.free()
+        dxb.free()
+
     res = {
         "metric": "MoE-layer fwd tokens/s (Mixtral shape, bf16); MFMA util %; dispatch GB/s",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -132,6 +157,7 @@ def main():
                      "mfma_only_probe": probe},
         "block_form": {"what": "out = x + layer(rmsnorm(x)) in one call (omega_moe_forward_block)", "ms_per_step": block_ms,
                        "tokens/s": cfg.T / (block_ms * 1e-3), "prenorm_kernel_ms": rms_ms},
+        "backward": backward,
         "stages": {
             "avg_ms": stage_ms, "profiled_forwards": n_prof,
             "experts_down": {"TFLOP/s": down_tflops, "frac_mfma": down_tflops / peak},

@@ -140,6 +140,12 @@ int omega_moe_get_norm(omega_moe *moe, int T, float *rms_host);
  * softmax_back (J/engine/gpu/SoftmaxKernel.cu:101-112) -> gate linear layer.  The expert ids and the permutation carry
  * no gradient.  Asynchronous on the context's stream. */
 int omega_moe_backward(omega_moe *moe, const void *x_dev, const void *dout_dev, int T, void *dx_dev);
+/* Training mode (off at creation).  The reference's layers keep their outputs for back() (LlamaMLPLayer.diff reads
+ * active.getOutput() and getLinear3().getOutput(), J/engine/nn/layer/llama/LlamaMLPLayer.java:148-152); with training
+ * on, omega_moe_forward of a bf16 layer likewise stores h1 and h3 (fp32, from the accumulators of its up product) and
+ * omega_moe_backward reads them instead of recomputing them.  Same results either way; the forward pass writes
+ * 8*H bytes more per expert row.  fp32 layers ignore the switch. */
+int omega_moe_set_training(omega_moe *moe, int on);
 /* One parameter gradient of the last omega_moe_backward, always fp32, in the layout of the weight it belongs to
  * (which / expert as for omega_moe_set_weights; OMEGA_W_NORM has none).  Stands in for reading layer.diffW / diffB
  * (LlamaMLPLayer.putParamterGrads, J/engine/nn/layer/llama/LlamaMLPLayer.java:285-295). */

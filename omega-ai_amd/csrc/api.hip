@@ -513,6 +513,13 @@ static int check_T(omega_moe *m, const void *x, int T, bool need_x)
     return OMEGA_OK;
 }
 
+// a stage run on its own rewrites part of what a backward pass would read: the last forward no longer counts
+static void stage_invalidates(omega_moe *m)
+{
+    m->fwd_T = -1;
+    m->rec_valid = false;
+}
+
 static int stage_router(omega_moe *m, const void *x, int T)
 {
     OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, nullptr, m->ctx->stream));
@@ -565,6 +572,13 @@ static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block
     const void *resid = block ? x : nullptr;
     const void *xin = block ? m->hbuf : x;
     m->fwd_T = block ? -1 : T;
+    // training mode (bf16 layers): the up product also leaves h1 / h3 for the backward pass
+    const bool keep = m->training && !block && m->cfg.dtype == OMEGA_DTYPE_BF16;
+    if (keep) {
+        m->bm = moe_tile_m(m, T);
+        RUN(moe_reserve_backward(m, T));
+    }
+    m->rec_valid = false;
     if (m->profiling) {
         // six events bracket the five stages; durations are read back by omega_moe_get_profile
         if (m->prof_used + 6 > m->prof_events.size()) {
@@ -588,6 +602,7 @@ static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block
         RUN(stage_combine(m, T, out, resid));
         OMEGA_HIP_CHECK(ctx, hipEventRecord(ev[5], ctx->stream));
         m->prof_used += 6;
+        m->rec_valid = keep;
         return OMEGA_OK;
     }
     if (block) OMEGA_HIP_CHECK(ctx, launch_rmsnorm(m, x, T, m->hbuf, ctx->stream));
@@ -596,6 +611,15 @@ static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block
     RUN(stage_experts(m, xin, T, 0));
     RUN(stage_experts(m, xin, T, 1));
     RUN(stage_combine(m, T, out, resid));
+    m->rec_valid = keep;
+    return OMEGA_OK;
+}
+
+int omega_moe_set_training(omega_moe *m, int on)
+{
+    MOE_ENTER(m);
+    m->training = on != 0;
+    m->rec_valid = false;
     return OMEGA_OK;
 }
 
@@ -747,6 +771,7 @@ int omega_moe_get_profile(omega_moe *m, float *stage_ms_sum, int *n_calls)
 int omega_moe_router(omega_moe *m, const void *x, int T)
 {
     MOE_ENTER(m);
+    stage_invalidates(m);
     RUN(check_T(m, x, T, true));
     if (T == 0) return OMEGA_OK;
     RUN(moe_reserve(m, T));
@@ -756,6 +781,7 @@ int omega_moe_router(omega_moe *m, const void *x, int T)
 int omega_moe_dispatch(omega_moe *m, const void *x, int T)
 {
     MOE_ENTER(m);
+    stage_invalidates(m);
     RUN(check_T(m, x, T, true));
     if (T == 0) return OMEGA_OK;
     if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "dispatch: router has not run for this T");
@@ -765,6 +791,7 @@ int omega_moe_dispatch(omega_moe *m, const void *x, int T)
 int omega_moe_experts_up(omega_moe *m, const void *x, int T)
 {
     MOE_ENTER(m);
+    stage_invalidates(m);
     RUN(check_T(m, x, T, m->cfg.Es > 0));
     if (T == 0) return OMEGA_OK;
     if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "experts: router has not run for this T");
@@ -774,6 +801,7 @@ int omega_moe_experts_up(omega_moe *m, const void *x, int T)
 int omega_moe_experts_down(omega_moe *m, int T)
 {
     MOE_ENTER(m);
+    stage_invalidates(m);
     RUN(check_T(m, nullptr, T, false));
     if (T == 0) return OMEGA_OK;
     if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "experts: router has not run for this T");
@@ -909,6 +937,7 @@ int omega_hip_mfma_probe(omega_ctx *ctx, int random_operands, int launches, floa
 int omega_moe_time_stage(omega_moe *m, int stage, const void *x, int T, void *out, int warmup, int iters, float *ms_avg)
 {
     MOE_ENTER(m);
+    stage_invalidates(m);
     RUN(check_T(m, x, T, stage == 0 || stage == 1 || stage == 5 || stage == 7 || stage == 8 || stage == 9));
     if ((stage == 6 || stage == 7) && m->bm == 0) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: dispatch has not run");
     if (!ms_avg || iters <= 0 || warmup < 0 || stage < 0 || stage > 9 || T <= 0)

@@ -456,7 +456,8 @@ hipError_t launch_backward_bf16(const omega_moe *m, const void *x, const void *d
     STEP(hipGetLastError());
     // h1, h3 (recomputed) as block records; d(a) = dy . W2 with the SwiGLU backward in its epilogue -> dh1 | dh3;
     // dxg = dh1 . W1 + dh3 . W3 as one product over the 2H columns of dh
-    STEP(launch_product_bf16(m, MODE_UPRAW, m->xg, m->xs, m->W1, m->W3, m->bw_h1, m->bw_h3, nullptr, m->wq_up, c.H, c.d, s));
+    if (!m->rec_valid)
+        STEP(launch_product_bf16(m, MODE_UPRAW, m->xg, m->xs, m->W1, m->W3, m->bw_h1, m->bw_h3, nullptr, m->wq_up, c.H, c.d, s));
     STEP(launch_product_bf16(m, MODE_DA, m->bw_dy16, m->bw_dys16, m->W2T, nullptr, m->bw_dh16, m->bw_h1, m->bw_h3, m->wq_da,
                              c.H, c.d, s));
     STEP(launch_product_bf16(m, MODE_DOWN, m->bw_dh16, nullptr, m->W13T, nullptr, m->bw_dxg, nullptr, nullptr, m->wq_down, c.d,

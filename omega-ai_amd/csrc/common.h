@@ -118,6 +118,8 @@ struct omega_moe {
     int bw_T_cap = 0;
     size_t bw_rows_cap = 0;
     int fwd_T = -1;                  // tokens of the last plain forward (what backward may follow), -1: none
+    bool training = false;           // forward keeps h1 / h3 (bf16 layers: as block records in bw_h1 / bw_h3)
+    bool rec_valid = false;          // bw_h1 / bw_h3 hold h1 / h3 of the last forward
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     // per-stage event profiling of forward calls (6 events per call), off by default
     bool profiling = false;
@@ -162,7 +164,7 @@ hipError_t launch_transpose_groups(const omega_moe *m, const void *src, const vo
 hipError_t launch_transpose_images(const void *src, int R, int cols, void *dst, int KTd, int k0, int n, size_t src_stride,
                                    size_t dst_stride, hipStream_t s);
 // products of the matrix-core kernel (experts_bf16.hip describes each)
-enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4 };
+enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4, MODE_UPREC = 5 };
 hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, const void *Aalt, const void *Wa, const void *Wb,
                                void *Cout, void *Aux1, void *Aux2, const omega_tile_desc *wq, int N, int Kd, hipStream_t s);
 hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, hipStream_t s);

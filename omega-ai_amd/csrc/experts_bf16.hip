@@ -40,12 +40,13 @@
 //   DOWN   tile 256 x 256, fp32 row-major output
 //   UPRAW  as UP, but h1 and h3 are stored as they sit in the accumulators (Cout = h1, Aux1 = h3): one 4 KiB record
 //          per 32x32 MFMA block, [row block][column block][register 0..15][lane 0..63]
+//   UPREC  UP and UPRAW in one: the forward pass of a layer in training mode (a -> Cout, h1 -> Aux1, h3 -> Aux2)
 //   DA     tile 256 x 256 of d(a) = dy . W2 (B = packed W2^T); the epilogue reads the h1/h3 records of its blocks
 //          (Aux1, Aux2), applies the SwiGLU backward and writes dh1 | dh3 as one packed bf16 image with 2N columns
 //   WGRAD  tile 256 x 256 of dW = A^T . B over the rows of one expert: both operands are transposed packed images
 //          whose K axis is the experts' rows; the item names its operand row groups, first k step and k steps
 //          (a_rg, b_rg, kt0, xrow0); fp32 row-major output, row0 = expert * M + first row
-#define FUSED_TILE(M) ((M) == MODE_UP || (M) == MODE_UPRAW)
+#define FUSED_TILE(M) ((M) == MODE_UP || (M) == MODE_UPRAW || (M) == MODE_UPREC)
 #define SWAPPED(M) ((M) != MODE_DOWN && (M) != MODE_WGRAD)
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -280,7 +281,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     cur_io = cur;
 
     // ---- epilogue ----
-    if (MODE == MODE_UP) {
+    if (MODE == MODE_UP || MODE == MODE_UPREC) {
         // lane: row l32 of block i; register r -> column 8*(r/4) + 4*lhi + r%4 of the wave's 32 columns, which are
         // one k step of the packed `a` (K dimension = N): chunk r/4, bytes lhi*8 .. lhi*8+7
         const int KTa = N / BK;
@@ -308,14 +309,16 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
                 }
             }
         }
-    } else if (MODE == MODE_UPRAW) {
+    }
+    if (MODE == MODE_UPRAW || MODE == MODE_UPREC) {
         // the accumulators as they are, one record per 32x32 block (whole blocks: rows past the item's last are
         // never read back as valid)
         const size_t cb = (size_t)(ctx.n0 >> 5) + wn, ncb = (size_t)(N >> 5);
+        float *r1 = (float *)(MODE == MODE_UPRAW ? Cout : Aux1), *r3 = (float *)(MODE == MODE_UPRAW ? Aux1 : Aux2);
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
             const size_t rb = (size_t)(ctx.row0 >> 5) + 2 * i + wm;
-            float *o1 = (float *)Cout + (rb * ncb + cb) * 1024 + lane, *o3 = (float *)Aux1 + (rb * ncb + cb) * 1024 + lane;
+            float *o1 = r1 + (rb * ncb + cb) * 1024 + lane, *o3 = r3 + (rb * ncb + cb) * 1024 + lane;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 o1[r * 64] = acc[i][0][r];
@@ -358,7 +361,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
                 }
             }
         }
-    } else {
+    } else if (MODE == MODE_DOWN || MODE == MODE_WGRAD) {
         // lane: column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
@@ -434,7 +437,7 @@ hipError_t experts_bf16_init(void)
 {
     const void *fns[] = {(const void *)experts_bf16_kernel<MODE_UP>, (const void *)experts_bf16_kernel<MODE_DOWN>,
                          (const void *)experts_bf16_kernel<MODE_UPRAW>, (const void *)experts_bf16_kernel<MODE_DA>,
-                         (const void *)experts_bf16_kernel<MODE_WGRAD>};
+                         (const void *)experts_bf16_kernel<MODE_WGRAD>, (const void *)experts_bf16_kernel<MODE_UPREC>};
     for (const void *f : fns) {
         hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
         if (e != hipSuccess) return e;
@@ -449,7 +452,12 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
     (void)x;
     // the ring must be shorter than an item: K >= (NSTAGE + 1) * BK (guaranteed at creation: d, H >= 256)
     if ((which == 0 ? c.d : c.H) < (NSTAGE + 1) * BK) return hipErrorInvalidValue;
-    if (which == 0) {
+    if (which == 0 && m->training && m->bw_h1 != nullptr) {
+        // training mode: h1 and h3 are kept for the backward pass, as the reference's layers keep their outputs
+        hipLaunchKernelGGL(experts_bf16_kernel<MODE_UPREC>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s,
+                           (const bf16_t *)m->xg, (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a,
+                           (void *)m->bw_h1, (void *)m->bw_h3, m->wq_up, c.H, c.d);
+    } else if (which == 0) {
         hipLaunchKernelGGL(experts_bf16_kernel<MODE_UP>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
                            (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
                            (void *)nullptr, m->wq_up, c.H, c.d);
@@ -475,6 +483,7 @@ hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, cons
         case MODE_UPRAW: LAUNCH(MODE_UPRAW); break;
         case MODE_DA: LAUNCH(MODE_DA); break;
         case MODE_WGRAD: LAUNCH(MODE_WGRAD); break;
+        case MODE_UPREC: LAUNCH(MODE_UPREC); break;
         default: return hipErrorInvalidValue;
     }
 #undef LAUNCH

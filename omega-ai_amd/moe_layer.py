@@ -218,6 +218,10 @@ class MoELayer:
     def getLayerType(self):
         return "feed_forward"
 
+    def set_training(self, on=True):
+        """Forward keeps h1 / h3 for back(), as the reference's layers keep their outputs."""
+        self.ctx.check(self.lib.omega_moe_set_training(self.handle, int(bool(on))))
+
     def initBack(self):
         """(Re)allocates the input gradient when the batch size changes (FullyLayer.initBack,
         J/engine/nn/layer/FullyLayer.java:130-144); the parameter gradients live in the native handle."""

@@ -126,6 +126,14 @@ def test_backward_bf16_matches_oracle(name, kw):
     assert np.array_equal(layer.back(g).to_numpy(), dx)
     assert np.array_equal(layer.grad(L.W_W2, 0), w2)
     assert np.array_equal(layer.forward(x).to_numpy(), out)
+    # training mode: the forward pass keeps h1 / h3, the backward pass skips their recomputation - same bits
+    w13 = (layer.grad(L.W_W1, cfg.E - 1), layer.grad(L.W_W3, 0))
+    layer.set_training(True)
+    assert np.array_equal(layer.forward(x).to_numpy(), out)
+    assert np.array_equal(layer.back(g).to_numpy(), dx)
+    assert np.array_equal(layer.grad(L.W_W2, 0), w2)
+    assert np.array_equal(layer.grad(L.W_W1, cfg.E - 1), w13[0]) and np.array_equal(layer.grad(L.W_W3, 0), w13[1])
+    layer.set_training(False)
     # new weights invalidate the transposed copies the pass keeps: gradients follow the new weights
     W2n = O.round_bf16(inp["W2"][0] * np.float32(0.5))
     layer.set_expert(0, inp["W1"][0], inp["W3"][0], W2n)
