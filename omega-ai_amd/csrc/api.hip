@@ -522,7 +522,9 @@ static void stage_invalidates(omega_moe *m)
 
 static int stage_router(omega_moe *m, const void *x, int T)
 {
-    OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, nullptr, m->ctx->stream));
+    // training mode (bf16 layers, backward workspace in place): the probabilities are kept for the backward pass
+    float *probs = (m->training && m->cfg.dtype == OMEGA_DTYPE_BF16 && m->bw_T_cap >= T) ? m->bw_probs : nullptr;
+    OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, probs, m->ctx->stream));
     return OMEGA_OK;
 }
 static int stage_dispatch(omega_moe *m, const void *x, int T)

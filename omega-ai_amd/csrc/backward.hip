@@ -235,7 +235,7 @@ template <bool XBF>
 __global__ __launch_bounds__(256) void bw_gate_partial_kernel(const float *__restrict__ dlogits, const void *__restrict__ x,
                                                               int T, int d, int E, int tslice, float *__restrict__ part)
 {
-    __shared__ float dl[64][GW_EC];
+    __shared__ __attribute__((aligned(16))) float dl[64][GW_EC];
     const int k = blockIdx.x * 256 + threadIdx.x, e0 = blockIdx.z * GW_EC;
     const int t0 = blockIdx.y * tslice, t1 = min(T, t0 + tslice);
     float acc[GW_EC];
@@ -254,7 +254,13 @@ __global__ __launch_bounds__(256) void bw_gate_partial_kernel(const float *__res
                 const float xv = XBF ? bf16_to_f32(((const bf16_t *)x)[(size_t)(tb + tt) * d + k])
                                      : ((const float *)x)[(size_t)(tb + tt) * d + k];
 #pragma unroll
-                for (int e = 0; e < GW_EC; ++e) acc[e] = fmaf(dl[tt][e], xv, acc[e]);
+                for (int e4 = 0; e4 < GW_EC / 4; ++e4) {  // the whole wave reads the same 16 bytes: one broadcast read
+                    const float4 v = *(const float4 *)&dl[tt][e4 * 4];
+                    acc[e4 * 4 + 0] = fmaf(v.x, xv, acc[e4 * 4 + 0]);
+                    acc[e4 * 4 + 1] = fmaf(v.y, xv, acc[e4 * 4 + 1]);
+                    acc[e4 * 4 + 2] = fmaf(v.z, xv, acc[e4 * 4 + 2]);
+                    acc[e4 * 4 + 3] = fmaf(v.w, xv, acc[e4 * 4 + 3]);
+                }
             }
         }
     }
@@ -304,13 +310,74 @@ __global__ __launch_bounds__(256) void bw_gate_bias_kernel(const float *__restri
     if (threadIdx.x == 0) dbg[e] = tot;
 }
 
-// One workgroup per token: dx[t,:] = sum_j dxg[row(t,j),:] (slot order) + shared-expert rows + dlogits[t,:] . Wg.
-// XBF: Wg and dx are bf16 (one rounding of the fp32 sum).
+// dx[t,:] = sum_j dxg[row(t,j),:] (slot order) + shared-expert rows + dlogits[t,:] . Wg.  One workgroup per DX_TT
+// tokens and 512 columns (a thread owns two adjacent columns): a gate weight is read once for the DX_TT tokens.
+// XBF: Wg and dx are bf16 (one rounding of the fp32 sum).  d must be even.
+#define DX_TT 8
 template <bool XBF>
 __global__ __launch_bounds__(256) void bw_dx_kernel(const float *__restrict__ dxg, const int32_t *__restrict__ dstp,
                                                     const float *__restrict__ dlogits, const void *__restrict__ Wg,
-                                                    const int32_t *__restrict__ tile_meta, int K, int d, int E, int Es,
+                                                    const int32_t *__restrict__ tile_meta, int T, int K, int d, int E, int Es,
                                                     int bm, void *__restrict__ dx)
+{
+    extern __shared__ __attribute__((aligned(16))) float dl[];  // [E][DX_TT]
+    const int t0 = blockIdx.x * DX_TT, nt = min(DX_TT, T - t0);
+    for (int i = threadIdx.x; i < E * DX_TT; i += 256) {
+        const int e = i / DX_TT, tt = i % DX_TT;
+        dl[i] = tt < nt ? dlogits[(size_t)(t0 + tt) * E + e] : 0.0f;
+    }
+    __syncthreads();
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 2;
+    if (c >= d) return;
+    float g0[DX_TT], g1[DX_TT];
+#pragma unroll
+    for (int tt = 0; tt < DX_TT; ++tt) g0[tt] = g1[tt] = 0.0f;
+    for (int e = 0; e < E; ++e) {
+        float w0, w1;
+        if (XBF) {
+            const uint32_t u = *(const uint32_t *)((const bf16_t *)Wg + (size_t)e * d + c);
+            w0 = __uint_as_float(u << 16);
+            w1 = __uint_as_float(u & 0xffff0000u);
+        } else {
+            const float2 f = *(const float2 *)((const float *)Wg + (size_t)e * d + c);
+            w0 = f.x;
+            w1 = f.y;
+        }
+        const float4 da = *(const float4 *)&dl[e * DX_TT], db = *(const float4 *)&dl[e * DX_TT + 4];
+        const float dv[DX_TT] = {da.x, da.y, da.z, da.w, db.x, db.y, db.z, db.w};
+#pragma unroll
+        for (int tt = 0; tt < DX_TT; ++tt) {
+            g0[tt] = fmaf(dv[tt], w0, g0[tt]);
+            g1[tt] = fmaf(dv[tt], w1, g1[tt]);
+        }
+    }
+#pragma unroll
+    for (int tt = 0; tt < DX_TT; ++tt) {
+        if (tt >= nt) break;
+        const int t = t0 + tt;
+        float a0 = 0.0f, a1 = 0.0f;
+        for (int j = 0; j < K; ++j) {
+            const float2 v = *(const float2 *)(dxg + (size_t)dstp[(size_t)t * K + j] * d + c);
+            a0 += v.x;
+            a1 += v.y;
+        }
+        for (int s = 0; s < Es; ++s) {
+            const float2 v = *(const float2 *)(dxg + ((size_t)tile_meta[1 + E + s] * bm + t) * d + c);
+            a0 += v.x;
+            a1 += v.y;
+        }
+        a0 += g0[tt];
+        a1 += g1[tt];
+        if (XBF) *(uint32_t *)((bf16_t *)dx + (size_t)t * d + c) = (uint32_t)f32_to_bf16(a0) | ((uint32_t)f32_to_bf16(a1) << 16);
+        else *(float2 *)((float *)dx + (size_t)t * d + c) = make_float2(a0, a1);
+    }
+}
+
+// fp32 layers whose width is odd: one workgroup per token, one column per thread and step
+__global__ __launch_bounds__(256) void bw_dx_scalar_kernel(const float *__restrict__ dxg, const int32_t *__restrict__ dstp,
+                                                           const float *__restrict__ dlogits, const float *__restrict__ Wg,
+                                                           const int32_t *__restrict__ tile_meta, int K, int d, int E, int Es,
+                                                           int bm, float *__restrict__ dx)
 {
     const int t = blockIdx.x;
     extern __shared__ float dl[];  // E floats
@@ -321,10 +388,8 @@ __global__ __launch_bounds__(256) void bw_dx_kernel(const float *__restrict__ dx
         for (int j = 0; j < K; ++j) acc += dxg[(size_t)dstp[(size_t)t * K + j] * d + c];
         for (int s = 0; s < Es; ++s) acc += dxg[((size_t)tile_meta[1 + E + s] * bm + t) * d + c];
         float gs = 0.0f;
-        for (int e = 0; e < E; ++e)
-            gs = fmaf(dl[e], XBF ? bf16_to_f32(((const bf16_t *)Wg)[(size_t)e * d + c]) : ((const float *)Wg)[(size_t)e * d + c], gs);
-        if (XBF) ((bf16_t *)dx)[(size_t)t * d + c] = f32_to_bf16(acc + gs);
-        else ((float *)dx)[(size_t)t * d + c] = acc + gs;
+        for (int e = 0; e < E; ++e) gs = fmaf(dl[e], Wg[(size_t)e * d + c], gs);
+        dx[(size_t)t * d + c] = acc + gs;
     }
 }
 
@@ -384,8 +449,14 @@ hipError_t launch_backward_f32(const omega_moe *m, const void *xv, const void *d
     if ((e = launch_gate_wgrad(m, x, T, s)) != hipSuccess) return e;
     if (c.has_gate_bias)
         hipLaunchKernelGGL(bw_gate_bias_kernel, dim3(c.E), dim3(256), 0, s, (const float *)m->bw_dlogits, T, c.E, m->dbg);
-    hipLaunchKernelGGL(bw_dx_kernel<false>, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,
-                       (const float *)m->bw_dlogits, (const void *)m->Wg, m->tile_meta, c.K, c.d, c.E, c.Es, m->bm, dxv);
+    if (c.d % 2 == 0 && ((uintptr_t)dxv % 8) == 0)
+        hipLaunchKernelGGL(bw_dx_kernel<false>, dim3(ceil_div(T, DX_TT), ceil_div(c.d, 512)), dim3(256),
+                           c.E * DX_TT * sizeof(float), s, (const float *)m->bw_dxg, m->dstp, (const float *)m->bw_dlogits,
+                           (const void *)m->Wg, m->tile_meta, T, c.K, c.d, c.E, c.Es, m->bm, dxv);
+    else
+        hipLaunchKernelGGL(bw_dx_scalar_kernel, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,
+                           (const float *)m->bw_dlogits, (const float *)m->Wg, m->tile_meta, c.K, c.d, c.E, c.Es, m->bm,
+                           (float *)dxv);
     return hipGetLastError();
 }
 
@@ -449,7 +520,7 @@ hipError_t launch_backward_bf16(const omega_moe *m, const void *x, const void *d
     const size_t HD = (size_t)c.H * c.d;
     hipError_t e;
 #define STEP(expr) if ((e = (expr)) != hipSuccess) return e
-    STEP(launch_router(m, x, T, nullptr, m->bw_probs, s));
+    if (!m->rec_valid) STEP(launch_router(m, x, T, nullptr, m->bw_probs, s));  // a training forward kept the probabilities
     STEP(launch_backward_tables(m, T, s));
     hipLaunchKernelGGL(bw_combine_bf16_kernel, dim3(T), dim3(256), 0, s, (const uint4 *)dout, (const float *)m->y, m->dstp, m->w,
                        c.K, c.d, (unsigned char *)m->bw_dy16, (unsigned char *)m->bw_dys16, m->bw_dw);
@@ -471,15 +542,16 @@ hipError_t launch_backward_bf16(const omega_moe *m, const void *x, const void *d
                              m->bw_ksteps_cap * 32, s));
     STEP(launch_product_bf16(m, MODE_WGRAD, m->bw_dhT, nullptr, m->bw_xgT, nullptr, m->dW13, nullptr, nullptr, m->wq_w13, c.d,
                              m->bw_ksteps_cap * 32, s));
-    hipLaunchKernelGGL(bw_zero_empty_kernel, dim3(G, 32), dim3(256), 0, s, m->counts, c.E, T, m->dW13, m->dW2, HD);
+    hipLaunchKernelGGL(bw_zero_empty_kernel, dim3(G, 128), dim3(256), 0, s, m->counts, c.E, T, m->dW13, m->dW2, HD);
     // router and gate
     hipLaunchKernelGGL(bw_router_kernel, dim3(ceil_div(T, 256)), dim3(256), 0, s, (const float *)m->bw_probs, m->ids, m->w,
                        (const float *)m->bw_dw, T, c.E, c.K, c.renorm, m->bw_dlogits);
     STEP(launch_gate_wgrad(m, x, T, s));
     if (c.has_gate_bias)
         hipLaunchKernelGGL(bw_gate_bias_kernel, dim3(c.E), dim3(256), 0, s, (const float *)m->bw_dlogits, T, c.E, m->dbg);
-    hipLaunchKernelGGL(bw_dx_kernel<true>, dim3(T), dim3(256), c.E * sizeof(float), s, (const float *)m->bw_dxg, m->dstp,
-                       (const float *)m->bw_dlogits, (const void *)m->Wg, m->tile_meta, c.K, c.d, c.E, c.Es, m->bm, dx);
+    hipLaunchKernelGGL(bw_dx_kernel<true>, dim3(ceil_div(T, DX_TT), ceil_div(c.d, 512)), dim3(256), c.E * DX_TT * sizeof(float), s,
+                       (const float *)m->bw_dxg, m->dstp, (const float *)m->bw_dlogits, (const void *)m->Wg, m->tile_meta, T, c.K,
+                       c.d, c.E, c.Es, m->bm, dx);
 #undef STEP
     return hipGetLastError();
 }

@@ -468,8 +468,8 @@ hipError_t launch_unpack_rows(void *dst_rowmajor, const void *src_packed, int R,
 __device__ __forceinline__ int kspace_steps(int rows) { return rows > 0 ? max((rows + 63) / 64 * 2, 6) : 0; }
 
 // One workgroup per group g: the items of the d(a) product (256-column tiles over H, table as the forward ones), the
-// group's place in k space, and its items of the two weight-gradient products (all 256 x 256 tiles of dW_g, column
-// tile by column tile; descriptor: row0 = g*M + first row, xrow0 = k steps, a_rg / b_rg = operand row groups).
+// group's place in k space, and its items of the two weight-gradient products (all 256 x 256 tiles of dW_g;
+// descriptor: row0 = g*M + first row, xrow0 = k steps, a_rg / b_rg = operand row groups).
 __global__ __launch_bounds__(256) void bw_tables_kernel(int32_t *__restrict__ tile_meta, const int32_t *__restrict__ counts,
                                                         int E, int Es, int T, int bm, omega_tile_desc *__restrict__ desc_da,
                                                         int nt_da, int32_t *__restrict__ kt0,
@@ -512,8 +512,11 @@ __global__ __launch_bounds__(256) void bw_tables_kernel(int32_t *__restrict__ ti
     for (int pass = 0; pass < 2; ++pass) {
         omega_tile_desc *desc = pass == 0 ? desc_w2 : desc_w13;
         const int M = pass == 0 ? M2 : M13, MT = M / 256, NT = pass == 0 ? NT2 : NT13;
+        // the tile index with fewer values runs fastest, so that the 32 consecutive items an XCD works on at a time
+        // form a block of row tiles x column tiles that is as square as possible and share operand tiles in its L2
+        const bool m_fast = MT <= NT;
         for (int l = tid; l < MT * NT; l += 256) {
-            const int mi = l % MT, n = l / MT;
+            const int mi = m_fast ? l % MT : l / NT, n = m_fast ? l / MT : l % NT;
             omega_tile_desc dsc;
             dsc.g = g;
             dsc.row0 = g * M + mi * 256;
