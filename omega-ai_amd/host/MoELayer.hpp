@@ -111,8 +111,9 @@ public:
     ~MoELayer() override
     {
         omega_moe_destroy(moe_);
-        if (xLow_) omega_hip_free(ctx_.get(), xLow_);
-        if (outLow_) omega_hip_free(ctx_.get(), outLow_);
+        void *low[] = {xLow_, outLow_, deltaLow_, diffLow_};
+        for (void *p : low)
+            if (p) omega_hip_free(ctx_.get(), p);
     }
 
     // parameters arrive as fp32 host arrays in the reference's [out,in] layout
@@ -144,7 +145,20 @@ public:
             }
         }
     }
-    void initBack() override {}
+    // (re)allocates the input gradient when the batch size changes (FullyLayer.initBack,
+    // J/engine/nn/layer/FullyLayer.java:130-144); the parameter gradients live in the native handle
+    void initBack() override
+    {
+        if (!diff_ || diff_->number != number) {
+            diff_.reset(new Tensor(number, oChannel, oHeight, oWidth, &ctx_, true));
+            if (dtype_ == OMEGA_DTYPE_BF16) {
+                if (deltaLow_) omega_hip_free(ctx_.get(), deltaLow_);
+                if (diffLow_) omega_hip_free(ctx_.get(), diffLow_);
+                check(ctx_.get(), omega_hip_malloc(ctx_.get(), (size_t)number * embedDim_ * 2, &deltaLow_));
+                check(ctx_.get(), omega_hip_malloc(ctx_.get(), (size_t)number * embedDim_ * 2, &diffLow_));
+            }
+        }
+    }
     void initParam() override {}
     void output() override { run(false); }
     // second half of the transformer block in one call: output = input + layer(rmsnorm(input))
@@ -170,11 +184,52 @@ public:
         init();
         output();
     }
-    void diff() override { unsupported(); }
-    void back() override { unsupported(); }
-    void back(Tensor &) override { unsupported(); }
-    void update() override { unsupported(); }
-    void accGrad(float) override { unsupported(); }
+    // back(Tensor delta) = initBack -> setDelta -> diff (LlamaMLPLayer.back, J/engine/nn/layer/llama/LlamaMLPLayer.java:186-199);
+    // must follow forward(Tensor) of the same input.  The input gradient is getDiff(); the parameter gradients are
+    // overwritten inside the handle (grad()).
+    void back(Tensor &delta) override
+    {
+        if (!input || !output_) throw std::runtime_error("Error code 1:back without a forward");
+        if (delta.number != number || delta.width != embedDim_ || !delta.isHasGPU())
+            throw std::runtime_error("Error code 1:delta shape does not match the output or tensor has no device data");
+        initBack();
+        delta_ = &delta;
+        diff();
+    }
+    void back() override
+    {
+        if (!delta_) throw std::runtime_error("Error code 1:back() without a delta");
+        initBack();
+        diff();
+    }
+    void diff() override
+    {
+        const size_t n = (size_t)number * embedDim_;
+        if (dtype_ == OMEGA_DTYPE_BF16) {
+            // xLow_ still holds the input of the forward call
+            check(ctx_.get(), omega_hip_convert(ctx_.get(), deltaLow_, OMEGA_DTYPE_BF16, delta_->gpuData, OMEGA_DTYPE_F32, n));
+            check(ctx_.get(), omega_moe_backward(moe_, xLow_, deltaLow_, number, diffLow_));
+            check(ctx_.get(), omega_hip_convert(ctx_.get(), diff_->gpuData, OMEGA_DTYPE_F32, diffLow_, OMEGA_DTYPE_BF16, n));
+        } else {
+            check(ctx_.get(), omega_moe_backward(moe_, input->gpuData, delta_->gpuData, number, diff_->gpuData));
+        }
+    }
+    Tensor *getDiff() { return diff_.get(); }
+    // forward keeps h1 / h3 for back(), as the reference's layers keep their outputs
+    void setTraining(bool on) { check(ctx_.get(), omega_moe_set_training(moe_, on ? 1 : 0)); }
+    // update() of a layer without an updater: w -= learnRate * diffW (FullyLayer.update, FullyLayer.java:569-590)
+    float learnRate = 0.0f;
+    void update() override { check(ctx_.get(), omega_moe_update(moe_, learnRate)); }
+    void accGrad(float scale) override { check(ctx_.get(), omega_moe_acc_grad(moe_, scale)); }
+    // one parameter gradient (fp32, layout of its weight): OMEGA_W_GATE, OMEGA_W_GATE_BIAS, OMEGA_W_W1 / W3 / W2 of expert g
+    std::vector<float> grad(int which, int g = 0)
+    {
+        const size_t n = which == OMEGA_W_GATE ? (size_t)nExperts_ * embedDim_ : which == OMEGA_W_GATE_BIAS ? (size_t)nExperts_
+                                                                                                            : (size_t)hidden_ * embedDim_;
+        std::vector<float> h(n);
+        check(ctx_.get(), omega_moe_get_grad(moe_, which, g, h.data(), 0));
+        return h;
+    }
     const char *getLayerType() const override { return "feed_forward"; }
 
     void getRouting(std::vector<int32_t> &ids, std::vector<float> &w, std::vector<int32_t> &counts)
@@ -201,7 +256,6 @@ private:
             check(ctx_.get(), fwd(moe_, input->gpuData, number, output_->gpuData));
         }
     }
-    [[noreturn]] static void unsupported() { throw std::logic_error("MoELayer is forward-only"); }
     template <class F> void eachParam(F f)
     {
         f(OMEGA_W_GATE, 0, (size_t)nExperts_ * embedDim_);
@@ -253,8 +307,9 @@ private:
     int embedDim_, hidden_, nExperts_, topK_, nShared_;
     bool bias_;
     int dtype_;
-    std::unique_ptr<Tensor> output_;
-    void *xLow_ = nullptr, *outLow_ = nullptr;
+    std::unique_ptr<Tensor> output_, diff_;
+    Tensor *delta_ = nullptr;
+    void *xLow_ = nullptr, *outLow_ = nullptr, *deltaLow_ = nullptr, *diffLow_ = nullptr;
 };
 
 }  // namespace omega

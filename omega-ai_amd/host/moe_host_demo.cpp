@@ -1,7 +1,7 @@
 // Drives omega::MoELayer the way a transformer block drives its FFN slot
 // (J/engine/nn/layer/llama/LlamaTransformerBlock.java:135: getMlp().forward(norm2.getOutput())).
-// Reads inputs and weights as raw little-endian float32 files, runs forward, writes the output and
-// the routing; used by tests/test_gpu_host_cpp.py, which compares against the CPU oracle.
+// Reads inputs and weights as raw little-endian float32 files, runs forward (and backward, block form), writes the
+// outputs and the routing; used by tests/test_gpu_host_cpp.py, which compares against the CPU oracle.
 //   moe_host_demo <dir> T d E K H Es renorm dtype(0|1)
 #include <cstdlib>
 #include <cstring>
@@ -45,6 +45,26 @@ int main(int argc, char **argv)
         FILE *fi = fopen((dir + "/ids.bin").c_str(), "wb");
         fwrite(ids.data(), 4, ids.size(), fi);
         fclose(fi);
+        // backward, when the directory holds an output gradient: dx and two parameter gradients
+        if (FILE *fd = fopen((dir + "/dout.bin").c_str(), "rb")) {
+            fclose(fd);
+            omega::Tensor delta(T, 1, 1, d, &ctx, true);
+            delta.data = read_f32(dir + "/dout.bin", (size_t)T * d);
+            delta.hostToDevice();
+            mlp.back(delta);
+            omega::Tensor *dx = mlp.getDiff();
+            dx->syncHost();
+            FILE *fx = fopen((dir + "/dx.bin").c_str(), "wb");
+            fwrite(dx->data.data(), 4, dx->data.size(), fx);
+            fclose(fx);
+            const std::vector<float> g2 = mlp.grad(OMEGA_W_W2, E - 1), gg = mlp.grad(OMEGA_W_GATE);
+            FILE *fg2 = fopen((dir + "/dW2_last.bin").c_str(), "wb");
+            fwrite(g2.data(), 4, g2.size(), fg2);
+            fclose(fg2);
+            FILE *fgg = fopen((dir + "/dWg.bin").c_str(), "wb");
+            fwrite(gg.data(), 4, gg.size(), fgg);
+            fclose(fgg);
+        }
         // block form (norm2 -> mlp -> residual add), when the directory holds the norm weight
         if (FILE *fg = fopen((dir + "/gamma.bin").c_str(), "rb")) {
             fclose(fg);
@@ -66,8 +86,10 @@ int main(int argc, char **argv)
         bool raised = false;
         try { mlp.forward(bad); } catch (const std::runtime_error &) { raised = true; }
         if (!raised) throw std::runtime_error("mismatching input was accepted");
-        try { mlp.update(); raised = false; } catch (const std::logic_error &) { raised = true; }
-        if (!raised) throw std::runtime_error("update() did not raise");
+        // a backward pass must follow a plain forward: after forwardBlock / a failed forward it raises
+        omega::Tensor delta2(T, 1, 1, d + 1, &ctx, true);
+        try { mlp.back(delta2); raised = false; } catch (const std::runtime_error &) { raised = true; }
+        if (!raised) throw std::runtime_error("mismatching delta was accepted");
         printf("ok layerType=%s T=%d\n", mlp.getLayerType(), T);
         return 0;
     } catch (const std::exception &e) {

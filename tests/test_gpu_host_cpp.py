@@ -30,6 +30,10 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
         model.astype("<f4").tofile(os.path.join(td, "model.bin"))
         gamma = (O.fill_normal(cfg.d, 17, C.STREAM_NORM, 1.0) * np.float32(0.1) + np.float32(1.0)).astype(np.float32)
         gamma.astype("<f4").tofile(os.path.join(td, "gamma.bin"))
+        dout = O.fill_normal(cfg.T * cfg.d, 17, 900, 1.0).reshape(cfg.T, cfg.d)
+        if dtype == "bf16":
+            dout = O.round_bf16(dout)
+        dout.astype("<f4").tofile(os.path.join(td, "dout.bin"))
         r = subprocess.run([DEMO, td, str(cfg.T), str(cfg.d), str(cfg.E), str(cfg.K), str(cfg.H), str(cfg.Es), "1",
                             "1" if dtype == "bf16" else "0"], capture_output=True, text=True, timeout=100)
         assert r.returncode == 0, r.stderr
@@ -38,6 +42,9 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
         ids = np.fromfile(os.path.join(td, "ids.bin"), "<i4").reshape(cfg.T, cfg.K)
         saved = np.fromfile(os.path.join(td, "model_saved.bin"), "<f4")
         out_block = np.fromfile(os.path.join(td, "out_block.bin"), "<f4").reshape(cfg.T, cfg.d)
+        dx = np.fromfile(os.path.join(td, "dx.bin"), "<f4").reshape(cfg.T, cfg.d)
+        dW2_last = np.fromfile(os.path.join(td, "dW2_last.bin"), "<f4").reshape(cfg.d, cfg.H)
+        dWg = np.fromfile(os.path.join(td, "dWg.bin"), "<f4").reshape(cfg.E, cfg.d)
     ref = O.moe_forward(inp["x"], inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es, bf16=dtype == "bf16")
     assert np.array_equal(ids, ref["ids"])
     assert N.rel_l2(out, ref["out"]) <= (1e-2 if dtype == "bf16" else 1e-5)
@@ -45,3 +52,8 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
     blk = O.block_forward(inp["x"], gamma, inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es,
                           bf16=dtype == "bf16")
     assert N.rel_l2(out_block, blk["out"]) <= (1e-2 if dtype == "bf16" else 1e-5)   # forwardBlock of the C++ layer
+    bw = O.moe_backward(inp["x"], dout, inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es,
+                        bf16=dtype == "bf16")
+    tol = 1e-2 if dtype == "bf16" else 1e-5
+    assert N.rel_l2(dx, bw["dx"]) <= tol                                            # back(Tensor) of the C++ layer
+    assert N.rel_l2(dW2_last, bw["dW2"][cfg.E - 1]) <= tol and N.rel_l2(dWg, bw["dWg"]) <= tol
