@@ -27,7 +27,7 @@ PEAK_HBM_GBPS = 8000.0
 
 # HBM traffic per launch of the dominant kernel from the committed rocprofv3 --pmc runs
 # (profiles/experts_bf16_c2_mixtral_pmc.txt): FETCH_SIZE + WRITE_SIZE in bytes, scaled by the copy-kernel factor.
-TRAFFIC_BYTES = {"c2_mixtral": 5.12e9}
+TRAFFIC_BYTES = {"c2_mixtral": 4.94e9}
 
 
 def main():
@@ -150,7 +150,7 @@ def main():
         "config": {"workload": f"{cfg.name}: T={cfg.T} ({cfg.batch}x{cfg.seq}) d={cfg.d} E={cfg.E} K={cfg.K} H={cfg.H} "
                                f"Es={cfg.Es} renorm={int(cfg.renorm)} {cfg.dtype}, fp32 accumulate",
                    "router_mode": a.router, "seed": a.seed},
-        "roofline": {"bound": "mfma", "kernel": "experts_bf16_kernel<up>: a = silu(xg W1^T) * (xg W3^T)",
+        "roofline": {"bound": "mfma", "kernel": "experts_bf16_kernel<0> (up): a = silu(xg W1^T) * (xg W3^T)",
                      "achieved": up_tflops, "peak": peak, "unit": "TFLOP/s", "frac": up_tflops / peak,
                      "algorithmic_flops_per_launch": up_flops, "avg_launch_ms": stage_ms["experts_up"],
                      "traffic": TRAFFIC_BYTES.get(cfg.name),
