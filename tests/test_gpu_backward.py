@@ -216,3 +216,39 @@ def test_backward_full_size_mixtral():
     for gt, wt, nm in ((got2, want2, "dW2"), (got1, want1, "dW1"), (got3, want3, "dW3")):
         assert N.rel_l2(np.array(gt), np.array(wt)) < 1e-3, (nm, gt, wt)
     layer.close()
+
+
+def test_backward_call_order_and_growth():
+    """Error paths and workspace growth: a backward pass must follow a plain forward of the same T; a larger batch after a
+    smaller one regrows both workspaces, in training mode too."""
+    G, cfg, inp, dout, layer = _setup("c2_mixtral", dict(T=64, d=256, H=256, E=4, K=2), 3)
+    P = G.P
+    x = P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    layer.set_norm(np.ones(cfg.d, np.float32))
+    layer.forward_block(x)
+    with pytest.raises(RuntimeError):          # the block form has no backward pass
+        layer.back(g)
+    layer.forward(x)
+    layer.stage("router", x)
+    with pytest.raises(RuntimeError):          # a stage run on its own invalidates the forward
+        layer.back(g)
+    with pytest.raises(RuntimeError):          # update on a bf16 layer: no fp32 master weights
+        layer.forward(x); layer.back(g); layer.update(0.1)
+    dx_small = layer.back(g).to_numpy()
+    # a batch four times as large (new workspace), training mode on, then the small one again
+    cfg2 = scaled(cfg, T=256)
+    inp2 = make_inputs(cfg2, 4)
+    dout2 = O.round_bf16(O.fill_normal(cfg2.T * cfg2.d, 4, 900, 1.0).reshape(cfg2.T, cfg2.d))
+    x2 = P.DeviceBuffer.from_numpy(G.ctx(), inp2["x"], cfg.dtype)
+    g2 = P.DeviceBuffer.from_numpy(G.ctx(), dout2, cfg.dtype)
+    layer.set_training(True)
+    layer.forward(x2)
+    dx2 = layer.back(g2).to_numpy()
+    ref2 = O.moe_backward(inp2["x"], dout2, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es,
+                          bf16=True)
+    assert N.rel_l2(dx2, ref2["dx"]) < 1e-2
+    assert N.rel_l2(layer.grad(L.W_W2, 1), ref2["dW2"][1]) < 1e-2
+    layer.forward(x)
+    assert np.array_equal(layer.back(g).to_numpy(), dx_small)
+    layer.close()
