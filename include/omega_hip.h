@@ -140,6 +140,14 @@ int omega_moe_get_norm(omega_moe *moe, int T, float *rms_host);
  * softmax_back (J/engine/gpu/SoftmaxKernel.cu:101-112) -> gate linear layer.  The expert ids and the permutation carry
  * no gradient.  Asynchronous on the context's stream. */
 int omega_moe_backward(omega_moe *moe, const void *x_dev, const void *dout_dev, int T, void *dx_dev);
+/* Backward of the block form, after omega_moe_forward_block of the same x_dev and T:
+ *   getMlp().back(delta); getNorm2().back(getMlp().diff); Tensor_OP().add(getNorm2().diff, delta, getNorm2().diff)
+ * (J/engine/nn/layer/llama/LlamaTransformerBlock.java:156-158), the norm backward being rmsnorm_backward_kernel2
+ * (J/engine/nn/layer/normalization/gpu/RMSKernel.cu:226-277, launched by RMSLayer.diff, RMSLayer.java:292).  The layer's
+ * input gradient stays inside the library; dx_dev receives dout + norm backward of it (one rounding in bf16 layers), and
+ * the gradient of the norm weight becomes available as omega_moe_get_grad(moe, OMEGA_W_NORM, ...) (it is zero after a
+ * plain omega_moe_backward).  The weight gradient is summed in a fixed order (the reference uses atomicAdd). */
+int omega_moe_backward_block(omega_moe *moe, const void *x_dev, const void *dout_dev, int T, void *dx_dev);
 /* Training mode (off at creation).  The reference's layers keep their outputs for back() (LlamaMLPLayer.diff reads
  * active.getOutput() and getLinear3().getOutput(), J/engine/nn/layer/llama/LlamaMLPLayer.java:148-152); with training
  * on, omega_moe_forward of a bf16 layer likewise stores h1 and h3 (fp32, from the accumulators of its up product) and
@@ -147,7 +155,7 @@ int omega_moe_backward(omega_moe *moe, const void *x_dev, const void *dout_dev, 
  * 8*H bytes more per expert row.  fp32 layers ignore the switch. */
 int omega_moe_set_training(omega_moe *moe, int on);
 /* One parameter gradient of the last omega_moe_backward, always fp32, in the layout of the weight it belongs to
- * (which / expert as for omega_moe_set_weights; OMEGA_W_NORM has none).  Stands in for reading layer.diffW / diffB
+ * (which / expert as for omega_moe_set_weights).  Stands in for reading layer.diffW / diffB
  * (LlamaMLPLayer.putParamterGrads, J/engine/nn/layer/llama/LlamaMLPLayer.java:285-295). */
 int omega_moe_get_grad(omega_moe *moe, int which, int expert, void *dst, int is_device);
 /* accGrad(scale): the first call after an update copies the gradients into the accumulators, later calls add

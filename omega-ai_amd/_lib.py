@@ -47,6 +47,7 @@ SIGNATURES = {
     "omega_moe_backward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "omega_moe_time_backward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int,
                                           C.POINTER(C.c_float)]),
+    "omega_moe_backward_block": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "omega_moe_set_training": (C.c_int, [C.c_void_p, C.c_int]),
     "omega_moe_get_grad": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
     "omega_moe_acc_grad": (C.c_int, [C.c_void_p, C.c_float]),

@@ -155,7 +155,7 @@ int omega_hip_convert(omega_ctx *ctx, void *dst, int dst_dtype, const void *src,
 static void moe_free_backward_workspace(omega_moe *m)
 {
     void **bw[] = {(void **)&m->bw_probs, (void **)&m->bw_dw, (void **)&m->bw_dlogits, (void **)&m->bw_gpart, (void **)&m->bw_dy, (void **)&m->bw_h1,
-                   (void **)&m->bw_h3, (void **)&m->bw_dxg, &m->bw_dy16, &m->bw_dys16, &m->bw_dh16, &m->bw_dyT, &m->bw_aT,
+                   (void **)&m->bw_h3, (void **)&m->bw_dxg, &m->bw_dhx, &m->bw_dy16, &m->bw_dys16, &m->bw_dh16, &m->bw_dyT, &m->bw_aT,
                    &m->bw_xgT, &m->bw_dhT, (void **)&m->bw_kt0, (void **)&m->desc_da, (void **)&m->wq_da,
                    (void **)&m->desc_w2, (void **)&m->wq_w2, (void **)&m->desc_w13, (void **)&m->wq_w13};
     for (void **p : bw) {
@@ -183,8 +183,8 @@ static void moe_free_workspace(omega_moe *m)
 static size_t grad_block_floats(const omega_moe *m)
 {
     const omega_moe_config &c = m->cfg;
-    // dWg, dbg (rounded up to whole 16-byte units, so the expert gradients stay 16-byte aligned), dW13, dW2
-    return (size_t)c.E * c.d + (size_t)((c.E + 3) & ~3) + 3 * (size_t)m->G * c.H * c.d;
+    // dWg, dbg and dgamma (each rounded up to whole 16-byte units, so the expert gradients stay 16-byte aligned), dW13, dW2
+    return (size_t)c.E * c.d + (size_t)((c.E + 3) & ~3) + (size_t)((c.d + 3) & ~3) + 3 * (size_t)m->G * c.H * c.d;
 }
 
 // Gradient buffers (once) and the workspace of the backward pass for the current forward workspace.
@@ -200,7 +200,8 @@ static int moe_reserve_backward(omega_moe *m, int T)
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(blk, 0, grad_block_floats(m) * 4, ctx->stream));
         m->dWg = blk;
         m->dbg = m->dWg + (size_t)c.E * c.d;
-        m->dW13 = m->dbg + ((c.E + 3) & ~3);
+        m->dgamma = m->dbg + ((c.E + 3) & ~3);
+        m->dW13 = m->dgamma + ((c.d + 3) & ~3);
         m->dW2 = m->dW13 + 2 * (size_t)m->G * HD;
     }
     if (bf && !m->W2T) {
@@ -226,6 +227,7 @@ static int moe_reserve_backward(omega_moe *m, int T)
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dw, (size_t)Tc * c.K * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dlogits, (size_t)Tc * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_gpart, (size_t)32 * c.E * c.d * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc(&m->bw_dhx, (size_t)Tc * c.d * m->esize));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h1, rc * c.H * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_h3, rc * c.H * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_dxg, rc * c.d * 4));
@@ -517,6 +519,7 @@ static int check_T(omega_moe *m, const void *x, int T, bool need_x)
 static void stage_invalidates(omega_moe *m)
 {
     m->fwd_T = -1;
+    m->fwd_block = false;
     m->rec_valid = false;
 }
 
@@ -573,9 +576,10 @@ static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block
     // block form: the layer runs on the normalised rows h (one small kernel writes them and rms), the combine adds x back
     const void *resid = block ? x : nullptr;
     const void *xin = block ? m->hbuf : x;
-    m->fwd_T = block ? -1 : T;
+    m->fwd_T = T;
+    m->fwd_block = block != 0;
     // training mode (bf16 layers): the up product also leaves h1 / h3 for the backward pass
-    const bool keep = m->training && !block && m->cfg.dtype == OMEGA_DTYPE_BF16;
+    const bool keep = m->training && m->cfg.dtype == OMEGA_DTYPE_BF16;
     if (keep) {
         m->bm = moe_tile_m(m, T);
         RUN(moe_reserve_backward(m, T));
@@ -637,24 +641,44 @@ int omega_moe_forward_block(omega_moe *m, const void *x, int T, void *out)
     return forward_impl(m, x, T, out, 1);
 }
 
-int omega_moe_backward(omega_moe *m, const void *x, const void *dout, int T, void *dx)
+static int backward_impl(omega_moe *m, const void *x, const void *dout, int T, void *dx, bool block)
 {
-    MOE_ENTER(m);
+    omega_ctx *ctx = m->ctx;
     RUN(check_T(m, x, T, true));
-    if (T != m->fwd_T) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "backward: no omega_moe_forward has run for this T");
+    if (T != m->fwd_T || block != m->fwd_block)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, block ? "backward_block: no omega_moe_forward_block has run for this T"
+                                                     : "backward: no omega_moe_forward has run for this T");
     if (T == 0) return OMEGA_OK;
     if (!dout || !dx) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "backward: dout or dx is NULL");
     RUN(moe_reserve_backward(m, T));
-    if (m->cfg.dtype == OMEGA_DTYPE_BF16) OMEGA_HIP_CHECK(ctx, launch_backward_bf16(m, x, dout, T, dx, ctx->stream));
-    else OMEGA_HIP_CHECK(ctx, launch_backward_f32(m, x, dout, T, dx, ctx->stream));
+    const bool bf = m->cfg.dtype == OMEGA_DTYPE_BF16;
+    // block form: the layer ran on the normalised rows it still holds; its input gradient then passes the norm backwards
+    // and meets the gradient of the residual branch
+    const void *xin = block ? m->hbuf : x;
+    void *dxl = block ? m->bw_dhx : dx;
+    OMEGA_HIP_CHECK(ctx, bf ? launch_backward_bf16(m, xin, dout, T, dxl, ctx->stream) : launch_backward_f32(m, xin, dout, T, dxl, ctx->stream));
+    if (block) OMEGA_HIP_CHECK(ctx, launch_rmsnorm_backward(m, x, m->bw_dhx, dout, T, dx, ctx->stream));
+    else OMEGA_HIP_CHECK(ctx, launch_zero_f32(m->dgamma, (size_t)m->cfg.d, ctx->stream));  // the norm took no part
     return OMEGA_OK;
+}
+
+int omega_moe_backward(omega_moe *m, const void *x, const void *dout, int T, void *dx)
+{
+    MOE_ENTER(m);
+    return backward_impl(m, x, dout, T, dx, false);
+}
+
+int omega_moe_backward_block(omega_moe *m, const void *x, const void *dout, int T, void *dx)
+{
+    MOE_ENTER(m);
+    return backward_impl(m, x, dout, T, dx, true);
 }
 
 int omega_moe_time_backward(omega_moe *m, const void *x, const void *dout, int T, void *dx, int warmup, int iters, float *ms_avg)
 {
     MOE_ENTER(m);
     RUN(check_T(m, x, T, true));
-    if (T <= 0 || T != m->fwd_T) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_backward: no omega_moe_forward has run for this T");
+    if (T <= 0 || T != m->fwd_T || m->fwd_block) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_backward: no omega_moe_forward has run for this T");
     if (!dout || !dx || !ms_avg || iters <= 0 || warmup < 0) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_backward: bad argument");
     RUN(moe_reserve_backward(m, T));
     const bool bf = m->cfg.dtype == OMEGA_DTYPE_BF16;
@@ -677,6 +701,7 @@ static int grad_slot(omega_moe *m, int which, int expert, float **ptr, size_t *f
     switch (which) {
         case OMEGA_W_GATE: *ptr = m->dWg; *floats = (size_t)c.E * c.d; return OMEGA_OK;
         case OMEGA_W_GATE_BIAS: *ptr = m->dbg; *floats = (size_t)c.E; return OMEGA_OK;
+        case OMEGA_W_NORM: *ptr = m->dgamma; *floats = (size_t)c.d; return OMEGA_OK;
         case OMEGA_W_W1: case OMEGA_W_W3: case OMEGA_W_W2:
             if (expert < 0 || expert >= m->G) return OMEGA_ERR_INVALID_ARG;
             *ptr = which == OMEGA_W_W2 ? m->dW2 + per * (size_t)expert
@@ -727,6 +752,7 @@ int omega_moe_update(omega_moe *m, float lr)
     const size_t per = (size_t)c.H * c.d;
     OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->Wg, m->dWg, -lr, (size_t)c.E * c.d, ctx->stream));
     if (c.has_gate_bias) OMEGA_HIP_CHECK(ctx, launch_axpy_f32(m->bg, m->dbg, -lr, (size_t)c.E, ctx->stream));
+    if (m->gamma_set) OMEGA_HIP_CHECK(ctx, launch_axpy_f32(m->gamma, m->dgamma, -lr, (size_t)c.d, ctx->stream));
     for (int g = 0; g < m->G; ++g) {
         OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W1 + per * g, m->dW13 + per * 2 * g, -lr, per, ctx->stream));
         OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W3 + per * g, m->dW13 + per * (2 * g + 1), -lr, per, ctx->stream));

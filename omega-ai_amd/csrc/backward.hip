@@ -400,6 +400,20 @@ __global__ __launch_bounds__(256) void bw_axpy_kernel(float *__restrict__ dst, c
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = fmaf(scale, src[i], dst[i]);
 }
 
+__global__ __launch_bounds__(256) void bw_zero_kernel(float *__restrict__ dst, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = 0.0f;
+}
+
+// a fill kernel, not a memset node: safe inside a captured graph
+hipError_t launch_zero_f32(float *dst, size_t n, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    const int grid = (int)((n + 255) / 256 < 1024 ? (n + 255) / 256 : 1024);
+    hipLaunchKernelGGL(bw_zero_kernel, dim3(grid), dim3(256), 0, s, dst, n);
+    return hipGetLastError();
+}
+
 hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, hipStream_t s)
 {
     if (n == 0) return hipSuccess;

@@ -91,8 +91,8 @@ struct omega_moe {
     // backward pass (allocated by the first omega_moe_backward): parameter gradients, always fp32, in the layout of
     // their weights, the accumulators of accGrad, and the workspace of the pass, indexed by physical rows like xg / a / y
     // (dW13: [G][2][H,d], the gradients of W1 and W3 of an expert back to back)
-    float *dWg = nullptr, *dbg = nullptr, *dW13 = nullptr, *dW2 = nullptr;
-    float *acc_grad = nullptr;       // accumulators, one block in the order dWg, dbg, dW13, dW2
+    float *dWg = nullptr, *dbg = nullptr, *dgamma = nullptr, *dW13 = nullptr, *dW2 = nullptr;
+    float *acc_grad = nullptr;       // accumulators, one block in the order dWg, dbg, dgamma, dW13, dW2
     bool acc_valid = false;          // accGrad has run since the last update
     float *bw_probs = nullptr;       // [T,E] softmax of the gate logits
     float *bw_dw = nullptr;          // [T,K] gradient of the combine weights
@@ -117,7 +117,9 @@ struct omega_moe {
     bool wT_valid = false;           // the transposed copies match the weights
     int bw_T_cap = 0;
     size_t bw_rows_cap = 0;
-    int fwd_T = -1;                  // tokens of the last plain forward (what backward may follow), -1: none
+    int fwd_T = -1;                  // tokens of the last forward (what a backward pass may follow), -1: none
+    bool fwd_block = false;          // ... and whether it was the block form
+    void *bw_dhx = nullptr;          // [T,d] layer dtype: input gradient of the layer inside the block form
     bool training = false;           // forward keeps h1 / h3 (bf16 layers: as block records in bw_h1 / bw_h3)
     bool rec_valid = false;          // bw_h1 / bw_h3 hold h1 / h3 of the last forward
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -149,6 +151,8 @@ hipError_t launch_convert(void *dst, int dst_dtype, const void *src, int src_dty
 
 // h[t,:] = (x[t,:] / rms[t]) * gamma in the layer's storage type, rms[t] into m->rms; h == nullptr: statistics only
 hipError_t launch_rmsnorm(const omega_moe *m, const void *x, int T, void *h, hipStream_t s);
+hipError_t launch_rmsnorm_backward(const omega_moe *m, const void *x, const void *dh, const void *resid, int T, void *dx,
+                                   hipStream_t s);
 hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s);
 hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s);
 hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipStream_t s);
@@ -167,6 +171,7 @@ hipError_t launch_transpose_images(const void *src, int R, int cols, void *dst, 
 enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4, MODE_UPREC = 5 };
 hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, const void *Aalt, const void *Wa, const void *Wb,
                                void *Cout, void *Aux1, void *Aux2, const omega_tile_desc *wq, int N, int Kd, hipStream_t s);
+hipError_t launch_zero_f32(float *dst, size_t n, hipStream_t s);
 hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, hipStream_t s);
 hipError_t launch_mfma_probe(float *scratch, int num_cus, int random_operands, int launches, hipStream_t s,
                              double *flop_per_launch);

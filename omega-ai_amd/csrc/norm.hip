@@ -138,3 +138,93 @@ hipError_t launch_rmsnorm(const omega_moe *m, const void *x, int T, void *h, hip
         hipLaunchKernelGGL(rmsnorm_kernel<false>, dim3(grid), dim3(256), 0, s, x, m->gamma, T, c.d, m->rms, h);
     return hipGetLastError();
 }
+
+// ---- backward of the pre-norm (block form) ----
+// rmsnorm_backward_kernel2 (J/engine/nn/layer/normalization/gpu/RMSKernel.cu:226-277): per row, with the forward's rms,
+//   drms = sum_i x[i]*dh[i]*w[i] (lane l adds i = l, l+32, ... in order: product x*dh, then one fused multiply-add with w;
+//          xor butterfly over the 32 lanes) * (-1 / (rms^3 * C))
+//   dx[i] = dh[i]*w[i]/rms + drms*x[i]   (+ resid[i]: the gradient that bypasses the norm, Tensor_OP().add(norm2.diff, delta),
+//          J/engine/nn/layer/llama/LlamaTransformerBlock.java:157-158), rounded once in bf16 layers
+// 8 rows x 32 lanes per workgroup, rows read straight from memory (this kernel moves 4 rows of T x d once).
+template <bool XBF>
+__global__ __launch_bounds__(256) void rmsnorm_backward_kernel(const void *__restrict__ x, const void *__restrict__ dh,
+                                                               const float *__restrict__ gamma, const float *__restrict__ rms,
+                                                               const void *__restrict__ resid, int T, int d, void *__restrict__ dx)
+{
+    const int r = threadIdx.x >> 5, l = threadIdx.x & 31;
+    const int t = blockIdx.x * NORM_ROWS + r;
+    if (t >= T) return;  // whole 32-lane groups leave together; the shuffles below stay within a group
+    const size_t base = (size_t)t * d;
+    auto ld = [&](const void *p, int i) {
+        return XBF ? bf16_to_f32(((const bf16_t *)p)[base + i]) : ((const float *)p)[base + i];
+    };
+    float s = 0.0f;
+    for (int i = l; i < d; i += 32) {
+        const float pr = ld(x, i) * ld(dh, i);
+        s = fmaf(pr, gamma[i], s);
+    }
+#pragma unroll
+    for (int m = 16; m >= 1; m >>= 1) s = s + __shfl_xor(s, m, 32);
+    const float rv = rms[t];
+    const float drms = s * (-1.0f / (rv * rv * rv * (float)d));
+    for (int i = l; i < d; i += 32) {
+        const float a = ld(dh, i) * gamma[i];
+        const float q = a / rv;
+        float v = fmaf(drms, ld(x, i), q);
+        if (resid != nullptr) v = v + ld(resid, i);
+        if (XBF) ((bf16_t *)dx)[base + i] = f32_to_bf16(v);
+        else ((float *)dx)[base + i] = v;
+    }
+}
+
+// dgamma[c] = sum_t (x[t,c]/rms[t]) * dh[t,c]: partial sums over 32 slices of the rows (fixed order, no atomics; the
+// reference accumulates with atomicAdd in no defined order), then their sum.
+template <bool XBF>
+__global__ __launch_bounds__(256) void rmsnorm_dgamma_partial_kernel(const void *__restrict__ x, const void *__restrict__ dh,
+                                                                     const float *__restrict__ rms, int T, int d, int tslice,
+                                                                     float *__restrict__ part)
+{
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= d) return;
+    const int t0 = blockIdx.y * tslice, t1 = min(T, t0 + tslice);
+    float acc = 0.0f;
+    for (int t = t0; t < t1; ++t) {
+        const size_t o = (size_t)t * d + c;
+        const float xv = XBF ? bf16_to_f32(((const bf16_t *)x)[o]) : ((const float *)x)[o];
+        const float gv = XBF ? bf16_to_f32(((const bf16_t *)dh)[o]) : ((const float *)dh)[o];
+        const float n = xv / rms[t];
+        const float pr = n * gv;
+        acc = acc + pr;
+    }
+    part[(size_t)blockIdx.y * d + c] = acc;
+}
+
+__global__ __launch_bounds__(256) void rmsnorm_dgamma_reduce_kernel(const float *__restrict__ part, int nslices, int d,
+                                                                    float *__restrict__ dgamma)
+{
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= d) return;
+    float s = 0.0f;
+    for (int q = 0; q < nslices; ++q) s = s + part[(size_t)q * d + c];
+    dgamma[c] = s;
+}
+
+// dx = resid + rmsnorm backward of dh; dgamma into m->dgamma (partials in m->bw_gpart: at least 32 x d floats)
+hipError_t launch_rmsnorm_backward(const omega_moe *m, const void *x, const void *dh, const void *resid, int T, void *dx,
+                                   hipStream_t s)
+{
+    const omega_moe_config &c = m->cfg;
+    const int grid = ceil_div(T, NORM_ROWS);
+    const int tslice = ceil_div(T, 32), nsl = ceil_div(T, tslice);
+    const dim3 pg(ceil_div(c.d, 256), nsl);
+    if (c.dtype == OMEGA_DTYPE_BF16) {
+        hipLaunchKernelGGL(rmsnorm_backward_kernel<true>, dim3(grid), dim3(256), 0, s, x, dh, m->gamma, m->rms, resid, T, c.d, dx);
+        hipLaunchKernelGGL(rmsnorm_dgamma_partial_kernel<true>, pg, dim3(256), 0, s, x, dh, m->rms, T, c.d, tslice, m->bw_gpart);
+    } else {
+        hipLaunchKernelGGL(rmsnorm_backward_kernel<false>, dim3(grid), dim3(256), 0, s, x, dh, m->gamma, m->rms, resid, T, c.d, dx);
+        hipLaunchKernelGGL(rmsnorm_dgamma_partial_kernel<false>, pg, dim3(256), 0, s, x, dh, m->rms, T, c.d, tslice, m->bw_gpart);
+    }
+    hipLaunchKernelGGL(rmsnorm_dgamma_reduce_kernel, dim3(ceil_div(c.d, 256)), dim3(256), 0, s, (const float *)m->bw_gpart, nsl,
+                       c.d, m->dgamma);
+    return hipGetLastError();
+}

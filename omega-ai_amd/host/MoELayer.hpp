@@ -202,16 +202,30 @@ public:
         initBack();
         diff();
     }
-    void diff() override
+    // backward of forwardBlock: getMlp().back(delta); getNorm2().back(getMlp().diff); add(norm2.diff, delta)
+    // (J/engine/nn/layer/llama/LlamaTransformerBlock.java:156-158); getDiff() is the gradient of the block's input,
+    // grad(OMEGA_W_NORM) the gradient of the norm weight
+    void backBlock(Tensor &delta)
+    {
+        if (!input || !output_) throw std::runtime_error("Error code 1:back without a forward");
+        if (delta.number != number || delta.width != embedDim_ || !delta.isHasGPU())
+            throw std::runtime_error("Error code 1:delta shape does not match the output or tensor has no device data");
+        initBack();
+        delta_ = &delta;
+        runBack(true);
+    }
+    void diff() override { runBack(false); }
+    void runBack(bool block)
     {
         const size_t n = (size_t)number * embedDim_;
+        auto bwd = block ? omega_moe_backward_block : omega_moe_backward;
         if (dtype_ == OMEGA_DTYPE_BF16) {
             // xLow_ still holds the input of the forward call
             check(ctx_.get(), omega_hip_convert(ctx_.get(), deltaLow_, OMEGA_DTYPE_BF16, delta_->gpuData, OMEGA_DTYPE_F32, n));
-            check(ctx_.get(), omega_moe_backward(moe_, xLow_, deltaLow_, number, diffLow_));
+            check(ctx_.get(), bwd(moe_, xLow_, deltaLow_, number, diffLow_));
             check(ctx_.get(), omega_hip_convert(ctx_.get(), diff_->gpuData, OMEGA_DTYPE_F32, diffLow_, OMEGA_DTYPE_BF16, n));
         } else {
-            check(ctx_.get(), omega_moe_backward(moe_, input->gpuData, delta_->gpuData, number, diff_->gpuData));
+            check(ctx_.get(), bwd(moe_, input->gpuData, delta_->gpuData, number, diff_->gpuData));
         }
     }
     Tensor *getDiff() { return diff_.get(); }
@@ -224,8 +238,10 @@ public:
     // one parameter gradient (fp32, layout of its weight): OMEGA_W_GATE, OMEGA_W_GATE_BIAS, OMEGA_W_W1 / W3 / W2 of expert g
     std::vector<float> grad(int which, int g = 0)
     {
-        const size_t n = which == OMEGA_W_GATE ? (size_t)nExperts_ * embedDim_ : which == OMEGA_W_GATE_BIAS ? (size_t)nExperts_
-                                                                                                            : (size_t)hidden_ * embedDim_;
+        const size_t n = which == OMEGA_W_GATE        ? (size_t)nExperts_ * embedDim_
+                         : which == OMEGA_W_GATE_BIAS ? (size_t)nExperts_
+                         : which == OMEGA_W_NORM      ? (size_t)embedDim_
+                                                      : (size_t)hidden_ * embedDim_;
         std::vector<float> h(n);
         check(ctx_.get(), omega_moe_get_grad(moe_, which, g, h.data(), 0));
         return h;

@@ -76,6 +76,22 @@ int main(int argc, char **argv)
             FILE *fb = fopen((dir + "/out_block.bin").c_str(), "wb");
             fwrite(ob->data.data(), 4, ob->data.size(), fb);
             fclose(fb);
+            if (FILE *fd2 = fopen((dir + "/dout.bin").c_str(), "rb")) {
+                fclose(fd2);
+                omega::Tensor delta(T, 1, 1, d, &ctx, true);
+                delta.data = read_f32(dir + "/dout.bin", (size_t)T * d);
+                delta.hostToDevice();
+                mlp.backBlock(delta);
+                omega::Tensor *dxb = mlp.getDiff();
+                dxb->syncHost();
+                FILE *fxb = fopen((dir + "/dx_block.bin").c_str(), "wb");
+                fwrite(dxb->data.data(), 4, dxb->data.size(), fxb);
+                fclose(fxb);
+                const std::vector<float> dgm = mlp.grad(OMEGA_W_NORM);
+                FILE *fgm = fopen((dir + "/dgamma.bin").c_str(), "wb");
+                fwrite(dgm.data(), 4, dgm.size(), fgm);
+                fclose(fgm);
+            }
         }
         // round trip of the checkpoint format
         FILE *sv = fopen((dir + "/model_saved.bin").c_str(), "wb");

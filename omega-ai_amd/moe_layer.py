@@ -243,9 +243,22 @@ class MoELayer:
         self.ctx.check(self.lib.omega_moe_backward(self.handle, self.input.ptr, delta.ptr, self.number, self.diff.ptr))
         return self.diff
 
+    def back_block(self, delta):
+        """Backward of forward_block: mlp.back(delta); norm2.back(mlp.diff); add(norm2.diff, delta)
+        (J/engine/nn/layer/llama/LlamaTransformerBlock.java:156-158).  Returns the gradient of the block's input; the
+        gradient of the norm weight is grad(W_NORM)."""
+        if self.input is None:
+            raise RuntimeError("Error code 1:back without a forward")
+        if tuple(delta.shape) != (self.number, self.embedDim):
+            raise RuntimeError("Error code 1:delta shape does not match the output")
+        self.initBack()
+        self.delta = delta
+        self.ctx.check(self.lib.omega_moe_backward_block(self.handle, self.input.ptr, delta.ptr, self.number, self.diff.ptr))
+        return self.diff
+
     def grad(self, which, expert=0):
         """Host copy of one parameter gradient (fp32), in the layout of its weight."""
-        shape = {L.W_GATE: (self.nExperts, self.embedDim), L.W_GATE_BIAS: (self.nExperts,),
+        shape = {L.W_GATE: (self.nExperts, self.embedDim), L.W_GATE_BIAS: (self.nExperts,), L.W_NORM: (self.embedDim,),
                  L.W_W1: (self.hidden, self.embedDim), L.W_W3: (self.hidden, self.embedDim),
                  L.W_W2: (self.embedDim, self.hidden)}[which]
         g = np.empty(shape, np.float32)

@@ -24,6 +24,11 @@
  *                      summation order of the reference's cuBLAS products cannot be reproduced: bits "parity unpinned")
  *   orc_moe_backward_routed   the same code path with the routing passed in: equals orc_moe_backward on the same tokens
  *                      when given its routing (pinned by that identity)
+ *   orc_rmsnorm_backward / orc_block_backward   torch float64 autograd of x + layer(rmsnorm(x)) with the routing fixed,
+ *                      closed forms (gamma = 1 and dh orthogonal to x: dx = dh/rms; dh = x: dgamma = sum x^2/rms)
+ *                      (pinned to tolerance; the order of the atomicAdd accumulation of dweight over the rows is
+ *                      undefined in the reference and the additions inside cooperative_groups::reduce are library
+ *                      code: "parity unpinned" at the ulp level)
  */
 #include <stdlib.h>
 
@@ -34,6 +39,7 @@ void orc_softmax(const float *logits, int T, int E, float *p);
 void orc_topk(const float *p, int T, int E, int K, int renorm, int32_t *ids, float *w);
 void orc_dispatch(const int32_t *ids, int T, int K, int E, int32_t *counts, int32_t *offsets, int32_t *dst,
                   int32_t *src_row);
+void orc_rmsnorm(const float *x, const float *gamma, int T, int d, int bf16_mode, float *h, float *rms_o);
 
 /* Backward of the SwiGLU expert g over `rows` rows.  xin: the rows' inputs (rows x d, row r at xin + r*d); dy: their
  * output gradients (rows x d).  Writes dxin (rows x d) and OVERWRITES dW1,dW3 [H,d], dW2 [d,H] (zero when rows == 0).
@@ -283,4 +289,70 @@ void orc_moe_backward_routed(const float *x, const float *dout, const float *Wg,
 {
     backward_core(x, dout, Wg, p, ids, wid, w, W1, W3, W2, T, d, E, Ew, K, H, Es, renorm, bf16_mode, dx, NULL, NULL,
                   NULL, NULL, NULL, dw_o, dlogits_o);
+}
+
+/* Backward of the pre-norm of the block: rmsnorm_backward_kernel2 (J/engine/nn/layer/normalization/gpu/RMSKernel.cu:226-277,
+ * the kernel RMSLayer.diff launches, J/engine/nn/layer/normalization/RMSLayer.java:292 -> RMSKernel.java:296-310).
+ * Per row, one 32-lane group: rms as in the forward kernel (passed in); dweight[i] += (inp[i]/rms) * dout[i] (atomicAdd
+ * over the rows in the reference: the order of those additions is not defined there; here rows in index order);
+ * drms = sum_i inp[i]*dout[i]*weight[i], lane l adding i = l, l+32, ... in index order (the product inp*dout rounded,
+ * then one fused multiply-add with weight, nvcc's default contraction), xor butterfly over the lanes, times
+ * -1/(rms*rms*rms*C); dinp[i] = dout[i]*weight[i]/rms + drms*inp[i] (the last multiply-add fused).
+ * resid != NULL: the gradient that reaches the block's input past the norm is added (Tensor_OP().add(norm2.diff, delta),
+ * J/engine/nn/layer/llama/LlamaTransformerBlock.java:157-158) before the one rounding of bf16 mode. */
+void orc_rmsnorm_backward(const float *x, const float *dh, const float *gamma, const float *rms, const float *resid, int T,
+                          int d, int bf16_mode, float *dx, float *dgamma)
+{
+    for (int c = 0; c < d; ++c) dgamma[c] = 0.0f;
+    for (int t = 0; t < T; ++t) {
+        const float *xr = x + (size_t)t * d, *gr = dh + (size_t)t * d;
+        const float r = rms[t];
+        for (int c = 0; c < d; ++c) {
+            float n = xr[c] / r;
+            float pr = n * gr[c];
+            dgamma[c] = dgamma[c] + pr;
+        }
+        float part[32];
+        for (int l = 0; l < 32; ++l) {
+            float s = 0.0f;
+            for (int i = l; i < d; i += 32) {
+                float pr = xr[i] * gr[i];
+                s = fmaf(pr, gamma[i], s);
+            }
+            part[l] = s;
+        }
+        for (int m = 16; m >= 1; m >>= 1) {
+            float nxt[32];
+            for (int l = 0; l < 32; ++l) nxt[l] = part[l] + part[l ^ m];
+            memcpy(part, nxt, sizeof(part));
+        }
+        float drms = part[0] * (-1.0f / (r * r * r * (float)d));
+        for (int c = 0; c < d; ++c) {
+            float a = gr[c] * gamma[c];
+            float q = a / r;
+            float v = fmaf(drms, xr[c], q);
+            if (resid) v = v + resid[(size_t)t * d + c];
+            dx[(size_t)t * d + c] = bf16_mode ? bf16_round(v) : v;
+        }
+    }
+}
+
+/* Backward of the block form out = x + layer(rmsnorm(x)):
+ *   getMlp().back(delta); getNorm2().back(getMlp().diff); Tensor_OP().add(getNorm2().diff, delta, getNorm2().diff)
+ * (J/engine/nn/layer/llama/LlamaTransformerBlock.java:156-158).  The layer's input gradient dh is its `diff` (rounded to
+ * bf16 in bf16 mode, like every activation the layer hands out).  Outputs as orc_moe_backward plus dgamma [d]; dh_o [T,d]
+ * may be NULL. */
+void orc_block_backward(const float *x, const float *gamma, const float *dout, const float *Wg, const float *bg,
+                        const float *W1, const float *W3, const float *W2, int T, int d, int E, int K, int H, int Es,
+                        int renorm, int bf16_mode, float *dx, float *dgamma, float *dWg, float *dbg, float *dW1, float *dW3,
+                        float *dW2, float *dh_o)
+{
+    float *h = (float *)malloc(sizeof(float) * (size_t)T * d);
+    float *rms = (float *)malloc(sizeof(float) * (size_t)T);
+    float *dh = (float *)malloc(sizeof(float) * (size_t)T * d);
+    orc_rmsnorm(x, gamma, T, d, bf16_mode, h, rms);
+    orc_moe_backward(h, dout, Wg, bg, W1, W3, W2, T, d, E, K, H, Es, renorm, bf16_mode, dh, dWg, dbg, dW1, dW3, dW2, NULL, NULL);
+    orc_rmsnorm_backward(x, dh, gamma, rms, dout, T, d, bf16_mode, dx, dgamma);
+    if (dh_o) memcpy(dh_o, dh, sizeof(float) * (size_t)T * d);
+    free(h); free(rms); free(dh);
 }

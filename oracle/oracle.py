@@ -51,6 +51,9 @@ def lib():
         L.orc_moe_backward.argtypes = ([_f, _f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8
                                        + [_f, _f, C.c_void_p, _f, _f, _f, _f, _f])
         L.orc_moe_backward_routed.argtypes = ([_f, _f, _f, _f, _i, _i, _f, _f, _f, _f] + [C.c_int] * 9 + [_f, _f, _f])
+        L.orc_rmsnorm_backward.argtypes = [_f, _f, _f, _f, C.c_void_p, C.c_int, C.c_int, C.c_int, _f, _f]
+        L.orc_block_backward.argtypes = ([_f, _f, _f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8
+                                         + [_f, _f, _f, C.c_void_p, _f, _f, _f, _f])
         L.orc_cpu_baseline_forward.restype = C.c_double
         L.orc_cpu_baseline_forward.argtypes = [_f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8 + [_f]
         L.orc_cpu_sgemm_tn.argtypes = [C.c_int, C.c_int, C.c_int, _f, C.c_int, _f, C.c_int, _f, C.c_int, C.c_int]
@@ -204,6 +207,31 @@ def moe_backward_routed(x, dout, Wg, p, ids, wid, w, W1, W3, W2, Es, renorm, bf1
     lib().orc_moe_backward_routed(c(x, np.float32), c(dout, np.float32), c(Wg, np.float32), c(p, np.float32),
                                   c(ids, np.int32), c(wid, np.int32), c(w, np.float32), c(W1), c(W3), c(W2), n, d, E, Ew, K,
                                   H, Es, int(renorm), int(bf16), r["dx"], r["dw"], r["dlogits"])
+    return r
+
+
+def rmsnorm_backward(x, dh, gamma, rms, resid=None, bf16=False):
+    """Backward of the pre-norm: returns (dx [T,d], dgamma [d]); resid (the gradient that bypasses the norm) is added to dx."""
+    T, d = x.shape
+    dx, dg = np.empty((T, d), np.float32), np.empty(d, np.float32)
+    c = np.ascontiguousarray
+    lib().orc_rmsnorm_backward(c(x, np.float32), c(dh, np.float32), c(gamma, np.float32), c(rms, np.float32),
+                               _opt(None if resid is None else c(resid, np.float32)), T, d, int(bf16), dx, dg)
+    return dx, dg
+
+
+def block_backward(x, gamma, dout, Wg, bg, W1, W3, W2, K, renorm, Es=0, bf16=False):
+    """Backward of out = x + layer(rmsnorm(x)).  Returns dict(dx, dgamma, dWg, dbg, dW1, dW3, dW2, dh)."""
+    T, d = x.shape
+    E = Wg.shape[0]
+    G, H = W1.shape[0], W1.shape[1]
+    r = dict(dx=np.empty((T, d), np.float32), dgamma=np.empty(d, np.float32), dWg=np.empty((E, d), np.float32),
+             dbg=None if bg is None else np.empty(E, np.float32), dW1=np.empty((G, H, d), np.float32),
+             dW3=np.empty((G, H, d), np.float32), dW2=np.empty((G, d, H), np.float32), dh=np.empty((T, d), np.float32))
+    c = np.ascontiguousarray
+    lib().orc_block_backward(c(x, np.float32), c(gamma, np.float32), c(dout, np.float32), Wg, _opt(bg), W1, W3, W2, T, d, E,
+                             K, H, Es, int(renorm), int(bf16), r["dx"], r["dgamma"], r["dWg"], _opt(r["dbg"]), r["dW1"],
+                             r["dW3"], r["dW2"], r["dh"])
     return r
 
 

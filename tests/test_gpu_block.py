@@ -100,3 +100,59 @@ def test_block_forward_full_size_mixtral():
     lay = layer.forward(hbuf).to_numpy()
     assert N.rel_l2(out.astype(np.float64) - xh, lay) < 5e-2
     layer.close()
+
+
+BW_CASES = [
+    ("c1_tiny_f32", {}, False),
+    ("c1_tiny_f32", dict(T=77, d=102, H=72), False),
+    ("c4_finegrained", dict(T=96, d=128, H=64, E=8, K=3, Es=2, dtype="f32"), False),
+    ("c2_mixtral", dict(T=300, d=256, H=384), False),
+    ("c4_finegrained", dict(T=200, d=256, H=256, E=16, K=4, Es=2), True),
+    ("c5_skewed", dict(T=257, d=512, H=256, E=32, K=4), True),
+]
+
+
+@pytest.mark.parametrize("name,kw,training", BW_CASES)
+def test_block_backward_matches_oracle(name, kw, training):
+    """back_block: the layer's backward on the normalised rows, the norm backward and the residual gradient; input
+    gradient, norm weight gradient and the layer's parameter gradients against the oracle."""
+    import importlib
+    from tests import gpu_util as G
+    L = importlib.import_module("omega-ai_amd._lib")
+    cfg = scaled(C.CONFIGS[name], **kw)
+    bf = cfg.dtype == "bf16"
+    inp = make_inputs(cfg, 61)
+    inp["Wg"] = inp["Wg"] * np.float32(8.0)
+    gamma = _gamma(cfg.d, 61)
+    dout = O.fill_normal(cfg.T * cfg.d, 61, 900, 1.0).reshape(cfg.T, cfg.d)
+    if bf:
+        dout = O.round_bf16(dout)
+    layer = G.build_layer(cfg, inp)
+    layer.set_norm(gamma)
+    layer.set_training(training)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = G.P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    layer.forward(x)
+    with pytest.raises(RuntimeError):      # the last forward was the plain one
+        layer.back_block(g)
+    out = layer.forward_block(x).to_numpy()
+    with pytest.raises(RuntimeError):      # ... and now it was the block form
+        layer.back(g)
+    dx = layer.back_block(g).to_numpy()
+    ref = O.block_backward(inp["x"], gamma, dout, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm,
+                           cfg.Es, bf)
+    tol = 1e-2 if bf else 1e-5
+    assert N.rel_l2(dx, ref["dx"]) < tol, N.rel_l2(dx, ref["dx"])
+    assert N.rel_l2(layer.grad(L.W_NORM), ref["dgamma"]) < tol
+    assert N.rel_l2(layer.grad(L.W_GATE), ref["dWg"]) < tol
+    for e in (0, cfg.E + cfg.Es - 1):
+        for which, k in ((L.W_W1, "dW1"), (L.W_W3, "dW3"), (L.W_W2, "dW2")):
+            if ref[k][e].any():
+                assert N.rel_l2(layer.grad(which, e), ref[k][e]) < tol, (k, e)
+    assert np.array_equal(layer.getOutput().to_numpy(), out)
+    assert np.array_equal(layer.back_block(g).to_numpy(), dx)       # reproducible: no atomics anywhere
+    # a plain backward afterwards leaves a zero norm gradient
+    layer.forward(x)
+    layer.back(g)
+    assert not layer.grad(L.W_NORM).any()
+    layer.close()

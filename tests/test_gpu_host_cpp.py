@@ -45,6 +45,8 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
         dx = np.fromfile(os.path.join(td, "dx.bin"), "<f4").reshape(cfg.T, cfg.d)
         dW2_last = np.fromfile(os.path.join(td, "dW2_last.bin"), "<f4").reshape(cfg.d, cfg.H)
         dWg = np.fromfile(os.path.join(td, "dWg.bin"), "<f4").reshape(cfg.E, cfg.d)
+        dx_block = np.fromfile(os.path.join(td, "dx_block.bin"), "<f4").reshape(cfg.T, cfg.d)
+        dgamma = np.fromfile(os.path.join(td, "dgamma.bin"), "<f4")
     ref = O.moe_forward(inp["x"], inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es, bf16=dtype == "bf16")
     assert np.array_equal(ids, ref["ids"])
     assert N.rel_l2(out, ref["out"]) <= (1e-2 if dtype == "bf16" else 1e-5)
@@ -57,3 +59,6 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
     tol = 1e-2 if dtype == "bf16" else 1e-5
     assert N.rel_l2(dx, bw["dx"]) <= tol                                            # back(Tensor) of the C++ layer
     assert N.rel_l2(dW2_last, bw["dW2"][cfg.E - 1]) <= tol and N.rel_l2(dWg, bw["dWg"]) <= tol
+    bb = O.block_backward(inp["x"], gamma, dout, inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es,
+                          bf16=dtype == "bf16")
+    assert N.rel_l2(dx_block, bb["dx"]) <= tol and N.rel_l2(dgamma, bb["dgamma"]) <= tol     # backBlock of the C++ layer

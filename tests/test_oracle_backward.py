@@ -170,3 +170,56 @@ def test_backward_routed_equals_full_on_a_token_subset():
     assert np.array_equal(got["dx"], full["dx"][tok])
     assert np.array_equal(got["dw"], full["dw"][tok])
     assert np.array_equal(got["dlogits"], full["dlogits"][tok])
+
+
+def _gamma(d, seed):
+    return (O.fill_normal(d, seed, C.STREAM_NORM, 1.0) * np.float32(0.1) + np.float32(1.0)).astype(np.float32)
+
+
+@pytest.mark.parametrize("name,kw", CASES[:3])
+def test_block_backward_matches_float64_autograd(name, kw):
+    cfg, inp, dout = _case(name, 9, **kw)
+    gamma = _gamma(cfg.d, 9)
+    fwd = O.block_forward(inp["x"], gamma, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es)
+    got = O.block_backward(inp["x"], gamma, dout, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm,
+                           cfg.Es)
+    t64 = lambda a: torch.tensor(np.asarray(a, np.float64), requires_grad=True)
+    x, gm, Wg, W1, W3, W2 = (t64(v) for v in (inp["x"], gamma, inp["Wg"], inp["W1"], inp["W3"], inp["W2"]))
+    bg = t64(inp["bg"]) if inp["bg"] is not None else None
+    h = x / torch.sqrt((x * x).mean(dim=1, keepdim=True) + 1e-6) * gm
+    logits = h @ Wg.T + (bg if bg is not None else 0.0)
+    p = torch.softmax(logits, dim=1)
+    idt = torch.tensor(fwd["ids"].astype(np.int64))
+    q = torch.gather(p, 1, idt)
+    w = q / q.sum(dim=1, keepdim=True) if cfg.renorm else q
+    out = x
+    for g in range(cfg.E + cfg.Es):
+        y = (torch.nn.functional.silu(h @ W1[g].T) * (h @ W3[g].T)) @ W2[g].T
+        out = out + ((w * (idt == g)).sum(dim=1, keepdim=True) * y if g < cfg.E else y)
+    (out * torch.tensor(dout.astype(np.float64))).sum().backward()
+    ref = dict(dx=x.grad, dgamma=gm.grad, dWg=Wg.grad, dW1=W1.grad, dW3=W3.grad, dW2=W2.grad)
+    for k, v in ref.items():
+        assert N.rel_l2(got[k], v.numpy()) < 2e-5, (k, N.rel_l2(got[k], v.numpy()))
+    if bg is not None:
+        assert N.rel_l2(got["dbg"], bg.grad.numpy()) < 2e-5
+
+
+def test_rmsnorm_backward_closed_forms():
+    rng = np.random.default_rng(8)
+    T, d = 5, 96
+    x = rng.standard_normal((T, d)).astype(np.float32)
+    ones = np.ones(d, np.float32)
+    _, rms = O.rmsnorm(x, ones)
+    # dh orthogonal to x and gamma = 1: the rms term vanishes, dx = dh / rms
+    dh = rng.standard_normal((T, d)).astype(np.float64)
+    dh -= (dh * x).sum(1, keepdims=True) / (x.astype(np.float64) ** 2).sum(1, keepdims=True) * x
+    dx, dg = O.rmsnorm_backward(x, dh.astype(np.float32), ones, rms)
+    assert N.rel_l2(dx, dh / rms[:, None]) < 1e-5
+    # dh = x: dgamma = sum_t x^2 / rms; and dx = x/rms * (1 - mean(x^2)/rms^2) = x/rms * 1e-6/rms^2 (tiny)
+    dx, dg = O.rmsnorm_backward(x, x, ones, rms)
+    assert N.rel_l2(dg, (x.astype(np.float64) ** 2 / rms[:, None]).sum(0)) < 1e-6
+    assert np.abs(dx).max() < 1e-4
+    # the residual gradient is added as it is
+    r = rng.standard_normal((T, d)).astype(np.float32)
+    dx2, _ = O.rmsnorm_backward(x, x, ones, rms, resid=r)
+    assert N.rel_l2(dx2, dx.astype(np.float64) + r) < 1e-6
