@@ -1,5 +1,5 @@
-// Backward pass of the layer, fp32 layers: gradients of the input, the gate and every expert for an output gradient
-// dout [T,d], composed from the backward steps of the reference primitives the forward pass is built from:
+// Backward pass of the layer: gradients of the input, the gate and every expert for an output gradient dout [T,d],
+// composed from the backward steps of the reference primitives the forward pass is built from:
 //   linear layer   diffW = delta^T . input (overwritten), diff = delta . W, diffB = column sums of delta
 //                  (FullyLayer.diff, J/engine/nn/layer/FullyLayer.java:292-334)
 //   SwiGLU wiring  w2 back; dh3 = d(a) * silu(h1); dh1 = silu'(h1) applied to d(a) * h3; input gradient = w1's + w3's
@@ -11,7 +11,9 @@
 // with the activations a and the expert outputs y; h1 and h3 are recomputed.  Expert rows keep their forward places:
 // dy, dh1, dh3 and dxg are indexed by the same physical rows as xg, a and y.
 //
-// Kernels (all plain LDS-tiled FMA code, the fp32 configuration is the parity case):
+// bf16 layers run every product on the matrix-core kernel of the forward pass (launch_backward_bf16 at the end of this
+// file; the products themselves are described in experts_bf16.hip, their tables and the transposes in dispatch.hip).
+// fp32 layers (the parity configuration) use the plain LDS-tiled FMA kernels below:
 //   bw_combine_kernel   dy[r,:] = w[t,j] * dout[t,:],  dw[t,j] = dout[t,:] . y[r,:]
 //   bw_rows_f32_kernel  row-tiled grouped products over the forward tile list (h1/h3, d(a) + SwiGLU backward, dxg)
 //   bw_wgrad_f32_kernel dW_g = A_g^T . B_g over the rows of group g
@@ -137,20 +139,18 @@ __global__ __launch_bounds__(256) void bw_rows_f32_kernel(const float *__restric
 // dW_g[m, n] = sum over the rows r of group g of A[r, m] * B[r, n]  (diffW = delta^T . input); always written, so a group
 // without rows gets zeros.  grid (ceil(N/64), ceil(M/64), groups).  Rows of group g: physical rows from
 // tile_meta[1+g]*bm, counts[g] of them for a routed expert, T for a shared one; a shared group reads token rows
-// 0..T-1 of Atok / Btok when those are given.  single_rows >= 0: one group, rows 0..single_rows-1 of Aphys / Bphys.
+// 0..T-1 of Atok / Btok when those are given.
 // gstride: floats between the outputs of consecutive groups.
 __global__ __launch_bounds__(256) void bw_wgrad_f32_kernel(const float *__restrict__ Aphys, const float *__restrict__ Atok,
                                                            const float *__restrict__ Bphys, const float *__restrict__ Btok,
                                                            float *__restrict__ dW, size_t gstride,
                                                            const int32_t *__restrict__ tile_meta,
                                                            const int32_t *__restrict__ counts, int E, int T, int bm,
-                                                           int M, int N, int single_rows)
+                                                           int M, int N)
 {
     const int g = blockIdx.z;
-    int rows, row0;
-    if (single_rows >= 0) { rows = single_rows; row0 = 0; }
-    else { rows = g < E ? counts[g] : T; row0 = tile_meta[1 + g] * bm; }
-    const bool shared = single_rows < 0 && g >= E;
+    const int rows = g < E ? counts[g] : T, row0 = tile_meta[1 + g] * bm;
+    const bool shared = g >= E;
     const float *A = (shared && Atok) ? Atok : Aphys + (size_t)row0 * M;
     const float *B = (shared && Btok) ? Btok : Bphys + (size_t)row0 * N;
     const int m0 = blockIdx.y * GBM, n0 = blockIdx.x * GBN;
@@ -450,13 +450,13 @@ hipError_t launch_backward_f32(const omega_moe *m, const void *xv, const void *d
     const size_t HD = (size_t)c.H * c.d;
     hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.H, GBN), ceil_div(c.d, GBM), G), dim3(256), 0, s,
                        (const float *)m->bw_dy, dout, a, (const float *)nullptr, m->dW2, HD, m->tile_meta, m->counts, c.E, T,
-                       m->bm, c.d, c.H, -1);
+                       m->bm, c.d, c.H);
     hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
                        (const float *)m->bw_h1, (const float *)nullptr, xg, x, m->dW13, 2 * HD, m->tile_meta, m->counts, c.E,
-                       T, m->bm, c.H, c.d, -1);
+                       T, m->bm, c.H, c.d);
     hipLaunchKernelGGL(bw_wgrad_f32_kernel, dim3(ceil_div(c.d, GBN), ceil_div(c.H, GBM), G), dim3(256), 0, s,
                        (const float *)m->bw_h3, (const float *)nullptr, xg, x, m->dW13 + HD, 2 * HD, m->tile_meta, m->counts,
-                       c.E, T, m->bm, c.H, c.d, -1);
+                       c.E, T, m->bm, c.H, c.d);
     // router and gate
     hipLaunchKernelGGL(bw_router_kernel, dim3(ceil_div(T, 256)), dim3(256), 0, s, (const float *)m->bw_probs, m->ids, m->w,
                        (const float *)m->bw_dw, T, c.E, c.K, c.renorm, m->bw_dlogits);

@@ -550,7 +550,7 @@ hipError_t launch_backward_tables(const omega_moe *m, int T, hipStream_t s)
 // ---- transposed packed images ----
 // dst[c][32*k0 + (r - r0)] = src[r][c] for the rows r0 .. r0+nr-1 of a source image (KTs k steps wide, all its
 // 32*KTs columns), zero for the next rows up to the end of the range's 32*ksteps places.  One workgroup moves
-// 64 rows x 64 columns through LDS.  by_group != 0: the row ranges are the experts' (grid.y covers k space, the
+// 64 rows x 64 columns through LDS (grid.x: rows / k space, grid.y: columns).  by_group != 0: the row ranges are the experts' (the
 // workgroup looks its group up in kt0; r0 = first physical row of the group, or row 0 of src_alt for a shared expert
 // when src_alt is given); by_group == 0: one range (r0 = 0, nr rows, k0) per z, images src + z*src_stride ->
 // dst + z*dst_stride.
@@ -564,11 +564,11 @@ __global__ __launch_bounds__(256) void transpose_packed_kernel(const unsigned ch
 {
     __shared__ uint16_t tile[64][64 + 8];
     const int tid = threadIdx.x;
-    const int c0 = blockIdx.x * 64;  // source columns = destination rows
+    const int c0 = blockIdx.y * 64;  // source columns = destination rows
     int r0, nr, kd0, rb;             // rb: first row of this workgroup within the range
     const unsigned char *sp = src;
     if (by_group) {
-        const int kb = blockIdx.y * 2;  // first k step of this workgroup
+        const int kb = blockIdx.x * 2;  // first k step of this workgroup
         if (kb >= kt0[G]) return;
         int lo = 0, hi = G;             // last group with kt0[g] <= kb (empty groups share their successor's kt0)
         while (hi - lo > 1) {
@@ -587,9 +587,9 @@ __global__ __launch_bounds__(256) void transpose_packed_kernel(const unsigned ch
         dst += blockIdx.z * dst_stride;
         r0 = 0;
         nr = nr_single;
-        rb = blockIdx.y * 64;
+        rb = blockIdx.x * 64;
         if (rb >= nr) return;
-        kd0 = k0_single + blockIdx.y * 2;
+        kd0 = k0_single + blockIdx.x * 2;
     }
     // load: 64 rows x 8 chunks of 8 columns
 #pragma unroll
@@ -626,7 +626,7 @@ hipError_t launch_transpose_groups(const omega_moe *m, const void *src, const vo
                                    hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
-    hipLaunchKernelGGL(transpose_packed_kernel, dim3(cols / 64, m->bw_ksteps_cap / 2), dim3(256), 0, s,
+    hipLaunchKernelGGL(transpose_packed_kernel, dim3(m->bw_ksteps_cap / 2, cols / 64), dim3(256), 0, s,
                        (const unsigned char *)src, (const unsigned char *)src_alt, cols / 32, (unsigned char *)dst,
                        m->bw_ksteps_cap, 1, m->bw_kt0, m->tile_meta, m->counts, c.E, c.E + c.Es, T, m->bm, 0, 0, (size_t)0,
                        (size_t)0);
@@ -637,7 +637,7 @@ hipError_t launch_transpose_groups(const omega_moe *m, const void *src, const vo
 hipError_t launch_transpose_images(const void *src, int R, int cols, void *dst, int KTd, int k0, int n, size_t src_stride,
                                    size_t dst_stride, hipStream_t s)
 {
-    hipLaunchKernelGGL(transpose_packed_kernel, dim3(cols / 64, R / 64, n), dim3(256), 0, s, (const unsigned char *)src,
+    hipLaunchKernelGGL(transpose_packed_kernel, dim3(R / 64, cols / 64, n), dim3(256), 0, s, (const unsigned char *)src,
                        (const unsigned char *)nullptr, cols / 32, (unsigned char *)dst, KTd, 0, (const int32_t *)nullptr,
                        (const int32_t *)nullptr, (const int32_t *)nullptr, 0, 0, 0, 0, R, k0, src_stride, dst_stride);
     return hipGetLastError();
