@@ -163,7 +163,10 @@ int omega_moe_get_grad(omega_moe *moe, int which, int expert, void *dst, int is_
 int omega_moe_acc_grad(omega_moe *moe, float scale);
 /* update() of a layer without an updater: the accumulated gradients, if any, replace the gradients, then
  * w -= lr * diffW, b -= lr * diffB, and the accumulators are cleared (FullyLayer.update,
- * J/engine/nn/layer/FullyLayer.java:569-590).  The optimisers behind Updater are not part of this library. */
+ * J/engine/nn/layer/FullyLayer.java:569-590).  The optimisers behind Updater are not part of this library.
+ * bf16 layers take the step on fp32 master copies of their weights (made from the weights at the first update after
+ * they were set, kept across updates) and re-round the weights from them.  The forward pass must run again before the
+ * next backward pass. */
 int omega_moe_update(omega_moe *moe, float lr);
 
 /* The four stages of forward, callable one at a time (per-stage timing and tests); they use the

@@ -416,6 +416,7 @@ int omega_moe_destroy(omega_moe *m)
         if (p) hipFree(p);
     if (m->dWg) hipFree(m->dWg);
     if (m->acc_grad) hipFree(m->acc_grad);
+    if (m->master) hipFree(m->master);
     if (m->W2T) hipFree(m->W2T);
     if (m->W13T) hipFree(m->W13T);
     hipEventDestroy(m->ev0);
@@ -459,6 +460,7 @@ int omega_moe_set_weights(omega_moe *m, int which, int expert, const void *src, 
     void *p; size_t bytes;
     if (!src || weight_slot(m, which, expert, &p, &bytes) != OMEGA_OK)
         OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "set_weights: bad kind, expert index or source");
+    m->master_valid = false;  // fp32 master copies of a bf16 layer are remade from the weights at the next update
     if (!weight_is_packed(m, which)) {
         OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(p, src, bytes, is_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream));
         OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
@@ -742,12 +744,26 @@ int omega_moe_acc_grad(omega_moe *m, float scale)
 int omega_moe_update(omega_moe *m, float lr)
 {
     MOE_ENTER(m);
-    if (m->cfg.dtype != OMEGA_DTYPE_F32) OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "update: fp32 layers only");
     if (!m->dWg) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "update: no backward has run");
     const omega_moe_config &c = m->cfg;
     if (m->acc_valid) {
         OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(m->dWg, m->acc_grad, grad_block_floats(m) * 4, hipMemcpyDeviceToDevice, ctx->stream));
         m->acc_valid = false;
+    }
+    if (c.dtype == OMEGA_DTYPE_BF16) {
+        // the step is taken on fp32 master copies (made from the weights at the first update after they were set); the
+        // layer's bf16 weights are the masters re-rounded, and the transposed copies of the backward pass follow
+        if (!m->master) OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->master, grad_block_floats(m) * 4));
+        if (!m->master_valid) {
+            OMEGA_HIP_CHECK(ctx, launch_update_bf16(m, m->master, 0.0f, 1, ctx->stream));
+            m->master_valid = true;
+        }
+        OMEGA_HIP_CHECK(ctx, launch_update_bf16(m, m->master, lr, 0, ctx->stream));
+        if (c.has_gate_bias) OMEGA_HIP_CHECK(ctx, launch_axpy_f32(m->bg, m->dbg, -lr, (size_t)c.E, ctx->stream));
+        if (m->gamma_set) OMEGA_HIP_CHECK(ctx, launch_axpy_f32(m->gamma, m->dgamma, -lr, (size_t)c.d, ctx->stream));
+        m->wT_valid = false;
+        stage_invalidates(m);
+        return OMEGA_OK;
     }
     const size_t per = (size_t)c.H * c.d;
     OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->Wg, m->dWg, -lr, (size_t)c.E * c.d, ctx->stream));
@@ -758,6 +774,7 @@ int omega_moe_update(omega_moe *m, float lr)
         OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W3 + per * g, m->dW13 + per * (2 * g + 1), -lr, per, ctx->stream));
     }
     OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W2, m->dW2, -lr, per * m->G, ctx->stream));
+    stage_invalidates(m);  // the weights changed: a backward pass needs a new forward
     return OMEGA_OK;
 }
 

@@ -422,6 +422,79 @@ hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, 
     return hipGetLastError();
 }
 
+// ---- update of bf16 layers: fp32 master copies of the weights, the layer's bf16 copies re-rounded from them ----
+// One thread per 16-byte chunk (8 consecutive columns of one row) of the packed tile image of expert blockIdx.y.
+// init != 0: master = weight (first update after the weights were set); else master -= lr * grad, weight = bf16(master).
+__global__ __launch_bounds__(256) void bw_update_packed_kernel(float *__restrict__ master, size_t mstride,
+                                                               const float *__restrict__ grad, size_t gstride,
+                                                               unsigned char *__restrict__ packed, size_t pstride, int R, int K,
+                                                               float lr, int init)
+{
+    const int g = blockIdx.y, nch = K >> 3, KT = K >> 5;
+    float *mg = master + (size_t)g * mstride;
+    const float *gg = grad + (size_t)g * gstride;
+    unsigned char *pg = packed + (size_t)g * pstride;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)R * nch; i += (size_t)gridDim.x * 256) {
+        const int r = (int)(i / nch), ch = (int)(i % nch);
+        uint4 *pk = (uint4 *)(pg + pk_chunk_off(r, ch >> 2, ch & 3, KT));
+        float4 *mp = (float4 *)(mg + (size_t)r * K + ch * 8);
+        if (init) {
+            const uint4 u = *pk;
+            mp[0] = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                                __uint_as_float(u.y & 0xffff0000u));
+            mp[1] = make_float4(__uint_as_float(u.z << 16), __uint_as_float(u.z & 0xffff0000u), __uint_as_float(u.w << 16),
+                                __uint_as_float(u.w & 0xffff0000u));
+        } else {
+            const float4 *gp = (const float4 *)(gg + (size_t)r * K + ch * 8);
+            float4 a = mp[0], b = mp[1];
+            const float4 ga = gp[0], gb = gp[1];
+            a.x = fmaf(-lr, ga.x, a.x); a.y = fmaf(-lr, ga.y, a.y); a.z = fmaf(-lr, ga.z, a.z); a.w = fmaf(-lr, ga.w, a.w);
+            b.x = fmaf(-lr, gb.x, b.x); b.y = fmaf(-lr, gb.y, b.y); b.z = fmaf(-lr, gb.z, b.z); b.w = fmaf(-lr, gb.w, b.w);
+            mp[0] = a;
+            mp[1] = b;
+            uint4 o;
+            o.x = (uint32_t)f32_to_bf16(a.x) | ((uint32_t)f32_to_bf16(a.y) << 16);
+            o.y = (uint32_t)f32_to_bf16(a.z) | ((uint32_t)f32_to_bf16(a.w) << 16);
+            o.z = (uint32_t)f32_to_bf16(b.x) | ((uint32_t)f32_to_bf16(b.y) << 16);
+            o.w = (uint32_t)f32_to_bf16(b.z) | ((uint32_t)f32_to_bf16(b.w) << 16);
+            *pk = o;
+        }
+    }
+}
+
+// the gate weight: row-major bf16
+__global__ __launch_bounds__(256) void bw_update_rows_bf16_kernel(float *__restrict__ master, const float *__restrict__ grad,
+                                                                  bf16_t *__restrict__ w, size_t n, float lr, int init)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        if (init) master[i] = bf16_to_f32(w[i]);
+        else {
+            const float v = fmaf(-lr, grad[i], master[i]);
+            master[i] = v;
+            w[i] = f32_to_bf16(v);
+        }
+    }
+}
+
+// masters laid out like the gradient block: mWg at `master`, mW13 and mW2 at the offsets of dW13 and dW2
+hipError_t launch_update_bf16(const omega_moe *m, float *master, float lr, int init, hipStream_t s)
+{
+    const omega_moe_config &c = m->cfg;
+    const size_t HD = (size_t)c.H * c.d;
+    float *mW13 = master + (m->dW13 - m->dWg), *mW2 = master + (m->dW2 - m->dWg);
+    const size_t nWg = (size_t)c.E * c.d;
+    hipLaunchKernelGGL(bw_update_rows_bf16_kernel, dim3((unsigned)((nWg + 255) / 256 < 1024 ? (nWg + 255) / 256 : 1024)), dim3(256), 0,
+                       s, master, (const float *)m->dWg, (bf16_t *)m->Wg, nWg, lr, init);
+    const dim3 grid(512, m->G);
+    hipLaunchKernelGGL(bw_update_packed_kernel, grid, dim3(256), 0, s, mW13, 2 * HD, (const float *)m->dW13, 2 * HD,
+                       (unsigned char *)m->W1, HD * 2, c.H, c.d, lr, init);
+    hipLaunchKernelGGL(bw_update_packed_kernel, grid, dim3(256), 0, s, mW13 + HD, 2 * HD, (const float *)m->dW13 + HD, 2 * HD,
+                       (unsigned char *)m->W3, HD * 2, c.H, c.d, lr, init);
+    hipLaunchKernelGGL(bw_update_packed_kernel, grid, dim3(256), 0, s, mW2, HD, (const float *)m->dW2, HD,
+                       (unsigned char *)m->W2, HD * 2, c.d, c.H, lr, init);
+    return hipGetLastError();
+}
+
 hipError_t launch_backward_f32(const omega_moe *m, const void *xv, const void *doutv, int T, void *dxv, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;

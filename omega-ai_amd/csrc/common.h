@@ -94,6 +94,8 @@ struct omega_moe {
     float *dWg = nullptr, *dbg = nullptr, *dgamma = nullptr, *dW13 = nullptr, *dW2 = nullptr;
     float *acc_grad = nullptr;       // accumulators, one block in the order dWg, dbg, dgamma, dW13, dW2
     bool acc_valid = false;          // accGrad has run since the last update
+    float *master = nullptr;         // bf16 layers: fp32 master copies of Wg, W1|W3, W2 (layout of the gradient block)
+    bool master_valid = false;       // ... and whether they match the weights (set_weights invalidates)
     float *bw_probs = nullptr;       // [T,E] softmax of the gate logits
     float *bw_dw = nullptr;          // [T,K] gradient of the combine weights
     float *bw_dlogits = nullptr;     // [T,E]
@@ -171,6 +173,7 @@ hipError_t launch_transpose_images(const void *src, int R, int cols, void *dst, 
 enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4, MODE_UPREC = 5 };
 hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, const void *Aalt, const void *Wa, const void *Wb,
                                void *Cout, void *Aux1, void *Aux2, const omega_tile_desc *wq, int N, int Kd, hipStream_t s);
+hipError_t launch_update_bf16(const omega_moe *m, float *master, float lr, int init, hipStream_t s);
 hipError_t launch_zero_f32(float *dst, size_t n, hipStream_t s);
 hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, hipStream_t s);
 hipError_t launch_mfma_probe(float *scratch, int num_cus, int random_operands, int launches, hipStream_t s,

@@ -270,7 +270,8 @@ class MoELayer:
 
     def update(self, learnRate):
         """The update of a layer without an updater: w -= learnRate * diffW (FullyLayer.update,
-        J/engine/nn/layer/FullyLayer.java:569-590)."""
+        J/engine/nn/layer/FullyLayer.java:569-590); bf16 layers step fp32 master copies and re-round.  forward() must run
+        again before the next back()."""
         self.ctx.check(self.lib.omega_moe_update(self.handle, float(learnRate)))
 
     # ---- stages and introspection

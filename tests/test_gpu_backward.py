@@ -233,8 +233,7 @@ def test_backward_call_order_and_growth():
     layer.stage("router", x)
     with pytest.raises(RuntimeError):          # a stage run on its own invalidates the forward
         layer.back(g)
-    with pytest.raises(RuntimeError):          # update on a bf16 layer: no fp32 master weights
-        layer.forward(x); layer.back(g); layer.update(0.1)
+    layer.forward(x)
     dx_small = layer.back(g).to_numpy()
     # a batch four times as large (new workspace), training mode on, then the small one again
     cfg2 = scaled(cfg, T=256)
@@ -251,4 +250,60 @@ def test_backward_call_order_and_growth():
     assert N.rel_l2(layer.grad(L.W_W2, 1), ref2["dW2"][1]) < 1e-2
     layer.forward(x)
     assert np.array_equal(layer.back(g).to_numpy(), dx_small)
+    layer.close()
+
+
+def test_update_bf16_keeps_fp32_masters():
+    """Two plain updates of a bf16 layer: the weights are the re-rounded fp32 masters w0 - lr*g1 - lr*g2, not a chain of
+    bf16 roundings; a backward pass straight after an update raises (the forward pass must run again); new weights
+    restart the masters."""
+    G, cfg, inp, dout, layer = _setup("c2_mixtral", dict(T=96, d=256, H=256, E=4, K=2), 13)
+    P = G.P
+    x = P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    lr = 0.37
+    shapes = {"W1": (L.W_W1, (cfg.H, cfg.d)), "W3": (L.W_W3, (cfg.H, cfg.d)), "W2": (L.W_W2, (cfg.d, cfg.H))}
+    w0 = {k: layer._download_weight(w, 2, s) for k, (w, s) in shapes.items()}
+    w0["Wg"] = layer._download_weight(L.W_GATE, 0, (cfg.E, cfg.d))
+    grads = []
+    for step in range(2):
+        layer.forward(x)
+        layer.back(g)
+        gr = {k: layer.grad(w, 2) for k, (w, s) in shapes.items()}
+        gr["Wg"] = layer.grad(L.W_GATE)
+        grads.append(gr)
+        layer.update(lr)
+        with pytest.raises(RuntimeError):
+            layer.back(g)
+    for k in ("W1", "W3", "W2", "Wg"):
+        got = layer._download_weight(*((shapes[k][0], 2, shapes[k][1]) if k != "Wg" else (L.W_GATE, 0, (cfg.E, cfg.d))))
+        m = w0[k].copy()
+        for gr in grads:
+            m = (np.float32(-lr) * gr[k] + m).astype(np.float32)     # one rounding per step: fused multiply-add
+        want = O.round_bf16(m)
+        chain = O.round_bf16(O.round_bf16(w0[k] - np.float32(lr) * grads[0][k]) - np.float32(lr) * grads[1][k])
+        # fused vs unfused multiply-add may move a value by one bf16 step when it sits on a rounding boundary
+        close = np.abs(got - want) <= np.abs(want) * 2.0 ** -7
+        assert close.all() and (got == want).mean() > 0.999, (k, (got == want).mean())
+        assert (got == want).mean() > (got == chain).mean()          # masters, not re-rounded bf16 weights
+    # the next forward / backward uses the updated weights (transposed copies rebuilt)
+    for e in range(cfg.E):
+        for k, (w, s) in shapes.items():
+            inp[k][e] = layer._download_weight(w, e, s)
+    inp["Wg"] = layer._download_weight(L.W_GATE, 0, (cfg.E, cfg.d))
+    layer.forward(x)
+    dx = layer.back(g).to_numpy()
+    ref = O.moe_backward(inp["x"], dout, inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K, cfg.renorm, cfg.Es,
+                         bf16=True)
+    assert N.rel_l2(dx, ref["dx"]) < 1e-2
+    assert N.rel_l2(layer.grad(L.W_W1, 0), ref["dW1"][0]) < 1e-2
+    # setting a weight restarts the masters from the weights
+    layer.set_expert(2, inp["W1"][2], inp["W3"][2], w0["W2"])
+    layer.forward(x)
+    layer.back(g)
+    g2 = layer.grad(L.W_W2, 2)
+    layer.update(lr)
+    got = layer._download_weight(L.W_W2, 2, (cfg.d, cfg.H))
+    want = O.round_bf16((np.float32(-lr) * g2 + w0["W2"]).astype(np.float32))
+    assert (got == want).mean() > 0.999
     layer.close()
