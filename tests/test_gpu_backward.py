@@ -307,3 +307,27 @@ def test_update_bf16_keeps_fp32_masters():
     want = O.round_bf16((np.float32(-lr) * g2 + w0["W2"]).astype(np.float32))
     assert (got == want).mean() > 0.999
     layer.close()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_sgd_steps_reduce_a_regression_loss(dtype):
+    """forward -> back(out - target) -> update, a few times: the squared error to a fixed target goes down
+    (the layer trains with the plain update, fp32 and bf16 with master weights)."""
+    G, cfg, inp, _, layer = _setup("c2_mixtral", dict(T=128, d=256, H=256, E=4, K=2, dtype=dtype), 23)
+    P = G.P
+    bf = dtype == "bf16"
+    x = P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    target = O.fill_normal(cfg.T * cfg.d, 23, 901, 0.5).reshape(cfg.T, cfg.d)
+    losses = []
+    layer.set_training(True)
+    for step in range(8):
+        out = layer.forward(x).to_numpy()
+        diff = (out - target).astype(np.float32)
+        losses.append(float(0.5 * (diff.astype(np.float64) ** 2).sum()))
+        g = P.DeviceBuffer.from_numpy(G.ctx(), O.round_bf16(diff) if bf else diff, cfg.dtype)
+        layer.back(g)
+        layer.update(2e-3)
+        g.free()
+    assert all(b < a for a, b in zip(losses, losses[1:])), losses
+    assert losses[-1] < 0.8 * losses[0], losses
+    layer.close()
