@@ -6,6 +6,7 @@ cover its building blocks with expected outputs), so the fixtures freeze what th
   * the fp32 parity configuration (256 tokens, d=128, 8 experts, top-2, H=256) under a fixed seed, and
   * small adversarial cases: ties (all-equal gate rows, duplicated gate rows), empty experts, K == E,
     shared experts without renormalisation.
+The backward pass of four of the cases is frozen the same way (bw_*.npz, see BW_CASES).
 Inputs are regenerated from the seed by the counter-based generator, so only expected outputs are stored:
 routing arrays in full, the layer output as float64 checksums plus a few rows.
 Run from the repository root:  python tests/golden/make_fixtures.py
@@ -55,10 +56,41 @@ def expected(spec):
                 out_abs_sum=np.array(np.abs(out64).sum()), out_head=r["out"][:4].copy(), out_tail=r["out"][-2:].copy())
 
 
+# Backward pass (pinned oracle: float64 autograd, finite differences): the output gradient is drawn from the case's
+# seed (stream 900); stored are the gate gradients in full, per-expert norms of the expert gradients, and rows and
+# float64 checksums of the input gradient.  Files bw_<case>.npz.
+BW_CASES = ("c1_tiny_f32_seed20251", "shared_no_renorm", "zipf_empty_experts", "bf16_small")
+
+
+def backward_dout(spec):
+    cfg = spec["cfg"]
+    g = O.fill_normal(cfg.T * cfg.d, spec["seed"], 900, 1.0).reshape(cfg.T, cfg.d)
+    return O.round_bf16(g) if cfg.dtype == "bf16" else g
+
+
+def expected_backward(spec):
+    cfg = spec["cfg"]
+    inp = case_inputs(spec)
+    r = O.moe_backward(inp["x"], backward_dout(spec), inp["Wg"], inp["bg"], inp["W1"], inp["W3"], inp["W2"], cfg.K,
+                       cfg.renorm, cfg.Es, bf16=cfg.dtype == "bf16")
+    dx64 = r["dx"].astype(np.float64)
+    norms = np.array([[np.sqrt((r[k][g].astype(np.float64) ** 2).sum()) for g in range(cfg.E + cfg.Es)]
+                      for k in ("dW1", "dW3", "dW2")])
+    out = dict(dx_head=r["dx"][:4].copy(), dx_tail=r["dx"][-2:].copy(), dx_sum=np.array(dx64.sum()),
+               dx_l2=np.array(np.sqrt((dx64 ** 2).sum())), dx_abs_sum=np.array(np.abs(dx64).sum()), dWg=r["dWg"],
+               dW_norms=norms, dW2_first_row=r["dW2"][int(np.argmax(norms[2]))][0].copy())
+    if r["dbg"] is not None:
+        out["dbg"] = r["dbg"]
+    return out
+
+
 def main():
     for name, spec in CASES.items():
         np.savez_compressed(os.path.join(HERE, name + ".npz"), **expected(spec))
         print("wrote", name)
+    for name in BW_CASES:
+        np.savez_compressed(os.path.join(HERE, "bw_" + name + ".npz"), **expected_backward(CASES[name]))
+        print("wrote bw_" + name)
 
 
 if __name__ == "__main__":

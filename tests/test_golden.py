@@ -48,3 +48,42 @@ def test_hip_path_reproduces_fixture(name):
     assert abs(np.sqrt((o64 ** 2).sum()) - want["out_l2"]) <= tol * want["out_l2"]
     assert abs(o64.sum() - want["out_sum"]) <= tol * want["out_abs_sum"]
     layer.close()
+
+
+@pytest.mark.parametrize("name", sorted(MF.BW_CASES))
+def test_oracle_reproduces_backward_fixture(name):
+    want, got = load("bw_" + name), MF.expected_backward(MF.CASES[name])
+    assert sorted(want) == sorted(got)
+    for k in want:
+        assert np.array_equal(want[k], got[k]), (name, k)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(MF.BW_CASES))
+def test_hip_path_reproduces_backward_fixture(name):
+    import importlib
+    from tests import gpu_util as G
+    L = importlib.import_module("omega-ai_amd._lib")
+    case = MF.CASES[name]
+    cfg, want = case["cfg"], load("bw_" + name)
+    inp = MF.case_inputs(case)
+    layer = G.build_layer(cfg, inp)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = G.P.DeviceBuffer.from_numpy(G.ctx(), MF.backward_dout(case), cfg.dtype)
+    layer.forward(x)
+    dx = layer.back(g).to_numpy()
+    tol = 1e-2 if cfg.dtype == "bf16" else 1e-5
+    assert N.rel_l2(dx[:4], want["dx_head"]) <= tol and N.rel_l2(dx[-2:], want["dx_tail"]) <= tol
+    d64 = dx.astype(np.float64)
+    assert abs(np.sqrt((d64 ** 2).sum()) - want["dx_l2"]) <= tol * want["dx_l2"]
+    assert abs(d64.sum() - want["dx_sum"]) <= tol * want["dx_abs_sum"]
+    assert N.rel_l2(layer.grad(L.W_GATE), want["dWg"]) <= tol
+    if "dbg" in want:
+        assert N.rel_l2(layer.grad(L.W_GATE_BIAS), want["dbg"]) <= tol
+    for i, which in enumerate((L.W_W1, L.W_W3, L.W_W2)):
+        for e in range(cfg.E + cfg.Es):
+            n = np.sqrt((layer.grad(which, e).astype(np.float64) ** 2).sum())
+            assert abs(n - want["dW_norms"][i, e]) <= tol * max(want["dW_norms"][i, e], 1e-30), (i, e)
+    e = int(np.argmax(want["dW_norms"][2]))
+    assert N.rel_l2(layer.grad(L.W_W2, e)[0], want["dW2_first_row"]) <= tol
+    layer.close()
