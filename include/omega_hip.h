@@ -86,6 +86,21 @@ int omega_hip_memset(omega_ctx *ctx, void *dptr, int value, size_t bytes);
 /* JCuda.cudaDeviceSynchronize() as used around timed regions (J/engine/nn/network/Llama3.java:140-156). */
 int omega_hip_sync(omega_ctx *ctx);
 
+/* java.util.Random on the host (no device involved), for initialising a layer with the numbers a Java run of the
+ * reference draws: RandomUtils keeps one java.util.Random (RandomUtils.setSeed / getInstance,
+ * J/common/utils/RandomUtils.java:18-28); omega_jrandom_normal is RandomUtils.normal_ (RandomUtils.java:697-703):
+ * out[i] = (float)(std * nextGaussian() + mean).  The state is plain data owned by the caller. */
+typedef struct {
+    int64_t state;              /* 48-bit state of the linear congruential generator */
+    double next_gaussian;       /* the second value of the last polar-method pair ... */
+    int32_t have_next_gaussian; /* ... if it has not been handed out yet              */
+} omega_jrandom;
+void omega_jrandom_seed(omega_jrandom *r, int64_t seed);
+int32_t omega_jrandom_next_int(omega_jrandom *r);
+double omega_jrandom_next_double(omega_jrandom *r);
+double omega_jrandom_next_gaussian(omega_jrandom *r);
+void omega_jrandom_normal(omega_jrandom *r, float *out, size_t n, float mean, float std);
+
 /* Seeded synthetic data on the device: element i of `stream` under `seed`, N(0,std), written as
  * `dtype`.  Counter-based, so any slice (first, n) of a stream can be produced independently.
  * Stands in for RandomUtils.normal_ (J/common/utils/RandomUtils.java:697-703) + Tensor upload. */

@@ -48,6 +48,11 @@ SIGNATURES = {
     "omega_moe_time_backward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int,
                                           C.POINTER(C.c_float)]),
     "omega_moe_backward_block": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+    "omega_jrandom_seed": (None, [C.c_void_p, C.c_int64]),
+    "omega_jrandom_next_int": (C.c_int32, [C.c_void_p]),
+    "omega_jrandom_next_double": (C.c_double, [C.c_void_p]),
+    "omega_jrandom_next_gaussian": (C.c_double, [C.c_void_p]),
+    "omega_jrandom_normal": (None, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_float]),
     "omega_moe_set_training": (C.c_int, [C.c_void_p, C.c_int]),
     "omega_moe_get_grad": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
     "omega_moe_acc_grad": (C.c_int, [C.c_void_p, C.c_float]),

@@ -132,6 +132,26 @@ public:
         upload(OMEGA_W_W2, g, W2, n);
     }
 
+    // RandomUtils.setSeed(seed) + the house-style initialisation of LlamaMLPLayer.initLayers
+    // (J/engine/nn/layer/llama/LlamaMLPLayer.java:68-90): every weight normal_(n, 0.01f, 0.02f) from ONE java.util.Random
+    // (J/common/utils/RandomUtils.java:18-28,697-703); the gate first (the reference has none: drawn like the others),
+    // then per expert linear1 (W1), linear2 (W2), linear3 (W3) in the order the reference constructs them
+    void initJava(int64_t seed, float mean = 0.01f, float std = 0.02f)
+    {
+        omega_jrandom r;
+        omega_jrandom_seed(&r, seed);
+        const size_t n = (size_t)hidden_ * embedDim_;
+        std::vector<float> wg((size_t)nExperts_ * embedDim_), w1(n), w2(n), w3(n);
+        omega_jrandom_normal(&r, wg.data(), wg.size(), mean, std);
+        setGate(wg.data());
+        for (int g = 0; g < nExperts_ + nShared_; ++g) {
+            omega_jrandom_normal(&r, w1.data(), n, mean, std);
+            omega_jrandom_normal(&r, w2.data(), n, mean, std);
+            omega_jrandom_normal(&r, w3.data(), n, mean, std);
+            setExpert(g, w1.data(), w3.data(), w2.data());
+        }
+    }
+
     void init() override
     {
         number = input->number;

@@ -361,6 +361,12 @@ class MoELayer:
                 raise RuntimeError("Error code 1:checkpoint ends early")
             self._upload(which, g, np.frombuffer(buf, "<f4").reshape(shape))
 
+    def initJava(self, seed, mean=0.01, std=0.02):
+        """RandomUtils.setSeed(seed) followed by the house-style initialisation (java_random.init_layer): the weights a
+        Java run of the reference would draw.  Returns the arrays that were set."""
+        from . import java_random
+        return java_random.init_layer(self, java_random.JavaRandom(seed), mean, std)
+
     def loadJson(self, weight_map, layer_index=0, scheme="omega", strict=True):
         """Weights by name from a JSON export of a PyTorch state dict (see weights_json.py; the reference's
         LagJsonReader + ModeLoaderlUtils.loadData route)."""

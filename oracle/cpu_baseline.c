@@ -105,7 +105,9 @@ double orc_cpu_baseline_forward(const float *x, const float *Wg, const float *bg
 {
     int P = T * K, G = E + Es;
     size_t rows_total = (size_t)P + (size_t)Es * T;
-    float *logits = (float *)malloc(sizeof(float) * (size_t)T * E);
+    /* the product outputs are zero-initialised, as Java's new float[n] is: the beta == 0 update C *= beta of the
+     * restated sgemm would turn stale NaN patterns of a recycled heap block into NaN results */
+    float *logits = (float *)calloc((size_t)T * E, sizeof(float));
     float *p = (float *)malloc(sizeof(float) * (size_t)T * E);
     int32_t *ids = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
     float *w = (float *)malloc(sizeof(float) * (size_t)P);
@@ -114,9 +116,9 @@ double orc_cpu_baseline_forward(const float *x, const float *Wg, const float *bg
     int32_t *dst = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
     int32_t *src_row = (int32_t *)malloc(sizeof(int32_t) * (size_t)P);
     float *xg = (float *)malloc(sizeof(float) * (size_t)P * d);
-    float *h1 = (float *)malloc(sizeof(float) * rows_total * H);
-    float *h3 = (float *)malloc(sizeof(float) * rows_total * H);
-    float *y = (float *)malloc(sizeof(float) * rows_total * d);
+    float *h1 = (float *)calloc(rows_total * H, sizeof(float));
+    float *h3 = (float *)calloc(rows_total * H, sizeof(float));
+    float *y = (float *)calloc(rows_total * d, sizeof(float));
     gemm_task *tasks = (gemm_task *)malloc(sizeof(gemm_task) * (size_t)G);
 
     double t0 = now_s();
