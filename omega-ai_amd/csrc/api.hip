@@ -647,10 +647,10 @@ static int backward_impl(omega_moe *m, const void *x, const void *dout, int T, v
 {
     omega_ctx *ctx = m->ctx;
     RUN(check_T(m, x, T, true));
+    if (T == 0) return OMEGA_OK;  // an empty batch: nothing to do, as in forward
     if (T != m->fwd_T || block != m->fwd_block)
         OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, block ? "backward_block: no omega_moe_forward_block has run for this T"
                                                      : "backward: no omega_moe_forward has run for this T");
-    if (T == 0) return OMEGA_OK;
     if (!dout || !dx) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "backward: dout or dx is NULL");
     RUN(moe_reserve_backward(m, T));
     const bool bf = m->cfg.dtype == OMEGA_DTYPE_BF16;

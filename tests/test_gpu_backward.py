@@ -250,6 +250,11 @@ def test_backward_call_order_and_growth():
     assert N.rel_l2(layer.grad(L.W_W2, 1), ref2["dW2"][1]) < 1e-2
     layer.forward(x)
     assert np.array_equal(layer.back(g).to_numpy(), dx_small)
+    # an empty batch is a no-op for every pass (and leaves the saved forward alone)
+    assert layer.lib.omega_moe_forward(layer.handle, None, 0, None) == 0
+    assert layer.lib.omega_moe_backward(layer.handle, None, None, 0, None) == 0
+    assert layer.lib.omega_moe_backward_block(layer.handle, None, None, 0, None) == 0
+    assert np.array_equal(layer.back(g).to_numpy(), dx_small)
     layer.close()
 
 
