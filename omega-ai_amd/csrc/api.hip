@@ -311,10 +311,11 @@ static int moe_reserve(omega_moe *m, int T)
     OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->a, 0, m->rows_cap * c.H * m->esize, ctx->stream));
     if (c.dtype == OMEGA_DTYPE_BF16) {
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_up, ((size_t)m->tiles_cap * (c.H / 128) + OMEGA_TAIL_EXTRA) * sizeof(omega_tile_desc)));
-        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_down, ((size_t)m->tiles_cap * (c.d / 256) + OMEGA_TAIL_EXTRA) * sizeof(omega_tile_desc)));
         m->n_wg = std::min(256, ctx->num_cus / 8 * 8);
+        // (room for the half-width items of small batches: at most n_wg of them)
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->desc_down, (std::max((size_t)m->tiles_cap * (c.d / 256), (size_t)m->n_wg) + OMEGA_TAIL_EXTRA) * sizeof(omega_tile_desc)));
         const size_t q_up = ((size_t)m->tiles_cap * (c.H / 128) + OMEGA_TAIL_EXTRA) / m->n_wg + 2;
-        const size_t q_down = ((size_t)m->tiles_cap * (c.d / 256) + OMEGA_TAIL_EXTRA) / m->n_wg + 2;
+        const size_t q_down = (std::max((size_t)m->tiles_cap * (c.d / 256), (size_t)m->n_wg) + OMEGA_TAIL_EXTRA) / m->n_wg + 2;
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->wq_up, q_up * m->n_wg * sizeof(omega_tile_desc)));
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->wq_down, q_down * m->n_wg * sizeof(omega_tile_desc)));
         // an all-zero queue is an empty one: the product kernels return at once if no dispatch has run yet
@@ -537,6 +538,7 @@ static int stage_dispatch(omega_moe *m, const void *x, int T)
     const int bm = moe_tile_m(m, T);
     m->bm = bm;
     m->max_m_tiles = moe_max_m_tiles(m, T, bm);
+    if (m->cfg.dtype == OMEGA_DTYPE_BF16) m->down_cols = m->max_m_tiles * (m->cfg.d / 256) <= m->n_wg / 2 ? 128 : 256;
     if (m->max_m_tiles > m->tiles_cap) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: workspace too small for this T");
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));

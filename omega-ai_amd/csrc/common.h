@@ -40,8 +40,9 @@ struct __attribute__((aligned(16))) omega_tile {
 struct __attribute__((aligned(32))) omega_tile_desc {
     int32_t g, row0, rows, xrow0;  // as omega_tile
     int32_t n0;                    // first output column of the tile
-    // weight-gradient items only (zero otherwise): row groups (128 rows) of the two operand tiles in their transposed
-    // images and the first k step of the expert's rows there; xrow0 then holds the item's number of k steps
+    // weight-gradient items: row groups (128 rows) of the two operand tiles in their transposed images and the first
+    // k step of the expert's rows there; xrow0 then holds the item's number of k steps.  Other items: zero, except
+    // b_rg = 1 in an item of the down product that covers 128 columns instead of 256
     int32_t a_rg, b_rg, kt0;
 };
 
@@ -81,6 +82,9 @@ struct omega_moe {
     // at [q * n_wg + w]; a queue ends with an entry of 0 rows
     omega_tile_desc *wq_up = nullptr, *wq_down = nullptr;
     int n_wg = 0;                          // workgroups of a product launch: one per compute unit, a multiple of 8
+    // columns of a work item of the down product: 256, or 128 when 256-column tiles would leave at least half of the
+    // compute units without an item (a few tokens: the product is bound by streaming W2, which every unit must share)
+    int down_cols = 256;
     void *xg = nullptr;              // [rows_cap,d]  gathered tokens (bf16: packed tile image, see pack.h)
     void *xs = nullptr;              // bf16 with shared experts: packed copy of x, [ceil(T/bm)*bm,d]
     void *a = nullptr;               // [rows_cap,H]  (bf16: packed tile image)

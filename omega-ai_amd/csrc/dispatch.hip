@@ -69,7 +69,8 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
         omega_tile_desc dsc;
         dsc.g = g;
         dsc.n0 = n * ncols;
-        dsc.a_rg = dsc.b_rg = dsc.kt0 = 0;
+        dsc.a_rg = dsc.kt0 = 0;
+        dsc.b_rg = ncols == 128 ? 1 : 0;  // read by the plain 256-column products only: a half-width item
         if (at < Nt - r) {
             dsc.row0 = mt0 * bm + tfirst;
             dsc.rows = trows;
@@ -403,7 +404,7 @@ hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t 
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(dispatch_rank_kernel, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_base, m->counts, T, c.K,
                        c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles, m->tile_meta, m->desc_up, c.H / 128, 128,
-                       m->desc_down, c.d / 256, 256);
+                       m->desc_down, c.d / m->down_cols, m->down_cols);
     return hipGetLastError();
 }
 

@@ -90,6 +90,7 @@ struct TileCtx {
     uint32_t a_off0, a_off1;  // this lane's byte offsets of its two A blocks within a k step
     int row0, rows, n0;
     int kt;                   // k steps of the item
+    int half;                 // plain 256-column products: the item covers the first 128 columns only
 };
 
 __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char *p)
@@ -113,6 +114,7 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
     if (MODE == MODE_WGRAD) {
         const size_t k0 = (size_t)d.kt0 * 8192;
         c.kt = d.xrow0;
+        c.half = 0;
         c.A = uniform_ptr((const unsigned char *)Axg + (size_t)d.a_rg * rg_bytes + k0);
         c.B0 = uniform_ptr((const unsigned char *)Wa + (size_t)d.b_rg * rg_bytes + k0);
         c.B1 = uniform_ptr(c.B0 + rg_bytes);
@@ -121,12 +123,15 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
         return c;
     }
     c.kt = KT;
+    c.half = FUSED ? 0 : d.b_rg;
     c.A = uniform_ptr((MODE != MODE_DOWN && Ax != nullptr && d.xrow0 >= 0)
                           ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
                           : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes);
     const size_t wrg = (size_t)d.g * (N >> 7) + (d.n0 >> 7);  // row group of the weight tile
     c.B0 = uniform_ptr((const unsigned char *)Wa + wrg * rg_bytes);
-    c.B1 = uniform_ptr(FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : c.B0 + rg_bytes);
+    // (a half-width item loads its 128 weight rows twice - the second copy comes out of the L2 - and drops the results
+    //  of the duplicate: the products it is used for are bound by streaming the weights from memory, not by the MFMAs)
+    c.B1 = uniform_ptr(FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : c.half ? c.B0 : c.B0 + rg_bytes);
     // Wave-load q (0..15) of an operand tile is the packed block q % 8 of row group q / 8; this wave issues q = wave
     // and q = wave + 8 of both operands.  A points at the row group of the whole row tile; a slice starts blk0
     // 16-row blocks into it.  A blocks that hold no valid row (ragged tile) are never used by an MFMA whose result
@@ -173,6 +178,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     ctx.row0 = __builtin_amdgcn_readfirstlane(ctx_in.row0);
     ctx.rows = __builtin_amdgcn_readfirstlane(ctx_in.rows);
     ctx.n0 = __builtin_amdgcn_readfirstlane(ctx_in.n0);
+    ctx.half = __builtin_amdgcn_readfirstlane(ctx_in.half);
     int cur = __builtin_amdgcn_readfirstlane(cur_io);
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -361,7 +367,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
                 }
             }
         }
-    } else if (MODE == MODE_DOWN || MODE == MODE_WGRAD) {
+    } else if ((MODE == MODE_DOWN || MODE == MODE_WGRAD) && !(ctx.half && wn >= 2)) {
         // lane: column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
