@@ -75,7 +75,8 @@ struct omega_moe {
     int32_t *src_row = nullptr;      // [T*K]
     omega_tile *tiles = nullptr;     // [max_m_tiles]
     int32_t *tile_meta = nullptr;    // [0] = number of row tiles; [1+g] = first row tile of group g (G+1 entries);
-                                     // [G+2], [G+3] = entries of desc_up, desc_down
+                                     // [G+2], [G+3] = entries of desc_up, desc_down; [G+4..G+6] = entries of the
+                                     // backward tables desc_da, desc_w2, desc_w13
     omega_tile_desc *desc_up = nullptr;    // bf16: [tiles_cap * H/128] output tiles of the up product
     omega_tile_desc *desc_down = nullptr;  // bf16: [tiles_cap * d/256] output tiles of the down product
     // bf16: the same work items as one queue per workgroup of the (persistent) product kernels, entry q of workgroup w
