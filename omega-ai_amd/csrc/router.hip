@@ -13,6 +13,7 @@
 //           top-k: K rounds of a cross-lane (value,index) butterfly arg-max, "greater value, or equal
 //           value and lower index" so ties go to the lowest expert; winners are masked out.
 //  phase 3  LDS-atomic histogram of the selected experts, flushed as row `tile` of tile_counts[.,E].
+// FAST mode of bf16 layers with more than 16 experts takes phase 1 to the matrix cores (router_mfma_kernel below).
 #include "common.h"
 
 #define TOK_TILE ROUTER_TOK_TILE
@@ -156,56 +157,18 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
     }
 }
 
-template <int EP, int KC, bool EXACT>
-__global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
-                                                     const float *__restrict__ bg, int T, int d, int E, int K,
-                                                     int renorm, int32_t *__restrict__ ids,
-                                                     float *__restrict__ wout, int32_t *__restrict__ tile_counts,
-                                                     float *__restrict__ logits_out, float *__restrict__ probs_out)
+// Phases 2 and 3 for the 32 tokens of one workgroup, from the logits in lg (all 256 threads; lg and hist are complete
+// and visible on entry).  RELAXED (the matrix-core FAST path only, tolerance mode): exponentials in single precision
+// and the softmax sum as a butterfly over the lanes instead of the reference's order - the ordered sum is a chain of
+// EP dependent cross-lane reads per token and dominates that path otherwise.
+template <int EP, bool RELAXED = false>
+__device__ __forceinline__ void router_select(float (*lg)[EP], int *hist, int t0, int tile, int T, int E, int K, int renorm,
+                                              int32_t *__restrict__ ids, float *__restrict__ wout,
+                                              int32_t *__restrict__ tile_counts, float *__restrict__ probs_out)
 {
-    constexpr int EPT = ROUTER_EPT(EP), EL = EP / EPT;  // phase 1: experts per thread, threads across the experts
-    constexpr int NT = TOK_TILE * EL / 256;             // tokens per thread in phase 1
-    constexpr int TPP = 256 / EL;                       // tokens per pass
-    constexpr int GS = EP < 64 ? EP : 64;    // lanes that share one token in phase 2
-    constexpr int VPL = EP / GS;             // experts per lane in phase 2
-    constexpr int LDW = KC + 4;  // LDS row stride in floats: rows stay 16-byte aligned and bank-staggered
-    __shared__ __attribute__((aligned(16))) float xs[TOK_TILE][LDW];
-    __shared__ __attribute__((aligned(16))) float ws[EP][LDW];
-    __shared__ float lg[TOK_TILE][EP];
-    __shared__ int hist[EP];
-
+    constexpr int GS = EP < 64 ? EP : 64;    // lanes that share one token
+    constexpr int VPL = EP / GS;             // experts per lane
     const int tid = threadIdx.x;
-    const int tile = blockIdx.x;
-    const int t0 = tile * TOK_TILE;
-    const int e1 = tid % EL, tg = tid / EL;
-    if (tid < EP) hist[tid] = 0;
-
-    float acc[NT * EPT];
-#pragma unroll
-    for (int i = 0; i < NT * EPT; ++i) acc[i] = 0.0f;
-
-    const bool fast_io = (d % KC == 0) && (((uintptr_t)x | (uintptr_t)Wg) % 16 == 0);
-    if (dtype == OMEGA_DTYPE_BF16) {
-        if (fast_io) router_sums<EP, KC, EXACT, true, true>(x, Wg, T, d, E, t0, xs, ws, acc);
-        else router_sums<EP, KC, EXACT, true, false>(x, Wg, T, d, E, t0, xs, ws, acc);
-    } else {
-        if (fast_io) router_sums<EP, KC, EXACT, false, true>(x, Wg, T, d, E, t0, xs, ws, acc);
-        else router_sums<EP, KC, EXACT, false, false>(x, Wg, T, d, E, t0, xs, ws, acc);
-    }
-#pragma unroll
-    for (int x_ = 0; x_ < EPT; ++x_) {
-        const int e = e1 + x_ * EL;
-        const float b = (bg != nullptr && e < E) ? bg[e] : 0.0f;
-#pragma unroll
-        for (int i = 0; i < NT; ++i) {
-            const float z = bg != nullptr ? acc[x_ * NT + i] + b : acc[x_ * NT + i];
-            lg[tg + i * TPP][e] = z;
-            const int t = t0 + tg + i * TPP;
-            if (logits_out != nullptr && t < T && e < E) logits_out[(size_t)t * E + e] = z;
-        }
-    }
-    __syncthreads();
-
     // ---- phase 2: each wave owns 8 tokens; GS lanes share a token ----
     const int lane = tid & 63, wave = tid >> 6;
     const int sub = lane % GS, grp = lane / GS;
@@ -228,15 +191,22 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
 #pragma unroll
         for (int q = 0; q < VPL; ++q) {
             const int e = sub + q * GS;
-            p[q] = e < E ? (float)exp((double)(v[q] - mx)) : 0.0f;
+            p[q] = e < E ? (RELAXED ? __expf(v[q] - mx) : (float)exp((double)(v[q] - mx))) : 0.0f;
         }
         float s = 0.0f;
+        if (RELAXED) {
 #pragma unroll
-        for (int q = 0; q < VPL; ++q)
-            for (int l = 0; l < GS; ++l) {
-                const float ev = __shfl(p[q], l, GS);
-                if (l + q * GS < E) s = s + ev;
-            }
+            for (int q = 0; q < VPL; ++q) s = s + p[q];
+#pragma unroll
+            for (int m = GS / 2; m >= 1; m >>= 1) s = s + __shfl_xor(s, m, GS);
+        } else {
+#pragma unroll
+            for (int q = 0; q < VPL; ++q)
+                for (int l = 0; l < GS; ++l) {
+                    const float ev = __shfl(p[q], l, GS);
+                    if (l + q * GS < E) s = s + ev;
+                }
+        }
 #pragma unroll
         for (int q = 0; q < VPL; ++q) {
             const int e = sub + q * GS;
@@ -278,12 +248,169 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
     for (int e = tid; e < E; e += 256) tile_counts[(size_t)tile * E + e] = hist[e];
 }
 
+template <int EP, int KC, bool EXACT>
+__global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
+                                                     const float *__restrict__ bg, int T, int d, int E, int K,
+                                                     int renorm, int32_t *__restrict__ ids,
+                                                     float *__restrict__ wout, int32_t *__restrict__ tile_counts,
+                                                     float *__restrict__ logits_out, float *__restrict__ probs_out)
+{
+    constexpr int EPT = ROUTER_EPT(EP), EL = EP / EPT;  // phase 1: experts per thread, threads across the experts
+    constexpr int NT = TOK_TILE * EL / 256;             // tokens per thread in phase 1
+    constexpr int TPP = 256 / EL;                       // tokens per pass
+    constexpr int LDW = KC + 4;  // LDS row stride in floats: rows stay 16-byte aligned and bank-staggered
+    __shared__ __attribute__((aligned(16))) float xs[TOK_TILE][LDW];
+    __shared__ __attribute__((aligned(16))) float ws[EP][LDW];
+    __shared__ float lg[TOK_TILE][EP];
+    __shared__ int hist[EP];
+
+    const int tid = threadIdx.x;
+    const int tile = blockIdx.x;
+    const int t0 = tile * TOK_TILE;
+    const int e1 = tid % EL, tg = tid / EL;
+    if (tid < EP) hist[tid] = 0;
+
+    float acc[NT * EPT];
+#pragma unroll
+    for (int i = 0; i < NT * EPT; ++i) acc[i] = 0.0f;
+
+    const bool fast_io = (d % KC == 0) && (((uintptr_t)x | (uintptr_t)Wg) % 16 == 0);
+    if (dtype == OMEGA_DTYPE_BF16) {
+        if (fast_io) router_sums<EP, KC, EXACT, true, true>(x, Wg, T, d, E, t0, xs, ws, acc);
+        else router_sums<EP, KC, EXACT, true, false>(x, Wg, T, d, E, t0, xs, ws, acc);
+    } else {
+        if (fast_io) router_sums<EP, KC, EXACT, false, true>(x, Wg, T, d, E, t0, xs, ws, acc);
+        else router_sums<EP, KC, EXACT, false, false>(x, Wg, T, d, E, t0, xs, ws, acc);
+    }
+#pragma unroll
+    for (int x_ = 0; x_ < EPT; ++x_) {
+        const int e = e1 + x_ * EL;
+        const float b = (bg != nullptr && e < E) ? bg[e] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            const float z = bg != nullptr ? acc[x_ * NT + i] + b : acc[x_ * NT + i];
+            lg[tg + i * TPP][e] = z;
+            const int t = t0 + tg + i * TPP;
+            if (logits_out != nullptr && t < T && e < E) logits_out[(size_t)t * E + e] = z;
+        }
+    }
+    __syncthreads();
+
+    router_select<EP>(lg, hist, t0, tile, T, E, K, renorm, ids, wout, tile_counts, probs_out);
+}
+
+// FAST mode of bf16 layers with 32 experts or more: the gate projection on the matrix cores.  x and Wg are bf16, so
+// every product is exact in fp32 and only the order of the additions differs from the sequential sum (tolerance
+// mode by definition).  One workgroup = 32 tokens x EP experts = EP/32 blocks of v_mfma_f32_32x32x16_bf16; its four
+// waves split the k range (partial sums are added in a fixed order through LDS) or, from 128 experts on, the blocks.  Operand fragments come straight from memory (16 bytes per lane; the 64 bytes a lane pair
+// needs of a row per 32 k are fetched by consecutive loads, so every line is read once): the kernel moves x once
+// (Wg stays in the L2) and has almost no arithmetic, it lives on loads in flight.
+typedef __attribute__((ext_vector_type(8))) __bf16 rt_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float rt_f32x16;
+
+template <int EP>
+__global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ Wg,
+                                                          const float *__restrict__ bg, int T, int d, int E, int K,
+                                                          int renorm, int32_t *__restrict__ ids, float *__restrict__ wout,
+                                                          int32_t *__restrict__ tile_counts, float *__restrict__ logits_out,
+                                                          float *__restrict__ probs_out)
+{
+    constexpr int NB = EP / 32;                 // expert blocks
+    // up to 64 experts every wave takes all blocks and a quarter of k; from 128 on the waves split the blocks (measured:
+    // 64 experts 0.064 -> 0.058 ms with the k split at T = 8192, d = 2048; 128 experts 0.125 -> 0.157 ms at T = 16384)
+    constexpr int KS = NB <= 2 ? 4 : 1;         // k splits
+    constexpr int BPW = NB <= 2 ? NB : NB / 4;  // expert blocks per wave
+    __shared__ float lg[TOK_TILE][EP];
+    __shared__ float part[KS > 1 ? KS : 1][KS > 1 ? TOK_TILE : 1][KS > 1 ? EP : 1];
+    __shared__ int hist[EP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tile = blockIdx.x, t0 = tile * TOK_TILE;
+    if (tid < EP) hist[tid] = 0;
+    const int l32 = lane & 31, kh = lane >> 5;
+    const int b0 = KS > 1 ? 0 : wave * BPW;           // first expert block of this wave
+    const int ks = KS > 1 ? wave : 0;
+    const int klen = d / KS, kbeg = ks * klen;        // d is a multiple of 256
+    const bf16_t *xrow = x + (size_t)min(t0 + l32, T - 1) * d + kh * 8;
+    const bf16_t *wrow[BPW];
+#pragma unroll
+    for (int b = 0; b < BPW; ++b) wrow[b] = Wg + (size_t)min((b0 + b) * 32 + l32, E - 1) * d + kh * 8;
+    rt_f32x16 acc[BPW];
+#pragma unroll
+    for (int b = 0; b < BPW; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[b][r] = 0.0f;
+    // 64 k per trip: 4 MFMA steps of 16 k; the fragments of the next trip are loaded while this one computes
+    rt_bf16x8 xa[2][4], wb[2][BPW][4];
+    auto fetch = [&](int buf, int k0) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            xa[buf][q] = *(const rt_bf16x8 *)(xrow + k0 + q * 16);
+#pragma unroll
+            for (int b = 0; b < BPW; ++b) wb[buf][b][q] = *(const rt_bf16x8 *)(wrow[b] + k0 + q * 16);
+        }
+    };
+    auto compute = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int b = 0; b < BPW; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[buf][q], wb[buf][b][q], acc[b], 0, 0, 0);
+    };
+    const int kend = kbeg + klen;  // klen is a multiple of 64
+    int k0 = kbeg;
+    fetch(0, k0);
+    for (; k0 + 128 <= kend; k0 += 128) {
+        fetch(1, k0 + 64);
+        compute(0);
+        fetch(0, min(k0 + 128, kend - 64));  // (past the end: re-reads the last trip, never used)
+        compute(1);
+    }
+    if (k0 < kend) compute(0);  // an odd number of trips: the last one sits in buffer 0
+    // lane: expert column l32 of its block; register r -> token 8*(r/4) + 4*kh + r%4
+#pragma unroll
+    for (int b = 0; b < BPW; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int tt = 8 * (r >> 2) + 4 * kh + (r & 3), e = (b0 + b) * 32 + l32;
+            if (KS > 1) part[ks][tt][e] = acc[b][r];
+            else lg[tt][e] = acc[b][r];
+        }
+    __syncthreads();
+    for (int i = tid; i < TOK_TILE * EP; i += 256) {
+        const int tt = i / EP, e = i % EP;
+        float z;
+        if (KS > 1) {
+            z = part[0][tt][e];
+#pragma unroll
+            for (int q = 1; q < KS; ++q) z = z + part[q][tt][e];
+        } else {
+            z = lg[tt][e];
+        }
+        if (bg != nullptr && e < E) z = z + bg[e];
+        lg[tt][e] = z;
+        if (logits_out != nullptr && t0 + tt < T && e < E) logits_out[(size_t)(t0 + tt) * E + e] = z;
+    }
+    __syncthreads();
+    router_select<EP, true>(lg, hist, t0, tile, T, E, K, renorm, ids, wout, tile_counts, probs_out);
+}
+
 hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
     const int tiles = ceil_div(T, TOK_TILE);
     const int exact = c.router_mode == OMEGA_ROUTER_EXACT;
     const float *bg = c.has_gate_bias ? m->bg : nullptr;
+    if (!exact && c.dtype == OMEGA_DTYPE_BF16 && c.E > 16 && ((uintptr_t)x % 16) == 0) {
+#define ROUTER_MFMA_LAUNCH(EPV)                                                                                          \
+    hipLaunchKernelGGL(router_mfma_kernel<EPV>, dim3(tiles), dim3(256), 0, s, (const bf16_t *)x, (const bf16_t *)m->Wg, bg, T, \
+                       c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out, probs_out)
+        if (c.E <= 32) ROUTER_MFMA_LAUNCH(32);
+        else if (c.E <= 64) ROUTER_MFMA_LAUNCH(64);
+        else if (c.E <= 128) ROUTER_MFMA_LAUNCH(128);
+        else ROUTER_MFMA_LAUNCH(256);
+#undef ROUTER_MFMA_LAUNCH
+        return hipGetLastError();
+    }
 #define ROUTER_LAUNCH(EPV, KCV)                                                                                    \
     do {                                                                                                           \
         if (exact)                                                                                                 \
