@@ -29,7 +29,11 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         myrow = dst[(size_t)t * K + lane];
         myw = w[(size_t)t * K + lane];
     }
-    for (int c0 = lane * VEC; c0 < d; c0 += 64 * VEC) {
+    // every lane makes every trip (lanes past the row's end work on column 0 and store nothing): the cross-lane reads
+    // of the slot rows and weights below must find their source lanes active
+    for (int cb = 0; cb < d; cb += 64 * VEC) {
+        const bool on = cb + lane * VEC < d;
+        const int c0 = on ? cb + lane * VEC : 0;
         float acc[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
@@ -83,6 +87,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                 acc[0] = acc[0] + r4.x; acc[1] = acc[1] + r4.y; acc[2] = acc[2] + r4.z; acc[3] = acc[3] + r4.w;
             }
         }
+        if (!on) continue;
         if (BF16) {
             uint32_t pk[VEC / 2];
 #pragma unroll
