@@ -60,3 +60,84 @@ def test_past_the_limits_is_refused():
         a.update(kw)
         with pytest.raises(RuntimeError, match="Error code"):
             G.P.MoELayer(a["embedDim"], a["hidden"], a["nExperts"], a["topK"], nShared=a["nShared"], ctx=G.ctx())
+
+
+def _one_hot_gate(cfg, inp, hot):
+    """A gate that sends every token to expert `hot` first (a huge bias on its row would need has_gate_bias; instead its
+    weight row is aligned with every token's mean direction): returns modified Wg."""
+    Wg = np.zeros_like(inp["Wg"])
+    Wg[hot] = np.float32(4.0) * np.sign(inp["x"].mean(axis=0) + 1e-3).astype(np.float32)
+    return Wg
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_all_tokens_to_one_expert(dtype):
+    """K = 1 and a gate that prefers one expert for (nearly) every token: one group with many row tiles, the others empty
+    or nearly so - forward, backward and exact zeros for the empty experts."""
+    from tests import gpu_util as G
+    cfg = C.MoEConfig("hot", T=1500 if dtype == "bf16" else 300, d=256 if dtype == "bf16" else 40, E=6, K=1,
+                      H=256 if dtype == "bf16" else 24, dtype=dtype)
+    bf = dtype == "bf16"
+    inp = make_inputs(cfg, 8)
+    inp["x"] = (inp["x"] + np.float32(0.75)).astype(np.float32)      # a common direction for the gate to pick up
+    if bf:
+        inp["x"] = O.round_bf16(inp["x"])
+    inp["Wg"] = _one_hot_gate(cfg, inp, 4)
+    dout = O.fill_normal(cfg.T * cfg.d, 8, 900, 1.0).reshape(cfg.T, cfg.d)
+    if bf:
+        dout = O.round_bf16(dout)
+    layer = G.build_layer(cfg, inp)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = G.P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    out = layer.forward(x).to_numpy()
+    ref = G.oracle_forward(cfg, inp)
+    assert ref["counts"][4] > 0.95 * cfg.T                           # the case is what it claims to be
+    G.assert_routing_bit_exact(layer.routing(), ref)
+    tol = 1e-2 if bf else 1e-5
+    assert N.rel_l2(out, ref["out"]) < tol
+    dx = layer.back(g).to_numpy()
+    bw = O.moe_backward(inp["x"], dout, inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], 1, True, 0, bf16=bf)
+    assert N.rel_l2(dx, bw["dx"]) < tol
+    for e in range(cfg.E):
+        for which, k in ((L.W_W1, "dW1"), (L.W_W3, "dW3"), (L.W_W2, "dW2")):
+            got = layer.grad(which, e)
+            if bw[k][e].any():
+                assert N.rel_l2(got, bw[k][e]) < tol, (k, e)
+            else:
+                assert not got.any(), (k, e)
+    layer.close()
+
+
+def test_two_layers_interleaved_and_device_side_copies():
+    """Two layers on one context keep their own workspaces (forward A, forward B, backward A); weights and gradients can
+    be set / fetched device to device."""
+    from tests import gpu_util as G
+    P = G.P
+    cfgA = C.MoEConfig("a", T=64, d=256, E=4, K=2, H=256, dtype="bf16")
+    cfgB = C.MoEConfig("b", T=48, d=64, E=3, K=2, H=40, Es=1, dtype="f32")
+    inpA, inpB = make_inputs(cfgA, 1), make_inputs(cfgB, 2)
+    A, B = G.build_layer(cfgA, inpA), G.build_layer(cfgB, inpB)
+    xA = P.DeviceBuffer.from_numpy(G.ctx(), inpA["x"], "bf16")
+    xB = P.DeviceBuffer.from_numpy(G.ctx(), inpB["x"], "f32")
+    dA = O.round_bf16(O.fill_normal(cfgA.T * cfgA.d, 1, 900, 1.0).reshape(cfgA.T, cfgA.d))
+    dB = O.fill_normal(cfgB.T * cfgB.d, 2, 900, 1.0).reshape(cfgB.T, cfgB.d)
+    gA, gB = P.DeviceBuffer.from_numpy(G.ctx(), dA, "bf16"), P.DeviceBuffer.from_numpy(G.ctx(), dB, "f32")
+    A.forward(xA)
+    B.forward(xB)
+    dxA = A.back(gA).to_numpy()
+    dxB = B.back(gB).to_numpy()
+    rA = O.moe_backward(inpA["x"], dA, inpA["Wg"], None, inpA["W1"], inpA["W3"], inpA["W2"], 2, True, 0, bf16=True)
+    rB = O.moe_backward(inpB["x"], dB, inpB["Wg"], None, inpB["W1"], inpB["W3"], inpB["W2"], 2, True, 1)
+    assert N.rel_l2(dxA, rA["dx"]) < 1e-2 and N.rel_l2(dxB, rB["dx"]) < 1e-5
+    # gradient fetched into a device buffer, weights set from a device buffer
+    gbuf = P.DeviceBuffer(G.ctx(), (cfgB.H, cfgB.d), "f32")
+    G.ctx().check(B.lib.omega_moe_get_grad(B.handle, L.W_W1, 1, gbuf.ptr, 1))
+    assert np.array_equal(gbuf.to_numpy(), B.grad(L.W_W1, 1))
+    wnew = P.DeviceBuffer.from_numpy(G.ctx(), (inpA["W2"][0] * np.float32(0.5)), "bf16")
+    G.ctx().check(A.lib.omega_moe_set_weights(A.handle, L.W_W2, 0, wnew.ptr, 1))
+    assert np.array_equal(A._download_weight(L.W_W2, 0, (cfgA.d, cfgA.H)), O.round_bf16(inpA["W2"][0] * np.float32(0.5)))
+    inpA["W2"][0] = O.round_bf16(inpA["W2"][0] * np.float32(0.5))
+    outA = A.forward(xA).to_numpy()
+    assert N.rel_l2(outA, G.oracle_forward(cfgA, inpA)["out"]) < 1e-2
+    A.close()
+    B.close()
