@@ -1,5 +1,5 @@
 /*
- * libomega_hip.so -- C ABI of the MI355X (gfx950) mixture-of-experts forward path.
+ * libomega_hip.so -- C ABI of the MI355X (gfx950) mixture-of-experts layer: forward, block form, backward, update.
  *
  * Plain C: opaque handles, raw device addresses, sizes and ints.  Every entry point returns an
  * omega_status (0 = OK) and never throws or aborts across the boundary; a human-readable message

@@ -1,4 +1,4 @@
-// C ABI of libomega_hip.so: contexts, device memory, the MoE layer handle and its forward stages.
+// C ABI of libomega_hip.so: contexts, device memory, the MoE layer handle, its forward stages, its backward pass and update.
 #include <stdio.h>
 #include <string.h>
 

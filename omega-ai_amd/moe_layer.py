@@ -10,7 +10,10 @@ argument meaning and error behaviour follow the reference's layers:
   * saveModel/loadModel: raw little-endian float32, no header, fixed order
     (J/engine/nn/network/utils/ModelUtils.java:58-93; order w1,w3,w2 per expert as LlamaMLPLayer.java:273-283)
   * a non-zero status from the library raises RuntimeError("Error code N:msg"), the checkCUDA style
-    (J/engine/gpu/CUDAMemoryManager.java:179-201); back/update raise: the path is forward-only.
+    (J/engine/gpu/CUDAMemoryManager.java:179-201)
+  * back(delta) = initBack -> setDelta -> diff (LlamaMLPLayer.java:186-199), accGrad(scale) and update() without an
+    updater (J/engine/nn/layer/FullyLayer.java:569-607); forward_block / back_block = the second half of
+    LlamaTransformerBlock (norm2 -> mlp -> residual add and its backward, LlamaTransformerBlock.java:134-136,156-158)
 """
 import ctypes as C
 
