@@ -117,7 +117,10 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
         __syncthreads();
         if (k0 + KC < d) fetch(k0 + KC);
         // the products are added one k at a time in index order: EXACT with a separate multiply and add,
-        // FAST with a fused multiply-add (one rounding per step)
+        // FAST with a fused multiply-add (one rounding per step).  With bf16 operands the two are the same
+        // arithmetic: a product of two 8-bit significands has 16 bits and is exact in fp32 (unless it falls below
+        // 2^-134, far outside anything a layer holds), so the separate multiply rounds nothing and EXACT takes the
+        // fused form too - bit for bit the sequential unfused sum, at one instruction per term.
 #define ROUTER_K4(k4)                                                                  \
     do {                                                                               \
         float4 wv[EPT];                                                                \
@@ -129,7 +132,7 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
             _Pragma("unroll") for (int x_ = 0; x_ < EPT; ++x_)                         \
             {                                                                          \
                 float &a_ = acc[x_ * NT + i];                                          \
-                if (EXACT) {                                                           \
+                if (EXACT && !XBF) {                                                   \
                     float prod;                                                        \
                     prod = xv.x * wv[x_].x; a_ = a_ + prod;                            \
                     prod = xv.y * wv[x_].y; a_ = a_ + prod;                            \
