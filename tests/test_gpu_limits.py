@@ -17,6 +17,9 @@ CASES = [
     C.MoEConfig("lim", T=5, d=24, E=12, K=3, H=8, Es=64, renorm=False, dtype="f32"),
     C.MoEConfig("lim", T=40, d=256, E=256, K=16, H=256, Es=1, dtype="bf16", zipf_bias=1.2),
     C.MoEConfig("lim", T=700, d=256, E=2, K=2, H=256, Es=3, dtype="bf16"),       # K = E: every expert takes every token
+    C.MoEConfig("lim", T=37, d=33, E=5, K=2, H=17, Es=1, dtype="f32"),            # odd widths: every scalar fallback
+    C.MoEConfig("lim", T=300, d=256, E=1, K=1, H=256, dtype="bf16"),              # one expert: the dense SwiGLU MLP
+    C.MoEConfig("lim", T=2, d=4, E=2, K=1, H=2, dtype="f32"),                     # tiny
 ]
 
 
@@ -42,7 +45,7 @@ def test_limits_forward_and_backward(cfg):
                         bf16=bf)
     assert N.rel_l2(dx, bw["dx"]) < tol
     assert N.rel_l2(layer.grad(L.W_GATE), bw["dWg"]) < tol
-    for e in (0, cfg.E - 1, cfg.E + cfg.Es - 1):
+    for e in sorted({0, cfg.E - 1, cfg.E + cfg.Es - 1}):
         for which, k in ((L.W_W1, "dW1"), (L.W_W3, "dW3"), (L.W_W2, "dW2")):
             got = layer.grad(which, e)
             if bw[k][e].any():
