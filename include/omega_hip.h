@@ -176,6 +176,15 @@ int omega_moe_get_grad(omega_moe *moe, int which, int expert, void *dst, int is_
 /* accGrad(scale): the first call after an update copies the gradients into the accumulators, later calls add
  * scale * gradient (FullyLayer.accGrad, J/engine/nn/layer/FullyLayer.java:593-607). */
 int omega_moe_acc_grad(omega_moe *moe, float scale);
+/* The layer's share of Network.clipGradNorm (J/engine/nn/network/Network.java:379-432).  grad_sumsq: the sum of the
+ * squares of all parameter gradients of the layer - of the accumulators when accGrad has run since the last update, as
+ * getAccGradNorm / getGradNorm choose (Network.java:325-378) - copied to the host (blocking); what the reference adds
+ * up over its layers as c.syncHost()[0] (Network.java:388-393).  Summed in a fixed order (the reference's
+ * vectorL2NormKernel, J/engine/gpu/GlobalNormKernel.cu:3-30, uses atomicAdd).  scale_grad: the same tensors times
+ * coef, rounded once per element (tensorOP.mul(diffW, clip_coef, diffW), Network.java:401-431).  The caller forms
+ * clip_coef = min(1, gradClip / (sqrt(total) + 1e-6)) from the totals of all its layers. */
+int omega_moe_grad_sumsq(omega_moe *moe, float *sumsq_host);
+int omega_moe_scale_grad(omega_moe *moe, float coef);
 /* update() of a layer without an updater: the accumulated gradients, if any, replace the gradients, then
  * w -= lr * diffW, b -= lr * diffB, and the accumulators are cleared (FullyLayer.update,
  * J/engine/nn/layer/FullyLayer.java:569-590).  The optimisers behind Updater are not part of this library.

@@ -417,6 +417,7 @@ int omega_moe_destroy(omega_moe *m)
         if (p) hipFree(p);
     if (m->dWg) hipFree(m->dWg);
     if (m->acc_grad) hipFree(m->acc_grad);
+    if (m->sumsq_part) hipFree(m->sumsq_part);
     if (m->master) hipFree(m->master);
     if (m->W2T) hipFree(m->W2T);
     if (m->W13T) hipFree(m->W13T);
@@ -740,6 +741,29 @@ int omega_moe_acc_grad(omega_moe *m, float scale)
     } else {
         OMEGA_HIP_CHECK(ctx, launch_axpy_f32(m->acc_grad, m->dWg, scale, n, ctx->stream));
     }
+    return OMEGA_OK;
+}
+
+int omega_moe_grad_sumsq(omega_moe *m, float *sumsq_host)
+{
+    MOE_ENTER(m);
+    if (!m->dWg) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "grad_sumsq: no backward has run");
+    if (!sumsq_host) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "grad_sumsq: destination is NULL");
+    if (!m->sumsq_part) OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->sumsq_part, OMEGA_SUMSQ_SLOTS * sizeof(double)));
+    // the gradients lie in one block whose padding is zero, so one pass covers every tensor
+    OMEGA_HIP_CHECK(ctx, launch_sumsq_f32(m->acc_valid ? m->acc_grad : m->dWg, grad_block_floats(m), m->sumsq_part, ctx->stream));
+    double total = 0.0;
+    OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(&total, m->sumsq_part + OMEGA_SUMSQ_SLOTS - 1, sizeof(double), hipMemcpyDeviceToHost, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+    *sumsq_host = (float)total;
+    return OMEGA_OK;
+}
+
+int omega_moe_scale_grad(omega_moe *m, float coef)
+{
+    MOE_ENTER(m);
+    if (!m->dWg) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "scale_grad: no backward has run");
+    OMEGA_HIP_CHECK(ctx, launch_scale_f32(m->acc_valid ? m->acc_grad : m->dWg, coef, grad_block_floats(m), ctx->stream));
     return OMEGA_OK;
 }
 

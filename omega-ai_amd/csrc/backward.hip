@@ -422,6 +422,64 @@ hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, 
     return hipGetLastError();
 }
 
+// ---- global gradient norm and clipping (Network.clipGradNorm, J/engine/nn/network/Network.java:379-432) ----
+// Sum of squares in two fixed-order stages (vectorL2NormKernel, J/engine/gpu/GlobalNormKernel.cu:3-30, adds its block
+// sums with atomicAdd in arrival order; here the same data always gives the same bits): a thread sums its grid-stride
+// elements in fp32, the workgroup and then one last workgroup add those in double.
+#define SUMSQ_WG 1024
+__global__ __launch_bounds__(256) void bw_sumsq_partial_kernel(const float *__restrict__ src, size_t n, double *__restrict__ part)
+{
+    __shared__ double red[256];
+    float acc = 0.0f;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) acc = fmaf(src[i], src[i], acc);
+    red[threadIdx.x] = (double)acc;
+    __syncthreads();
+    for (int h = 128; h > 0; h >>= 1) {
+        if ((int)threadIdx.x < h) red[threadIdx.x] += red[threadIdx.x + h];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) part[blockIdx.x] = red[0];
+}
+
+__global__ __launch_bounds__(256) void bw_sumsq_final_kernel(const double *__restrict__ part, int np, double *__restrict__ out)
+{
+    __shared__ double red[256];
+    double acc = 0.0;
+    for (int i = threadIdx.x; i < np; i += 256) acc += part[i];
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int h = 128; h > 0; h >>= 1) {
+        if ((int)threadIdx.x < h) red[threadIdx.x] += red[threadIdx.x + h];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = red[0];
+}
+
+// part: SUMSQ_WG + 1 doubles; the result lands in part[SUMSQ_WG]
+hipError_t launch_sumsq_f32(const float *src, size_t n, double *part, hipStream_t s)
+{
+    const int grid = (int)((n + 255) / 256 < SUMSQ_WG ? (n + 255) / 256 : SUMSQ_WG);
+    hipLaunchKernelGGL(bw_sumsq_partial_kernel, dim3(grid > 0 ? grid : 1), dim3(256), 0, s, src, n, part);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(bw_sumsq_final_kernel, dim3(1), dim3(256), 0, s, (const double *)part, grid > 0 ? grid : 1, part + SUMSQ_WG);
+    return hipGetLastError();
+}
+
+// dst *= coef, one rounding per element (TensorOP.mul(diffW, clip_coef, diffW), Network.java:416-431)
+__global__ __launch_bounds__(256) void bw_scale_kernel(float *__restrict__ dst, float coef, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] *= coef;
+}
+
+hipError_t launch_scale_f32(float *dst, float coef, size_t n, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    const int grid = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    hipLaunchKernelGGL(bw_scale_kernel, dim3(grid), dim3(256), 0, s, dst, coef, n);
+    return hipGetLastError();
+}
+
 // ---- update of bf16 layers: fp32 master copies of the weights, the layer's bf16 copies re-rounded from them ----
 // One thread per 16-byte chunk (8 consecutive columns of one row) of the packed tile image of expert blockIdx.y.
 // init != 0: master = weight (first update after the weights were set); else master -= lr * grad, weight = bf16(master).

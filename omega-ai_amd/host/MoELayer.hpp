@@ -255,6 +255,14 @@ public:
     float learnRate = 0.0f;
     void update() override { check(ctx_.get(), omega_moe_update(moe_, learnRate)); }
     void accGrad(float scale) override { check(ctx_.get(), omega_moe_acc_grad(moe_, scale)); }
+    // the layer's part of Network.clipGradNorm (Network.java:379-432): its term of the total, and the scaling
+    float gradSumSq()
+    {
+        float v = 0.0f;
+        check(ctx_.get(), omega_moe_grad_sumsq(moe_, &v));
+        return v;
+    }
+    void scaleGrad(float coef) { check(ctx_.get(), omega_moe_scale_grad(moe_, coef)); }
     // one parameter gradient (fp32, layout of its weight): OMEGA_W_GATE, OMEGA_W_GATE_BIAS, OMEGA_W_W1 / W3 / W2 of expert g
     std::vector<float> grad(int which, int g = 0)
     {

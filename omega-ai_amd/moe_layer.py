@@ -271,6 +271,27 @@ class MoELayer:
     def accGrad(self, scale):
         self.ctx.check(self.lib.omega_moe_acc_grad(self.handle, float(scale)))
 
+    def gradSumSq(self):
+        """Sum of the squares of every parameter gradient of the layer (of the accumulators once accGrad has run): the
+        layer's term of Network.clipGradNorm's total (J/engine/nn/network/Network.java:379-393)."""
+        v = C.c_float(0.0)
+        self.ctx.check(self.lib.omega_moe_grad_sumsq(self.handle, C.byref(v)))
+        return float(v.value)
+
+    def scaleGrad(self, coef):
+        """Gradients (or accumulators) times coef (tensorOP.mul(diffW, clip_coef, diffW), Network.java:401-431)."""
+        self.ctx.check(self.lib.omega_moe_scale_grad(self.handle, float(coef)))
+
+    def clipGradNorm(self, gradClip, other_sumsq=0.0):
+        """Network.clipGradNorm (Network.java:379-432) for a network whose other layers contribute other_sumsq:
+        clip_coef = min(1, gradClip / (sqrt(total) + 1e-6)) in float as there, applied to this layer.  Returns it."""
+        total = np.float32(np.float32(other_sumsq) + np.float32(self.gradSumSq()))
+        coef = np.float32(gradClip / (np.sqrt(np.float64(total)) + np.float64(np.float32(1e-6))))
+        if coef > 1:
+            coef = np.float32(1.0)
+        self.scaleGrad(coef)
+        return float(coef)
+
     def update(self, learnRate):
         """The update of a layer without an updater: w -= learnRate * diffW (FullyLayer.update,
         J/engine/nn/layer/FullyLayer.java:569-590); bf16 layers step fp32 master copies and re-round.  forward() must run

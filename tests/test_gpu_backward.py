@@ -336,3 +336,63 @@ def test_sgd_steps_reduce_a_regression_loss(dtype):
     assert all(b < a for a, b in zip(losses, losses[1:])), losses
     assert losses[-1] < 0.8 * losses[0], losses
     layer.close()
+
+
+def _all_grads(layer, cfg, with_norm):
+    out = [layer.grad(L.W_GATE)]
+    if cfg.zipf_bias:
+        out.append(layer.grad(L.W_GATE_BIAS))
+    if with_norm:
+        out.append(layer.grad(L.W_NORM))
+    for g in range(cfg.E + cfg.Es):
+        out += [layer.grad(L.W_W1, g), layer.grad(L.W_W3, g), layer.grad(L.W_W2, g)]
+    return out
+
+
+@pytest.mark.parametrize("name,kw,block", [
+    ("c1_tiny_f32", dict(T=50, d=48, H=40, E=16, K=2, zipf_bias=1.2), False),
+    ("c1_tiny_f32", dict(T=96, d=64, H=48, E=6, K=3, renorm=False, Es=2), True),
+    ("c2_mixtral", dict(T=300, d=256, H=384), True),
+])
+def test_grad_norm_and_clipping(name, kw, block):
+    """The layer's part of Network.clipGradNorm: its sum of squares against float64 over every gradient tensor read
+    back one by one, the same bits twice, and the scaling exact (one fp32 product per element), on the gradients and,
+    once accGrad has run, on the accumulators."""
+    G, cfg, inp, dout, layer = _setup(name, kw, 17)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = G.P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    with pytest.raises(RuntimeError):
+        layer.gradSumSq()                     # no backward yet
+    if block:
+        layer.set_norm((1.0 + 0.1 * O.fill_normal(cfg.d, 17, 901, 1.0)).astype(np.float32))
+        layer.forward_block(x)
+        layer.back_block(g)
+    else:
+        layer.forward(x)
+        layer.back(g)
+    grads = _all_grads(layer, cfg, block)
+    want = sum(float((a.astype(np.float64) ** 2).sum()) for a in grads)
+    got = layer.gradSumSq()
+    assert abs(got - want) <= 2e-6 * want, (got, want)
+    assert layer.gradSumSq() == got
+    # a clip below the norm: coefficient as Network.clipGradNorm forms it, every tensor scaled by exactly that float
+    clip = 0.5 * np.sqrt(want)
+    coef = layer.clipGradNorm(clip)
+    expect = np.float32(clip / (np.sqrt(np.float64(np.float32(got))) + np.float64(np.float32(1e-6))))
+    assert coef == float(expect) and 0.49 < coef < 0.51
+    after = _all_grads(layer, cfg, block)
+    for a, b in zip(grads, after):
+        assert np.array_equal(b, a * np.float32(coef))
+    assert abs(layer.gradSumSq() - coef * coef * want) <= 1e-5 * want
+    # a clip above the norm leaves everything alone
+    assert layer.clipGradNorm(10.0 * np.sqrt(want)) == 1.0
+    assert all(np.array_equal(a, b) for a, b in zip(after, _all_grads(layer, cfg, block)))
+    # with accumulators the norm and the scaling are theirs: acc = grad, then acc += 1 * grad -> 4 x the sum of squares
+    layer.accGrad(1.0)
+    layer.accGrad(1.0)
+    s_acc = layer.gradSumSq()
+    assert abs(s_acc - 4 * coef * coef * want) <= 1e-5 * 4 * want
+    layer.scaleGrad(0.5)
+    assert abs(layer.gradSumSq() - coef * coef * want) <= 1e-5 * want
+    assert all(np.array_equal(a, b) for a, b in zip(after, _all_grads(layer, cfg, block)))   # the plain gradients were not touched
+    layer.close()
