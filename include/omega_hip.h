@@ -192,6 +192,17 @@ int omega_moe_scale_grad(omega_moe *moe, float coef);
  * they were set, kept across updates) and re-round the weights from them.  The forward pass must run again before the
  * next backward pass. */
 int omega_moe_update(omega_moe *moe, float lr);
+/* update() of a layer whose network uses the AdamW updater (FullyLayer.update -> updater.update(this),
+ * J/engine/nn/layer/FullyLayer.java:569-590; AdamW.update, J/engine/updater/AdamW.java:69-92): every parameter tensor
+ * of the layer - gate weight and bias, expert weights, and the norm weight of the block form, which the reference
+ * steps through updateForBN with the same kernel - takes one step of adamw_kernel
+ * (J/engine/updater/gpu/updater.cu:31-52) with eps = 1e-8 and the bias corrections (float)(1 - pow(beta, train_time))
+ * formed on the host as AdamWKernel.updateW does (J/engine/updater/gpu/AdamWKernel.java:177-195); weight_decay
+ * applies to all of them, as there.  train_time is the network's step counter, starting at 1.  The moments live in
+ * the handle (zero at the first call, kept across set_weights).  Accumulated gradients, bf16 master copies and the
+ * need for a new forward pass are as for omega_moe_update.  Defaults of the reference: beta1 0.9, beta2 0.95
+ * (AdamWKernel.java:25-26), weight_decay 1e-4 (AdamW.java:27). */
+int omega_moe_update_adamw(omega_moe *moe, float lr, float beta1, float beta2, float weight_decay, int train_time);
 
 /* The four stages of forward, callable one at a time (per-stage timing and tests); they use the
  * same kernels and workspace as omega_moe_forward and must be called in this order for one T:

@@ -56,6 +56,7 @@ SIGNATURES = {
     "omega_moe_set_training": (C.c_int, [C.c_void_p, C.c_int]),
     "omega_moe_get_grad": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
     "omega_moe_acc_grad": (C.c_int, [C.c_void_p, C.c_float]),
+    "omega_moe_update_adamw": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int]),
     "omega_moe_grad_sumsq": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
     "omega_moe_scale_grad": (C.c_int, [C.c_void_p, C.c_float]),
     "omega_moe_update": (C.c_int, [C.c_void_p, C.c_float]),

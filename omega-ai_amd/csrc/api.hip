@@ -418,6 +418,8 @@ int omega_moe_destroy(omega_moe *m)
     if (m->dWg) hipFree(m->dWg);
     if (m->acc_grad) hipFree(m->acc_grad);
     if (m->sumsq_part) hipFree(m->sumsq_part);
+    if (m->adam_m) hipFree(m->adam_m);
+    if (m->adam_v) hipFree(m->adam_v);
     if (m->master) hipFree(m->master);
     if (m->W2T) hipFree(m->W2T);
     if (m->W13T) hipFree(m->W13T);
@@ -800,6 +802,44 @@ int omega_moe_update(omega_moe *m, float lr)
         OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W3 + per * g, m->dW13 + per * (2 * g + 1), -lr, per, ctx->stream));
     }
     OMEGA_HIP_CHECK(ctx, launch_axpy_f32((float *)m->W2, m->dW2, -lr, per * m->G, ctx->stream));
+    stage_invalidates(m);  // the weights changed: a backward pass needs a new forward
+    return OMEGA_OK;
+}
+
+int omega_moe_update_adamw(omega_moe *m, float lr, float beta1, float beta2, float weight_decay, int train_time)
+{
+    MOE_ENTER(m);
+    if (!m->dWg) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "update_adamw: no backward has run");
+    if (train_time < 1 || !(beta1 >= 0.0f && beta1 < 1.0f) || !(beta2 >= 0.0f && beta2 < 1.0f))
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "update_adamw: train_time starts at 1 and the betas lie in [0, 1)");
+    const omega_moe_config &c = m->cfg;
+    const size_t n = grad_block_floats(m);
+    if (m->acc_valid) {
+        OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(m->dWg, m->acc_grad, n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        m->acc_valid = false;
+    }
+    if (!m->adam_m) {
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->adam_m, n * 4));
+        if (hipMalloc((void **)&m->adam_v, n * 4) != hipSuccess) {
+            hipFree(m->adam_m);
+            m->adam_m = nullptr;
+            OMEGA_FAIL(ctx, OMEGA_ERR_OOM, "update_adamw: out of device memory for the moments");
+        }
+        OMEGA_HIP_CHECK(ctx, launch_zero_f32(m->adam_m, n, ctx->stream));
+        OMEGA_HIP_CHECK(ctx, launch_zero_f32(m->adam_v, n, ctx->stream));
+    }
+    // the corrections as the reference forms them on the host: (float)(1.0f - Math.pow(beta, train_time))
+    const omega_adamw p = {lr, beta1, beta2, (float)(1.0 - pow((double)beta1, (double)train_time)),
+                           (float)(1.0 - pow((double)beta2, (double)train_time)), 1e-8f, weight_decay};
+    if (c.dtype == OMEGA_DTYPE_BF16) {
+        if (!m->master) OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->master, n * 4));
+        if (!m->master_valid) {
+            OMEGA_HIP_CHECK(ctx, launch_update_bf16(m, m->master, 0.0f, 1, ctx->stream));
+            m->master_valid = true;
+        }
+        m->wT_valid = false;
+    }
+    OMEGA_HIP_CHECK(ctx, launch_update_adamw(m, m->master, m->adam_m, m->adam_v, p, ctx->stream));
     stage_invalidates(m);  // the weights changed: a backward pass needs a new forward
     return OMEGA_OK;
 }

@@ -100,6 +100,8 @@ struct omega_moe {
     float *acc_grad = nullptr;       // accumulators, one block in the order dWg, dbg, dgamma, dW13, dW2
     bool acc_valid = false;          // accGrad has run since the last update
     double *sumsq_part = nullptr;    // scratch of the gradient-norm reduction
+    float *adam_m = nullptr;         // AdamW moments, each laid out like the gradient block (allocated by the first AdamW update)
+    float *adam_v = nullptr;
     float *master = nullptr;         // bf16 layers: fp32 master copies of Wg, W1|W3, W2 (layout of the gradient block)
     bool master_valid = false;       // ... and whether they match the weights (set_weights invalidates)
     float *bw_probs = nullptr;       // [T,E] softmax of the gate logits
@@ -185,6 +187,10 @@ hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, 
 #define OMEGA_SUMSQ_SLOTS 1025  // doubles of scratch launch_sumsq_f32 needs; the result is the last one
 hipError_t launch_sumsq_f32(const float *src, size_t n, double *part, hipStream_t s);
 hipError_t launch_scale_f32(float *dst, float coef, size_t n, hipStream_t s);
+struct omega_adamw {
+    float lr, beta1, beta2, b1c, b2c, eps, wd;  // b1c, b2c: 1 - beta^t, formed on the host
+};
+hipError_t launch_update_adamw(const omega_moe *m, float *master, float *mw, float *vw, const omega_adamw &p, hipStream_t s);
 hipError_t launch_mfma_probe(float *scratch, int num_cus, int random_operands, int launches, hipStream_t s,
                              double *flop_per_launch);
 hipError_t launch_pack_rows(void *dst_packed, const void *src_rowmajor, int R, int Kd, hipStream_t s);

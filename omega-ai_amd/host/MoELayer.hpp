@@ -254,6 +254,11 @@ public:
     // update() of a layer without an updater: w -= learnRate * diffW (FullyLayer.update, FullyLayer.java:569-590)
     float learnRate = 0.0f;
     void update() override { check(ctx_.get(), omega_moe_update(moe_, learnRate)); }
+    // update() under the AdamW updater (AdamW.update, AdamW.java:69-92): trainTime is network.train_time, from 1
+    void updateAdamW(float lr, int trainTime, float beta1 = 0.9f, float beta2 = 0.95f, float weightDecay = 1e-4f)
+    {
+        check(ctx_.get(), omega_moe_update_adamw(moe_, lr, beta1, beta2, weightDecay, trainTime));
+    }
     void accGrad(float scale) override { check(ctx_.get(), omega_moe_acc_grad(moe_, scale)); }
     // the layer's part of Network.clipGradNorm (Network.java:379-432): its term of the total, and the scaling
     float gradSumSq()

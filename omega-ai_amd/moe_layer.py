@@ -298,6 +298,13 @@ class MoELayer:
         again before the next back()."""
         self.ctx.check(self.lib.omega_moe_update(self.handle, float(learnRate)))
 
+    def updateAdamW(self, learnRate, train_time, beta1=0.9, beta2=0.95, weight_decay=1e-4):
+        """update() under the AdamW updater (AdamW.update, J/engine/updater/AdamW.java:69-92; adamw_kernel,
+        J/engine/updater/gpu/updater.cu:31-52): train_time is network.train_time, starting at 1; the defaults are the
+        reference's (AdamWKernel.java:25-26, AdamW.java:27).  forward() must run again before the next back()."""
+        self.ctx.check(self.lib.omega_moe_update_adamw(self.handle, float(learnRate), float(beta1), float(beta2),
+                                                       float(weight_decay), int(train_time)))
+
     # ---- stages and introspection
     def stage(self, name, x=None, out=None):
         T = self.number
@@ -359,7 +366,7 @@ class MoELayer:
 
     # ---- checkpoint: raw LE float32, order gate, (gate bias), then w1,w3,w2 per expert, routed then shared
     def _download_weight(self, which, expert, shape):
-        raw_bf16 = self.dtype == "bf16" and which != L.W_GATE_BIAS
+        raw_bf16 = self.dtype == "bf16" and which not in (L.W_GATE_BIAS, L.W_NORM)   # those two are fp32 in every layer
         h = np.empty(shape, np.uint16 if raw_bf16 else np.float32)
         self.ctx.check(self.lib.omega_moe_get_weights(self.handle, which, expert, h.ctypes.data, 0))
         return bf16_bits_to_f32(h) if raw_bf16 else h

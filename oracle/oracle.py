@@ -54,6 +54,9 @@ def lib():
         L.orc_rmsnorm_backward.argtypes = [_f, _f, _f, _f, C.c_void_p, C.c_int, C.c_int, C.c_int, _f, _f]
         L.orc_block_backward.argtypes = ([_f, _f, _f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8
                                          + [_f, _f, _f, C.c_void_p, _f, _f, _f, _f])
+        L.orc_adamw_correction.restype = C.c_float
+        L.orc_adamw_correction.argtypes = [C.c_float, C.c_int]
+        L.orc_adamw.argtypes = [_f, _f, _f, _f, C.c_long] + [C.c_float] * 7
         L.orc_cpu_baseline_forward.restype = C.c_double
         L.orc_cpu_baseline_forward.argtypes = [_f, _f, C.c_void_p, _f, _f, _f] + [C.c_int] * 8 + [_f]
         L.orc_cpu_sgemm_tn.argtypes = [C.c_int, C.c_int, C.c_int, _f, C.c_int, _f, C.c_int, _f, C.c_int, C.c_int]
@@ -233,6 +236,17 @@ def block_backward(x, gamma, dout, Wg, bg, W1, W3, W2, K, renorm, Es=0, bf16=Fal
                              K, H, Es, int(renorm), int(bf16), r["dx"], r["dgamma"], r["dWg"], _opt(r["dbg"]), r["dW1"],
                              r["dW3"], r["dW2"], r["dh"])
     return r
+
+
+def adamw(w, grad, mw, vw, lr, beta1, beta2, wd, train_time, eps=1e-8):
+    """One AdamW step of the reference's adamw_kernel on flat copies; returns (w, mw, vw) as new arrays."""
+    w, mw, vw = (np.ascontiguousarray(a, np.float32).copy().reshape(-1) for a in (w, mw, vw))
+    g = np.ascontiguousarray(grad, np.float32).reshape(-1)
+    L = lib()
+    L.orc_adamw(w, g, mw, vw, w.size, lr, beta1, beta2, L.orc_adamw_correction(beta1, train_time),
+                L.orc_adamw_correction(beta2, train_time), eps, wd)
+    shape = np.shape(grad)
+    return w.reshape(shape), mw.reshape(shape), vw.reshape(shape)
 
 
 def cpu_baseline_forward(x, Wg, bg, W1, W3, W2, K, renorm, Es, n_threads):
