@@ -397,6 +397,23 @@ __global__ __launch_bounds__(256) void bw_dx_scalar_kernel(const float *__restri
 // FullyLayer.java:581-586)
 __global__ __launch_bounds__(256) void bw_axpy_kernel(float *__restrict__ dst, const float *__restrict__ src, float scale, size_t n)
 {
+    // 16-byte accesses when both pointers allow them
+    if ((((uintptr_t)dst | (uintptr_t)src) & 15) == 0) {
+        const size_t n4 = n >> 2;
+        float4 *d4 = (float4 *)dst;
+        const float4 *s4 = (const float4 *)src;
+        for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
+            float4 v = d4[i];
+            const float4 u = s4[i];
+            v.x = fmaf(scale, u.x, v.x); v.y = fmaf(scale, u.y, v.y); v.z = fmaf(scale, u.z, v.z); v.w = fmaf(scale, u.w, v.w);
+            d4[i] = v;
+        }
+        if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+            const size_t i = (n4 << 2) + threadIdx.x;
+            dst[i] = fmaf(scale, src[i], dst[i]);
+        }
+        return;
+    }
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = fmaf(scale, src[i], dst[i]);
 }
 
@@ -426,13 +443,24 @@ hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, 
 // Sum of squares in two fixed-order stages (vectorL2NormKernel, J/engine/gpu/GlobalNormKernel.cu:3-30, adds its block
 // sums with atomicAdd in arrival order; here the same data always gives the same bits): a thread sums its grid-stride
 // elements in fp32, the workgroup and then one last workgroup add those in double.
-#define SUMSQ_WG 1024
+#define SUMSQ_WG (OMEGA_SUMSQ_SLOTS - 1)
 __global__ __launch_bounds__(256) void bw_sumsq_partial_kernel(const float *__restrict__ src, size_t n, double *__restrict__ part)
 {
     __shared__ double red[256];
-    float acc = 0.0f;
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) acc = fmaf(src[i], src[i], acc);
-    red[threadIdx.x] = (double)acc;
+    // 16 bytes per load, four independent sums per thread; the last n % 4 elements go to the first thread
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+    const size_t n4 = n >> 2;
+    const float4 *src4 = (const float4 *)src;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
+        const float4 v = src4[i];
+        a0 = fmaf(v.x, v.x, a0);
+        a1 = fmaf(v.y, v.y, a1);
+        a2 = fmaf(v.z, v.z, a2);
+        a3 = fmaf(v.w, v.w, a3);
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        for (size_t i = n4 << 2; i < n; ++i) a0 = fmaf(src[i], src[i], a0);
+    red[threadIdx.x] = ((double)a0 + (double)a1) + ((double)a2 + (double)a3);
     __syncthreads();
     for (int h = 128; h > 0; h >>= 1) {
         if ((int)threadIdx.x < h) red[threadIdx.x] += red[threadIdx.x + h];
@@ -458,7 +486,8 @@ __global__ __launch_bounds__(256) void bw_sumsq_final_kernel(const double *__res
 // part: SUMSQ_WG + 1 doubles; the result lands in part[SUMSQ_WG]
 hipError_t launch_sumsq_f32(const float *src, size_t n, double *part, hipStream_t s)
 {
-    const int grid = (int)((n + 255) / 256 < SUMSQ_WG ? (n + 255) / 256 : SUMSQ_WG);
+    const size_t want = (n / 4 + 255) / 256;
+    const int grid = (int)(want < SUMSQ_WG ? want : SUMSQ_WG);
     hipLaunchKernelGGL(bw_sumsq_partial_kernel, dim3(grid > 0 ? grid : 1), dim3(256), 0, s, src, n, part);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -469,7 +498,14 @@ hipError_t launch_sumsq_f32(const float *src, size_t n, double *part, hipStream_
 // dst *= coef, one rounding per element (TensorOP.mul(diffW, clip_coef, diffW), Network.java:416-431)
 __global__ __launch_bounds__(256) void bw_scale_kernel(float *__restrict__ dst, float coef, size_t n)
 {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] *= coef;
+    const size_t n4 = n >> 2;
+    float4 *d4 = (float4 *)dst;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
+        float4 v = d4[i];
+        v.x *= coef; v.y *= coef; v.z *= coef; v.w *= coef;
+        d4[i] = v;
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) dst[(n4 << 2) + threadIdx.x] *= coef;
 }
 
 hipError_t launch_scale_f32(float *dst, float coef, size_t n, hipStream_t s)

@@ -184,7 +184,7 @@ hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, cons
 hipError_t launch_update_bf16(const omega_moe *m, float *master, float lr, int init, hipStream_t s);
 hipError_t launch_zero_f32(float *dst, size_t n, hipStream_t s);
 hipError_t launch_axpy_f32(float *dst, const float *src, float scale, size_t n, hipStream_t s);
-#define OMEGA_SUMSQ_SLOTS 1025  // doubles of scratch launch_sumsq_f32 needs; the result is the last one
+#define OMEGA_SUMSQ_SLOTS 2049  // doubles of scratch launch_sumsq_f32 needs; the result is the last one
 hipError_t launch_sumsq_f32(const float *src, size_t n, double *part, hipStream_t s);
 hipError_t launch_scale_f32(float *dst, float coef, size_t n, hipStream_t s);
 struct omega_adamw {
