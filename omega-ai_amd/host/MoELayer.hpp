@@ -10,7 +10,9 @@
 //                    saveModel/loadModel write raw little-endian float32 in the order gate, (gate bias), then
 //                    w1,w3,w2 per expert (routed, then shared), as LlamaMLPLayer.java:273-283 does for one MLP;
 //                    a failing library call throws std::runtime_error("Error code N:msg"), the checkCUDA style
-//                    (J/engine/gpu/CUDAMemoryManager.java:179-201); back/update throw: the path is forward-only.
+//                    (J/engine/gpu/CUDAMemoryManager.java:179-201); back(Tensor) = initBack -> setDelta -> diff
+//                    (LlamaMLPLayer.java:186-199), update()/accGrad() as FullyLayer.java:569-607, the AdamW branch
+//                    and the layer's part of Network.clipGradNorm beside them.
 // Host tensors are fp32 like the reference's; a bf16 layer converts on the device at the boundary.
 #pragma once
 #include <cstdint>
@@ -289,6 +291,22 @@ public:
         check(ctx_.get(), omega_moe_get_routing(moe_, number, ids.data(), w.data(), counts.data(), nullptr, nullptr, nullptr));
     }
 
+    // the block form's parameters in the order LlamaTransformerBlock.saveModel writes them for its FFN half: norm2
+    // (RMSLayer.saveModel: gamma), then the mlp (J/engine/nn/layer/llama/LlamaTransformerBlock.java:263-275)
+    void saveModelBlock(FILE *f)
+    {
+        std::vector<float> g(embedDim_);
+        check(ctx_.get(), omega_moe_get_weights(moe_, OMEGA_W_NORM, 0, g.data(), 0));
+        if (fwrite(g.data(), 4, g.size(), f) != g.size()) throw std::runtime_error("Error code 1:short write");
+        saveModel(f);
+    }
+    void loadModelBlock(FILE *f)
+    {
+        std::vector<float> g(embedDim_);
+        if (fread(g.data(), 4, g.size(), f) != g.size()) throw std::runtime_error("Error code 1:checkpoint ends early");
+        setNorm(g.data());
+        loadModel(f);
+    }
     void saveModel(FILE *f) { eachParam([&](int which, int g, size_t n) { std::vector<float> h = download(which, g, n); if (fwrite(h.data(), 4, n, f) != n) throw std::runtime_error("Error code 1:short write"); }); }
     void loadModel(FILE *f) { eachParam([&](int which, int g, size_t n) { std::vector<float> h(n); if (fread(h.data(), 4, n, f) != n) throw std::runtime_error("Error code 1:checkpoint ends early"); if (which == OMEGA_W_GATE_BIAS) check(ctx_.get(), omega_moe_set_weights(moe_, which, g, h.data(), 0)); else upload(which, g, h.data(), n); }); }
 

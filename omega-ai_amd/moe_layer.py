@@ -392,6 +392,19 @@ class MoELayer:
                 raise RuntimeError("Error code 1:checkpoint ends early")
             self._upload(which, g, np.frombuffer(buf, "<f4").reshape(shape))
 
+    def saveModelBlock(self, f):
+        """The block form's parameters in the order LlamaTransformerBlock.saveModel writes its FFN half: norm2 (gamma,
+        RMSLayer.saveModel), then the mlp (J/engine/nn/layer/llama/LlamaTransformerBlock.java:263-275)."""
+        f.write(self._download_weight(L.W_NORM, 0, (self.embedDim,)).astype("<f4").tobytes())
+        self.saveModel(f)
+
+    def loadModelBlock(self, f):
+        buf = f.read(4 * self.embedDim)
+        if len(buf) != 4 * self.embedDim:
+            raise RuntimeError("Error code 1:checkpoint ends early")
+        self.set_norm(np.frombuffer(buf, "<f4").copy())
+        self.loadModel(f)
+
     def initJava(self, seed, mean=0.01, std=0.02):
         """RandomUtils.setSeed(seed) followed by the house-style initialisation (java_random.init_layer): the weights a
         Java run of the reference would draw.  Returns the arrays that were set."""

@@ -156,3 +156,36 @@ def test_block_backward_matches_oracle(name, kw, training):
     layer.back(g)
     assert not layer.grad(L.W_NORM).any()
     layer.close()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_block_checkpoint_round_trip(dtype):
+    """saveModelBlock / loadModelBlock: norm weight first, then the layer, raw little-endian float32, byte-exact; a layer
+    loaded from it gives the same block output bit for bit."""
+    import importlib
+    import io
+    from tests import gpu_util as G
+    L = importlib.import_module("omega-ai_amd._lib")
+    cfg = scaled(C.CONFIGS["c2_mixtral"], T=40, d=256, H=256, E=4, K=2, Es=1, dtype=dtype)
+    inp = make_inputs(cfg, 71)
+    gamma = _gamma(cfg.d, 71)
+    layer = G.build_layer(cfg, inp)
+    layer.set_norm(gamma)
+    f = io.BytesIO()
+    layer.saveModelBlock(f)
+    raw = f.getvalue()
+    rnd = O.round_bf16 if dtype == "bf16" else (lambda a: a)
+    expect = np.concatenate([gamma.ravel(), rnd(inp["Wg"]).ravel()] +
+                            [np.concatenate([rnd(inp["W1"][g]).ravel(), rnd(inp["W3"][g]).ravel(), rnd(inp["W2"][g]).ravel()])
+                             for g in range(cfg.E + cfg.Es)]).astype("<f4").tobytes()
+    assert raw == expect
+    other = G.P.MoELayer(cfg.d, cfg.H, cfg.E, cfg.K, cfg.renorm, cfg.Es, False, ctx=G.ctx(), dtype=dtype)
+    other.loadModelBlock(io.BytesIO(raw))
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    assert np.array_equal(other.forward_block(x).to_numpy(), layer.forward_block(x).to_numpy())
+    with pytest.raises(RuntimeError, match="Error code"):
+        other.loadModelBlock(io.BytesIO(raw[:cfg.d * 4 - 8]))
+    with pytest.raises(RuntimeError, match="Error code"):
+        other.loadModelBlock(io.BytesIO(raw[:cfg.d * 4 + 100]))
+    layer.close()
+    other.close()
