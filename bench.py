@@ -132,13 +132,27 @@ def main():
         layer.forward(x)
         bw_train_ms = layer.time_backward(x, gbuf, cfg.T, dxb, warmup=2, iters=max(3, a.steps // 2))
         layer.set_training(False)
+        # optimiser step: AdamW on every parameter (learning rate 0: same traffic, weights unchanged), wall clock
+        # around a synchronised batch of calls; 30 bytes move per expert parameter of a bf16 layer (fp32 master, two
+        # moments and gradient read; master, moments and the bf16 weight written), 28 of an fp32 layer
+        layer.updateAdamW(0.0, 1, weight_decay=0.0)
+        ctx.sync()
+        t_up = time.perf_counter()
+        for i in range(3):
+            layer.updateAdamW(0.0, 2 + i, weight_decay=0.0)
+        ctx.sync()
+        adamw_ms = (time.perf_counter() - t_up) / 3 * 1e3
+        n_params = 3.0 * (cfg.E + cfg.Es) * cfg.H * cfg.d + cfg.E * cfg.d
+        adamw_bytes = n_params * (30.0 if cfg.dtype == "bf16" else 28.0)
         bw_flops = 12.0 * cfg.d * cfg.H * rows
         backward = {"what": "omega_moe_backward: dx and all parameter gradients (fp32) for one dout",
                     "ms": bw_ms, "algorithmic_TFLOP/s": bw_flops / (bw_ms * 1e-3) / 1e12,
                     "training_mode": {"forward_ms": fwd_train_ms, "backward_ms": bw_train_ms,
                                       "algorithmic_TFLOP/s": bw_flops / (bw_train_ms * 1e-3) / 1e12,
                                       "frac_mfma": bw_flops / (bw_train_ms * 1e-3) / 1e12 / peak,
-                                      "fwd+bwd_tokens/s": cfg.T / ((fwd_train_ms + bw_train_ms) * 1e-3)}}
+                                      "fwd+bwd_tokens/s": cfg.T / ((fwd_train_ms + bw_train_ms) * 1e-3)},
+                    "adamw_update": {"ms": adamw_ms, "parameters": n_params, "bound": "hbm",
+                                     "achieved_GB/s": adamw_bytes / (adamw_ms * 1e-3) / 1e9, "frac_hbm": adamw_bytes / (adamw_ms * 1e-3) / 8e12}}
         gbuf.free()
         dxb.free()
 
