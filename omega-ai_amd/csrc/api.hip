@@ -418,6 +418,7 @@ int omega_moe_destroy(omega_moe *m)
     if (m->dWg) hipFree(m->dWg);
     if (m->acc_grad) hipFree(m->acc_grad);
     if (m->sumsq_part) hipFree(m->sumsq_part);
+    if (m->y_slabs) hipFree(m->y_slabs);
     if (m->adam_m) hipFree(m->adam_m);
     if (m->adam_v) hipFree(m->adam_v);
     if (m->master) hipFree(m->master);
@@ -541,7 +542,18 @@ static int stage_dispatch(omega_moe *m, const void *x, int T)
     const int bm = moe_tile_m(m, T);
     m->bm = bm;
     m->max_m_tiles = moe_max_m_tiles(m, T, bm);
-    if (m->cfg.dtype == OMEGA_DTYPE_BF16) m->down_cols = m->max_m_tiles * (m->cfg.d / 256) <= m->n_wg / 2 ? 128 : 256;
+    if (m->cfg.dtype == OMEGA_DTYPE_BF16) {
+        // A batch whose down product has output tiles for at most half of the compute units is bound by the weight
+        // bytes each workgroup keeps in flight.  With H >= 512 the table builder then cuts every tile's k range into
+        // up to 8 slices (as many as fill the compute units; it knows how many experts have rows), which write partial
+        // results that a small kernel adds up; narrower layers get 128-column items instead.
+        const bool small = m->max_m_tiles * (m->cfg.d / 256) <= m->n_wg / 2;
+        m->down_ks_max = small && m->cfg.H >= 512 ? 8 : 1;
+        m->down_cols = small && m->down_ks_max == 1 ? 128 : 256;
+        // slices x tiles never exceed n_wg, so all partial results together are smaller than n_wg tiles of 256 x 256
+        if (m->down_ks_max > 1 && !m->y_slabs)
+            OMEGA_HIP_CHECK(m->ctx, hipMalloc((void **)&m->y_slabs, (size_t)m->n_wg * 256 * 256 * 4));
+    }
     if (m->max_m_tiles > m->tiles_cap) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: workspace too small for this T");
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));

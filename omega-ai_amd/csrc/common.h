@@ -86,6 +86,8 @@ struct omega_moe {
     // columns of a work item of the down product: 256, or 128 when 256-column tiles would leave at least half of the
     // compute units without an item (a few tokens: the product is bound by streaming W2, which every unit must share)
     int down_cols = 256;
+    int down_ks_max = 1;             // > 1: the down table of this batch may hold k slices (small batches)
+    float *y_slabs = nullptr;        // their partial results 1 .. KS-1, each laid out like the rows of y in use
     void *xg = nullptr;              // [rows_cap,d]  gathered tokens (bf16: packed tile image, see pack.h)
     void *xs = nullptr;              // bf16 with shared experts: packed copy of x, [ceil(T/bm)*bm,d]
     void *a = nullptr;               // [rows_cap,H]  (bf16: packed tile image)
@@ -178,7 +180,7 @@ hipError_t launch_transpose_groups(const omega_moe *m, const void *src, const vo
 hipError_t launch_transpose_images(const void *src, int R, int cols, void *dst, int KTd, int k0, int n, size_t src_stride,
                                    size_t dst_stride, hipStream_t s);
 // products of the matrix-core kernel (experts_bf16.hip describes each)
-enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4, MODE_UPREC = 5 };
+enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4, MODE_UPREC = 5, MODE_DOWNK = 6 };
 hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, const void *Aalt, const void *Wa, const void *Wb,
                                void *Cout, void *Aux1, void *Aux2, const omega_tile_desc *wq, int N, int Kd, hipStream_t s);
 hipError_t launch_update_bf16(const omega_moe *m, float *master, float lr, int init, hipStream_t s);

@@ -54,12 +54,23 @@ __global__ __launch_bounds__(256) void dispatch_scan_kernel(const int32_t *__res
 
 // The work items of group g in one product's table (see the comment in dispatch_rank_kernel): NT column tiles of
 // ncols columns, Mg row tiles starting at row tile mt0; the launch has total_mt row tiles in all.  All 256 threads.
+// K slices of a table (small batches of the down product, see write_group_items): Nt output tiles that would leave
+// at least half of the 256 compute units idle are each cut into KS <= ks_max slices of the k range, at least 8 k steps
+// long; 1 = no slicing.
+__device__ __forceinline__ int table_k_slices(int Nt, int ks_max, int KT)
+{
+    if (ks_max <= 1 || Nt <= 0 || Nt > 128) return 1;
+    return max(1, min(min(ks_max, 256 / Nt), KT / 8));
+}
+
 __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ desc, int NT, int ncols, int g, int rows,
-                                                  int Mg, int mt0, int total_mt, int bm, bool shared)
+                                                  int Mg, int mt0, int total_mt, int bm, bool shared, int ks_max = 1,
+                                                  int KT = 0)
 {
     if (desc == nullptr) return;
     const int Nt = total_mt * NT, r = Nt % 256;
-    const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
+    const int KS = table_k_slices(Nt, ks_max, KT);
+    const int S = (r == 0 || r > 128 || KS > 1) ? 1 : min(4, 256 / r);
     const int nblk = (rows + 31) >> 5;  // 32-row blocks of the group, dealt evenly to its Mg row tiles
     for (int l = threadIdx.x; l < Mg * NT; l += 256) {
         const int mt = l % Mg, n = l / Mg;
@@ -71,7 +82,18 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
         dsc.n0 = n * ncols;
         dsc.a_rg = dsc.kt0 = 0;
         dsc.b_rg = ncols == 128 ? 1 : 0;  // read by the plain 256-column products only: a half-width item
-        if (at < Nt - r) {
+        if (KS > 1) {
+            // slice ks of KS (a_rg = KS, kt0 = ks) adds its part of the k range into partial result ks; adjacent
+            // entries, so the slices of a tile run on one XCD and share its rows
+            dsc.row0 = mt0 * bm + tfirst;
+            dsc.rows = trows;
+            dsc.xrow0 = shared ? tfirst : -1;
+            dsc.a_rg = KS;
+            for (int ks = 0; ks < KS; ++ks) {
+                dsc.kt0 = ks;
+                desc[at * KS + ks] = dsc;
+            }
+        } else if (at < Nt - r) {
             dsc.row0 = mt0 * bm + tfirst;
             dsc.rows = trows;
             dsc.xrow0 = shared ? tfirst : -1;
@@ -90,9 +112,11 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
 }
 
 // entries of a table whose launch has total_mt row tiles and NT column tiles (with the last tiles sliced)
-__device__ __forceinline__ int table_entries(int total_mt, int NT)
+__device__ __forceinline__ int table_entries(int total_mt, int NT, int ks_max = 1, int KT = 0)
 {
     const int Nt = total_mt * NT, r = Nt % 256;
+    const int KS = table_k_slices(Nt, ks_max, KT);
+    if (KS > 1) return Nt * KS;
     const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
     return Nt - r + r * S;
 }
@@ -109,7 +133,7 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
                                                             int32_t *__restrict__ tile_meta,
                                                             omega_tile_desc *__restrict__ desc_up, int nt_up, int ncols_up,
                                                             omega_tile_desc *__restrict__ desc_down, int nt_down,
-                                                            int ncols_down)
+                                                            int ncols_down, int ks_max_down, int kt_down)
 {
     __shared__ int off_s[MAXE + 1];        // logical first row of each expert
     __shared__ int mt_s[MAXE + 64 + 1];    // first row tile of each group (routed, then shared)
@@ -193,12 +217,16 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     // the weight tile in its L2).  Group g is written by workgroup g (mod grid).
     if (desc_up != nullptr || desc_down != nullptr) {
         const int G = E + Es;
-        if (tile == 0 && tid < 2) tile_meta[G + 2 + tid] = table_entries(mt_s[G], tid == 0 ? nt_up : nt_down);
+        if (tile == 0 && tid == 0) {
+            tile_meta[G + 2] = table_entries(mt_s[G], nt_up);
+            tile_meta[G + 3] = table_entries(mt_s[G], nt_down, ks_max_down, kt_down);
+            tile_meta[G + 7] = table_k_slices(mt_s[G] * nt_down, ks_max_down, kt_down);  // partial results of the down product
+        }
         for (int g = tile; g < G; g += gridDim.x) {
             const int rows = g < E ? off_s[g + 1] - off_s[g] : T;
             const int Mg = mt_s[g + 1] - mt_s[g];
             write_group_items(desc_up, nt_up, ncols_up, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E);
-            write_group_items(desc_down, nt_down, ncols_down, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E);
+            write_group_items(desc_down, nt_down, ncols_down, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E, ks_max_down, kt_down);
         }
     }
 }
@@ -404,7 +432,7 @@ hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t 
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(dispatch_rank_kernel, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_base, m->counts, T, c.K,
                        c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles, m->tile_meta, m->desc_up, c.H / 128, 128,
-                       m->desc_down, c.d / m->down_cols, m->down_cols);
+                       m->desc_down, c.d / m->down_cols, m->down_cols, m->down_ks_max, c.H / 32);
     return hipGetLastError();
 }
 

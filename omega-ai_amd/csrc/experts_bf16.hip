@@ -47,7 +47,9 @@
 //          whose K axis is the experts' rows; the item names its operand row groups, first k step and k steps
 //          (a_rg, b_rg, kt0, xrow0); fp32 row-major output, row0 = expert * M + first row
 #define FUSED_TILE(M) ((M) == MODE_UP || (M) == MODE_UPRAW || (M) == MODE_UPREC)
-#define SWAPPED(M) ((M) != MODE_DOWN && (M) != MODE_WGRAD)
+#define PLAIN_DOWN(M) ((M) == MODE_DOWN || (M) == MODE_DOWNK)
+#define SWAPPED(M) (!PLAIN_DOWN(M) && (M) != MODE_WGRAD)
+#define ITEM_K(M) ((M) == MODE_WGRAD || (M) == MODE_DOWNK)  // the k range belongs to the item, not to the launch
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -91,6 +93,7 @@ struct TileCtx {
     int row0, rows, n0;
     int kt;                   // k steps of the item
     int half;                 // plain 256-column products: the item covers the first 128 columns only
+    int slab;                 // MODE_DOWNK: which partial result the item writes
 };
 
 __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char *p)
@@ -123,12 +126,24 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
         return c;
     }
     c.kt = KT;
+    c.slab = 0;
     c.half = FUSED ? 0 : d.b_rg;
-    c.A = uniform_ptr((MODE != MODE_DOWN && Ax != nullptr && d.xrow0 >= 0)
-                          ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
-                          : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes);
+    // k slices (tables of small batches, items with a_rg = KS > 1 and kt0 = ks): MODE_DOWNK runs slice ks over its own
+    // part of the k range; a launch that knows nothing of partial results (MODE_DOWN) computes the whole range in the
+    // item of slice 0 and only keeps the other slices' workgroups in step (no rows: loads and barriers, no results)
+    size_t k0 = 0;
+    if (MODE == MODE_DOWNK && d.a_rg > 1) {
+        const int first = (d.kt0 * KT) / d.a_rg;  // even parts: every slice has at least KT / KS >= 8 steps
+        c.kt = ((d.kt0 + 1) * KT) / d.a_rg - first;
+        c.slab = d.kt0;
+        k0 = (size_t)first * 8192;
+    }
+    if (MODE == MODE_DOWN && d.a_rg > 1 && d.kt0 > 0) c.rows = 0;
+    c.A = uniform_ptr(((!PLAIN_DOWN(MODE) && Ax != nullptr && d.xrow0 >= 0)
+                           ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
+                           : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes) + k0);
     const size_t wrg = (size_t)d.g * (N >> 7) + (d.n0 >> 7);  // row group of the weight tile
-    c.B0 = uniform_ptr((const unsigned char *)Wa + wrg * rg_bytes);
+    c.B0 = uniform_ptr((const unsigned char *)Wa + wrg * rg_bytes + k0);
     // (a half-width item loads its 128 weight rows twice - the second copy comes out of the L2 - and drops the results
     //  of the duplicate: the products it is used for are bound by streaming the weights from memory, not by the MFMAs)
     c.B1 = uniform_ptr(FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : c.half ? c.B0 : c.B0 + rg_bytes);
@@ -179,12 +194,13 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     ctx.rows = __builtin_amdgcn_readfirstlane(ctx_in.rows);
     ctx.n0 = __builtin_amdgcn_readfirstlane(ctx_in.n0);
     ctx.half = __builtin_amdgcn_readfirstlane(ctx_in.half);
+    ctx.slab = __builtin_amdgcn_readfirstlane(ctx_in.slab);
     int cur = __builtin_amdgcn_readfirstlane(cur_io);
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     const uint32_t lds_wave = lds0 + wave * 1024;
     const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
-    const int KT = MODE == MODE_WGRAD ? __builtin_amdgcn_readfirstlane(ctx_in.kt) : Kd / BK;
+    const int KT = ITEM_K(MODE) ? __builtin_amdgcn_readfirstlane(ctx_in.kt) : Kd / BK;
     const bool has_next = dn.rows > 0;
 
 // load n of virtual k step v: steps beyond this item's last belong to the next item
@@ -367,7 +383,12 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
                 }
             }
         }
-    } else if ((MODE == MODE_DOWN || MODE == MODE_WGRAD) && !(ctx.half && wn >= 2)) {
+    } else if ((PLAIN_DOWN(MODE) || MODE == MODE_WGRAD) && !(ctx.half && wn >= 2)) {
+        // MODE_DOWNK: slice 0 writes the output itself, slice s > 0 partial result s - 1 of those behind Aux1, each laid
+        // out like the rows of the output that are in use (Aux2[0] row tiles)
+        float *Cbase = (float *)Cout;
+        if (MODE == MODE_DOWNK && ctx.slab > 0)
+            Cbase = (float *)Aux1 + (size_t)(ctx.slab - 1) * ((size_t)((const int32_t *)Aux2)[0] * BM * N);
         // lane: column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
@@ -377,10 +398,10 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
                 if (row >= ctx.rows) continue;
                 // (32 lanes x 4 bytes = one 128-byte line per store; 16-byte stores of a transposed accumulator layout
                 //  write 32-byte pieces of 32 different lines and were 8 % slower on short-K shapes)
-                float *out = (float *)Cout + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l32;
+                float *out = Cbase + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l32;
 #pragma unroll
                 for (int j = 0; j < 2; ++j)  // (non-temporal stores of the weight gradients were 10 % slower)
-                    if (MODE == MODE_DOWN || ctx.n0 + wn * 64 + j * 32 < N) out[j * 32] = acc[i][j][r];
+                    if (PLAIN_DOWN(MODE) || ctx.n0 + wn * 64 + j * 32 < N) out[j * 32] = acc[i][j][r];
             }
         }
     }
@@ -439,11 +460,35 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
     }
 }
 
+// y += partial results 1 .. KS-1 of a k-sliced down product, in that order; KS comes from the table builder
+// (tile_meta[ks_slot]).  Workgroup (t, c): the valid rows of row tile t, columns c*1024 .. (16 bytes per lane and trip).
+__global__ __launch_bounds__(256) void down_slab_reduce_kernel(float *__restrict__ y, const float *__restrict__ slabs,
+                                                               const omega_tile *__restrict__ tiles,
+                                                               const int32_t *__restrict__ tile_meta, int ks_slot, int d)
+{
+    const int KS = tile_meta[ks_slot];
+    if (KS <= 1 || (int)blockIdx.x >= tile_meta[0]) return;
+    const size_t slab_floats = (size_t)tile_meta[0] * BM * d;
+    const omega_tile tl = tiles[blockIdx.x];
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+    if (c >= d) return;
+    for (int r = 0; r < tl.rows; ++r) {
+        const size_t o = (size_t)(tl.row0 + r) * d + c;
+        float4 v = *(const float4 *)(y + o);
+        for (int s = 0; s < KS - 1; ++s) {
+            const float4 u = *(const float4 *)(slabs + (size_t)s * slab_floats + o);
+            v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
+        }
+        *(float4 *)(y + o) = v;
+    }
+}
+
 hipError_t experts_bf16_init(void)
 {
     const void *fns[] = {(const void *)experts_bf16_kernel<MODE_UP>, (const void *)experts_bf16_kernel<MODE_DOWN>,
                          (const void *)experts_bf16_kernel<MODE_UPRAW>, (const void *)experts_bf16_kernel<MODE_DA>,
-                         (const void *)experts_bf16_kernel<MODE_WGRAD>, (const void *)experts_bf16_kernel<MODE_UPREC>};
+                         (const void *)experts_bf16_kernel<MODE_WGRAD>, (const void *)experts_bf16_kernel<MODE_UPREC>,
+                         (const void *)experts_bf16_kernel<MODE_DOWNK>};
     for (const void *f : fns) {
         hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
         if (e != hipSuccess) return e;
@@ -467,6 +512,15 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
         hipLaunchKernelGGL(experts_bf16_kernel<MODE_UP>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
                            (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
                            (void *)nullptr, m->wq_up, c.H, c.d);
+    } else if (m->down_ks_max > 1) {
+        // small batch: the table may hold k slices; their partial results are added into y right behind the product
+        hipLaunchKernelGGL(experts_bf16_kernel<MODE_DOWNK>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
+                           (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y,
+                           (void *)m->y_slabs, (void *)m->tile_meta, m->wq_down, c.d, c.H);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(down_slab_reduce_kernel, dim3(m->max_m_tiles, ceil_div(c.d, 1024)), dim3(256), 0, s, m->y,
+                           (const float *)m->y_slabs, m->tiles, m->tile_meta, m->G + 7, c.d);
     } else {
         hipLaunchKernelGGL(experts_bf16_kernel<MODE_DOWN>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
                            (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y,
@@ -490,6 +544,7 @@ hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, cons
         case MODE_DA: LAUNCH(MODE_DA); break;
         case MODE_WGRAD: LAUNCH(MODE_WGRAD); break;
         case MODE_UPREC: LAUNCH(MODE_UPREC); break;
+        case MODE_DOWNK: LAUNCH(MODE_DOWNK); break;
         default: return hipErrorInvalidValue;
     }
 #undef LAUNCH

@@ -135,6 +135,38 @@ def test_bf16_scaled_configs(G, name, kw):
     layer.close()
 
 
+@pytest.mark.parametrize("T,d,H,E,K,Es", [
+    (1, 512, 1024, 8, 2, 0),      # two experts with one row each: 32 k steps in 4 slices (no slice under 8 steps)
+    (3, 256, 2048, 8, 2, 0),      # 8 slices of 8 steps
+    (5, 512, 896, 8, 2, 0),       # 28 k steps in 3 uneven slices (9, 9, 10)
+    (17, 256, 640, 4, 2, 1),      # shared expert rows among the sliced tiles, 20 k steps in 2 slices
+    (64, 512, 1024, 8, 2, 0),     # every expert has rows: 2 slices
+    (40, 1024, 512, 16, 4, 0),    # 16 experts x 4 column tiles: 2 slices
+])
+def test_bf16_small_batches_slice_the_down_product(G, T, d, H, E, K, Es):
+    """Small batches: the down product's k range is cut into slices whose partial results are added up behind it.
+    Output and the y buffer against the oracle, the same bits on a second call, and a large batch on the same layer
+    in between (which takes the unsliced path) leaves the small one unchanged."""
+    cfg = scaled(C.CONFIGS["c2_mixtral"], T=T, d=d, H=H, E=E, K=K, Es=Es)
+    layer, x, out, r, ref, inp = G.run_case(cfg, seed=777)
+    G.assert_routing_bit_exact(r, ref)
+    assert N.rel_l2(out, ref["out"]) <= BF16_TOL
+    y = layer.workspace("y", cfg.T)
+    a = layer.workspace("a", cfg.T)
+    # y = a . W2^T row by row in float64 from the rows the layer itself holds (pins the sum of the partial results)
+    g_of_row = np.repeat(np.arange(E), r["counts"])
+    for row in range(0, T * K, max(1, T * K // 7)):
+        want = inp["W2"][g_of_row[row]].astype(np.float64) @ a[row].astype(np.float64)
+        assert N.rel_l2(y[row], want) < 1e-5, row
+    big = make_inputs(scaled(cfg, T=900), 778)
+    xb = G.P.DeviceBuffer.from_numpy(G.ctx(), big["x"], cfg.dtype)
+    ob = layer.forward(xb).to_numpy()
+    refb = G.oracle_forward(scaled(cfg, T=900), {**big, **{k: inp[k] for k in ("Wg", "bg", "W1", "W3", "W2")}})
+    assert N.rel_l2(ob, refb["out"]) <= BF16_TOL
+    assert np.array_equal(layer.forward(x).to_numpy(), out)
+    layer.close()
+
+
 def test_bf16_fast_router_agrees(G):
     cfg = scaled(C.CONFIGS["c2_mixtral"], T=512, d=512, H=1024)
     layer, x, out, r, ref, inp = G.run_case(cfg, seed=4242, router_mode="fast")
