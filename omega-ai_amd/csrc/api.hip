@@ -547,8 +547,12 @@ static int stage_dispatch(omega_moe *m, const void *x, int T)
         // bytes each workgroup keeps in flight.  With H >= 512 the table builder then cuts every tile's k range into
         // up to 8 slices (as many as fill the compute units; it knows how many experts have rows), which write partial
         // results that a small kernel adds up; narrower layers get 128-column items instead.
-        const bool small = m->max_m_tiles * (m->cfg.d / 256) <= m->n_wg / 2;
-        m->down_ks_max = small && m->cfg.H >= 512 ? 8 : 1;
+        // (The host knows only bounds of the number of row tiles: slicing is switched on when the fewest tiles this
+        //  batch can have would qualify, and the table builder decides by the tiles there are.)
+        const omega_moe_config &c = m->cfg;
+        const int min_tiles = ceil_div(T * c.K, bm) + c.Es * ceil_div(T, bm);
+        const bool small = m->max_m_tiles * (c.d / 256) <= m->n_wg / 2;
+        m->down_ks_max = min_tiles * (c.d / 256) <= m->n_wg / 2 && c.H >= 512 ? 8 : 1;
         m->down_cols = small && m->down_ks_max == 1 ? 128 : 256;
         // slices x tiles never exceed n_wg, so all partial results together are smaller than n_wg tiles of 256 x 256
         if (m->down_ks_max > 1 && !m->y_slabs)
