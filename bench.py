@@ -27,7 +27,7 @@ PEAK_HBM_GBPS = 8000.0
 
 # HBM traffic per launch of the dominant kernel from the committed rocprofv3 --pmc runs
 # (profiles/experts_bf16_c2_mixtral_pmc.txt): FETCH_SIZE + WRITE_SIZE in bytes, scaled by the copy-kernel factor.
-TRAFFIC_BYTES = {"c2_mixtral": 4.88e9}
+TRAFFIC_BYTES = {"c2_mixtral": 4.98e9}
 
 
 def main():
