@@ -110,6 +110,9 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
         }
     };
 
+    // a wave whose lowest token is past the end of the batch has no sum to form (small batches, ragged last tile):
+    // the sums are bound by LDS reads, which its silence leaves to the waves that have tokens
+    const bool wave_live = t0 + (tid & ~63) / EL < T;
     fetch(0);
     for (int k0 = 0; k0 < d; k0 += KC) {
         const int kend = min(KC, d - k0);
@@ -147,7 +150,9 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
             }                                                                          \
         }                                                                              \
     } while (0)
-        if (FAST_IO || kend == KC) {
+        if (!wave_live) {
+            // every token of this wave lies beyond T: it only stages and keeps the barriers
+        } else if (FAST_IO || kend == KC) {
             // whole chunk: no exit test inside, so the LDS reads of later steps are issued ahead of the sums
 #pragma unroll(NT * EPT >= 8 ? 4 : 16)
             for (int k4 = 0; k4 < KC / 4; ++k4) ROUTER_K4(k4);
