@@ -89,11 +89,15 @@ public:
     virtual void diff() = 0;
     virtual void forward() = 0;
     virtual void back() = 0;
+    virtual void backTemp() = 0;
     virtual void forward(Tensor &input) = 0;
     virtual void back(Tensor &delta) = 0;
     virtual void update() = 0;
     virtual void accGrad(float scale) = 0;
+    virtual void showDiff() = 0;
     virtual const char *getLayerType() const = 0;
+    virtual const float *output(const float *input) = 0;  // the legacy host-array path: float[][][][] output(float[][][][])
+    virtual void initCache() = 0;
     void setInput(Tensor &in) { input = &in; }
 };
 
@@ -237,6 +241,12 @@ public:
         runBack(true);
     }
     void diff() override { runBack(false); }
+    // the hooks LlamaMLPLayer leaves empty (J/engine/nn/layer/llama/LlamaMLPLayer.java:247-271): nothing to show, no
+    // legacy host-array path (it returns null there), no cache, no temporary backward
+    void backTemp() override {}
+    void showDiff() override {}
+    const float *output(const float *) override { return nullptr; }
+    void initCache() override {}
     void runBack(bool block)
     {
         const size_t n = (size_t)number * embedDim_;

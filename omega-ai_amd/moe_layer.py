@@ -221,6 +221,16 @@ class MoELayer:
     def getLayerType(self):
         return "feed_forward"
 
+    # the hooks LlamaMLPLayer leaves empty (J/engine/nn/layer/llama/LlamaMLPLayer.java:247-271)
+    def backTemp(self):
+        pass
+
+    def showDiff(self):
+        pass
+
+    def initCache(self):
+        pass
+
     def set_training(self, on=True):
         """Forward keeps h1 / h3 for back(), as the reference's layers keep their outputs."""
         self.ctx.check(self.lib.omega_moe_set_training(self.handle, int(bool(on))))

@@ -52,11 +52,13 @@ def test_version_and_error_paths_without_a_device(lib):
 def test_host_mirror_keeps_the_layer_contract():
     P = load_pkg()
     for name in ("init", "initBack", "output", "getOutput", "forward", "back", "update", "accGrad", "getLayerType",
-                 "saveModel", "loadModel", "setInput"):
+                 "saveModel", "loadModel", "setInput", "backTemp", "showDiff", "initCache", "updateAdamW", "gradSumSq",
+                 "scaleGrad", "clipGradNorm", "saveModelBlock", "loadModelBlock"):
         assert hasattr(P.MoELayer, name)
     hpp = open(os.path.join(ROOT, "omega-ai_amd", "host", "MoELayer.hpp")).read()
     for name in ("init()", "initBack()", "initParam()", "output()", "getOutput()", "forward(Tensor", "back(Tensor",
-                 "update()", "accGrad(", "getLayerType()", "saveModel(", "loadModel("):
+                 "update()", "accGrad(", "getLayerType()", "saveModel(", "loadModel(", "backTemp()", "showDiff()",
+                 "initCache()", "diff()", "updateAdamW(", "gradSumSq()", "scaleGrad("):
         assert name in hpp
 
 
