@@ -97,6 +97,25 @@ int main(int argc, char **argv)
         FILE *sv = fopen((dir + "/model_saved.bin").c_str(), "wb");
         mlp.saveModel(sv);
         fclose(sv);
+        // one optimiser step on the gradients of the last backward pass, as a Network would drive it: the layer's term
+        // of the global gradient norm, the clip, AdamW at train_time 1; then the block-order checkpoint
+        if (FILE *fd3 = fopen((dir + "/gamma.bin").c_str(), "rb")) {
+            fclose(fd3);
+            if (FILE *fd4 = fopen((dir + "/dout.bin").c_str(), "rb")) {
+                fclose(fd4);
+                const float ss = mlp.gradSumSq();
+                FILE *fs = fopen((dir + "/gradsumsq.bin").c_str(), "wb");
+                fwrite(&ss, 4, 1, fs);
+                fclose(fs);
+                mlp.scaleGrad(0.5f);
+                const float ss2 = mlp.gradSumSq();
+                if (!(ss2 > 0.24f * ss && ss2 < 0.26f * ss)) throw std::runtime_error("scaleGrad(0.5) did not quarter the sum of squares");
+                mlp.updateAdamW(2e-3f, 1, 0.9f, 0.95f, 0.0f);
+                FILE *st = fopen((dir + "/model_step.bin").c_str(), "wb");
+                mlp.saveModelBlock(st);
+                fclose(st);
+            }
+        }
         // error convention: a mismatching input must raise, not crash
         omega::Tensor bad(T, 1, 1, d + 1, &ctx, true);
         bool raised = false;

@@ -47,6 +47,8 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
         dWg = np.fromfile(os.path.join(td, "dWg.bin"), "<f4").reshape(cfg.E, cfg.d)
         dx_block = np.fromfile(os.path.join(td, "dx_block.bin"), "<f4").reshape(cfg.T, cfg.d)
         dgamma = np.fromfile(os.path.join(td, "dgamma.bin"), "<f4")
+        sumsq = float(np.fromfile(os.path.join(td, "gradsumsq.bin"), "<f4")[0])
+        stepped = np.fromfile(os.path.join(td, "model_step.bin"), "<f4")
     ref = O.moe_forward(inp["x"], inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es, bf16=dtype == "bf16")
     assert np.array_equal(ids, ref["ids"])
     assert N.rel_l2(out, ref["out"]) <= (1e-2 if dtype == "bf16" else 1e-5)
@@ -62,3 +64,20 @@ def test_cpp_layer_forward_and_checkpoint(dtype):
     bb = O.block_backward(inp["x"], gamma, dout, inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, cfg.Es,
                           bf16=dtype == "bf16")
     assert N.rel_l2(dx_block, bb["dx"]) <= tol and N.rel_l2(dgamma, bb["dgamma"]) <= tol     # backBlock of the C++ layer
+    # gradSumSq / scaleGrad / updateAdamW / saveModelBlock of the C++ layer, on the gradients of its block backward:
+    # the layer's term of the global norm against the oracle's gradients, and one AdamW step (train_time 1, no decay),
+    # which moves every parameter by lr * g / (|g| + eps): against the sign of its gradient, by at most lr
+    grads = [bb["dgamma"], bb["dWg"]] + [a for g in range(G) for a in (bb["dW1"][g], bb["dW3"][g], bb["dW2"][g])]
+    want_ss = sum(float((a.astype(np.float64) ** 2).sum()) for a in grads)
+    assert abs(sumsq - want_ss) <= 4 * tol * want_ss, (sumsq, want_ss)
+    before = np.concatenate([gamma, model.astype(np.float32)])
+    gflat = np.concatenate([a.ravel() for a in grads])
+    assert stepped.shape == before.shape == gflat.shape
+    move = stepped.astype(np.float64) - before
+    lr = 2e-3
+    assert np.abs(move).max() <= lr * 1.01 + (2.0 ** -8 * np.abs(before).max() if dtype == "bf16" else 0.0)
+    clear = np.abs(gflat) > 1e-3 * np.abs(gflat).max()          # gradients whose sign the tolerance cannot flip
+    assert clear.mean() > 0.3
+    agree = np.sign(move[clear]) == -np.sign(gflat[clear])
+    # (a bf16 weight moves only if the step crosses half a unit in the last place: most do at this step size)
+    assert agree.mean() > (0.9 if dtype == "bf16" else 0.999), agree.mean()
