@@ -21,6 +21,11 @@ Name schemes understood (layer index i, expert e):
               ....mlp.shared_experts.gate_proj|up_proj|down_proj.weight of width Es*H, cut into Es experts
               (the sum of Es SwiGLU experts is one SwiGLU MLP over the concatenated hidden units),
               model.layers.<i>.post_attention_layernorm.weight
+In the "omega" scheme an expert (routed, shared or the dense one) may also come in the fused form of DiTSwiGLUFFN
+(J/engine/nn/layer/dit/org/DiTSwiGLUFFN.java:79,127-141,296-303): "....w12.weight" [2H, d], whose first H rows are
+the branch that goes through SiLU (channel 0 of the [number, 2, 1, H] view, this layer's w1) and whose last H rows
+are the multiplier (channel 1, this layer's w3); the down projection then carries that class's name "....w3.weight"
+and has shape [d, H].
 Qwen-MoE checkpoints use the "deepseek" expert names; their sigmoid-gated shared expert is not part of this layer
 and is refused.
 """
@@ -95,12 +100,22 @@ def load_moe_weights(layer, weight_map, layer_index=0, scheme="omega", strict=Tr
         bg = get(nm["gate_bias"], (E,))
     if Wg is not None:
         layer.set_gate(Wg, bg)
-    dense = nm["dense"] is not None and E == 1 and nm["expert"](0, "w1") not in weight_map
-    for e in range(E):
-        key = (lambda w: nm["dense"](w)) if dense else (lambda w: nm["expert"](e, w))
+    def one_expert(key):
+        """(W1, W3, W2) of the expert whose parameter names key(w) gives, from the separate or the fused form."""
+        if scheme == "omega" and key("w12") in weight_map:
+            F, W2 = get(key("w12"), (2 * H, d)), get(key("w3"), (d, H))
+            if F is None or W2 is None:
+                return None
+            return np.ascontiguousarray(F[:H]), np.ascontiguousarray(F[H:]), W2
         W1, W3, W2 = get(key("w1"), (H, d)), get(key("w3"), (H, d)), get(key("w2"), (d, H))
-        if W1 is not None and W3 is not None and W2 is not None:
-            layer.set_expert(e, W1, W3, W2)
+        return None if W1 is None or W3 is None or W2 is None else (W1, W3, W2)
+
+    dense = (nm["dense"] is not None and E == 1 and nm["expert"](0, "w1") not in weight_map
+             and nm["expert"](0, "w12") not in weight_map)
+    for e in range(E):
+        got = one_expert((lambda w: nm["dense"](w)) if dense else (lambda w, e=e: nm["expert"](e, w)))
+        if got is not None:
+            layer.set_expert(e, *got)
     if Es > 0:
         if nm["fused_shared"] is not None:
             F1, F3 = get(nm["fused_shared"]("w1"), (Es * H, d)), get(nm["fused_shared"]("w3"), (Es * H, d))
@@ -112,10 +127,9 @@ def load_moe_weights(layer, weight_map, layer_index=0, scheme="omega", strict=Tr
                                      np.ascontiguousarray(F2[:, s * H:(s + 1) * H]))
         elif nm["shared"] is not None:
             for s in range(Es):
-                W1, W3 = get(nm["shared"](s, "w1"), (H, d)), get(nm["shared"](s, "w3"), (H, d))
-                W2 = get(nm["shared"](s, "w2"), (d, H))
-                if W1 is not None and W3 is not None and W2 is not None:
-                    layer.set_expert(E + s, W1, W3, W2)
+                got = one_expert(lambda w, s=s: nm["shared"](s, w))
+                if got is not None:
+                    layer.set_expert(E + s, *got)
         else:
             raise RuntimeError(f"Error code 1:scheme {scheme!r} has no names for shared experts")
     required_missing = list(missing)
@@ -128,18 +142,28 @@ def load_moe_weights(layer, weight_map, layer_index=0, scheme="omega", strict=Tr
     return missing
 
 
-def export_moe_weights(arrays, layer_index=0, scheme="omega", gamma=None):
+def export_moe_weights(arrays, layer_index=0, scheme="omega", gamma=None, fused12=False):
     """The inverse, for tests and for exporting a layer: arrays = dict(Wg [E,d], bg [E]|None, W1,W3 [E+Es,H,d],
-    W2 [E+Es,d,H]) -> {name: nested lists}."""
+    W2 [E+Es,d,H]) -> {name: nested lists}.  fused12 ("omega" only): every expert in the DiTSwiGLUFFN form, w12 =
+    [w1; w3] and the down projection under the name w3."""
+    if fused12 and scheme != "omega":
+        raise ValueError("fused12 belongs to the omega scheme")
     nm = _names(scheme, layer_index)
     E = arrays["Wg"].shape[0]
     G = arrays["W1"].shape[0]
     out = {nm["gate"]: arrays["Wg"].tolist()}
     if arrays.get("bg") is not None and nm["gate_bias"] is not None:
         out[nm["gate_bias"]] = arrays["bg"].tolist()
+    def put(key, g):
+        if fused12:
+            out[key("w12")] = np.concatenate([arrays["W1"][g], arrays["W3"][g]], axis=0).tolist()
+            out[key("w3")] = arrays["W2"][g].tolist()
+        else:
+            for w in ("w1", "w3", "w2"):
+                out[key(w)] = arrays["W" + w[1]][g].tolist()
+
     for e in range(E):
-        for w in ("w1", "w3", "w2"):
-            out[nm["expert"](e, w)] = arrays["W" + w[1]][e].tolist()
+        put(lambda w, e=e: nm["expert"](e, w), e)
     if G > E:
         if nm["fused_shared"] is not None:
             out[nm["fused_shared"]("w1")] = np.concatenate(list(arrays["W1"][E:]), axis=0).tolist()
@@ -147,8 +171,7 @@ def export_moe_weights(arrays, layer_index=0, scheme="omega", gamma=None):
             out[nm["fused_shared"]("w2")] = np.concatenate(list(arrays["W2"][E:]), axis=1).tolist()
         else:
             for s in range(G - E):
-                for w in ("w1", "w3", "w2"):
-                    out[nm["shared"](s, w)] = arrays["W" + w[1]][E + s].tolist()
+                put(lambda w, s=s: nm["shared"](s, w), E + s)
     if gamma is not None:
         out[nm["norm"]] = np.asarray(gamma).tolist()
     return out

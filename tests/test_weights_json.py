@@ -101,3 +101,36 @@ def test_errors():
         W.load_moe_weights(FakeLayer(d, H, E, 0), m3, scheme="deepseek")
     with pytest.raises(ValueError):
         W.load_moe_weights(FakeLayer(d, H, E, 0), {}, scheme="nope")
+
+
+def test_fused_w12_form_of_the_dit_ffn():
+    """DiTSwiGLUFFN's parameters: w12 [2H, d] = [SiLU branch; multiplier], down projection named w3 [d, H]; for routed
+    and shared experts and, with E == 1, under the dense names."""
+    d, H, E, Es = 6, 4, 3, 1
+    a = _arrays(d, H, E, Es, False, seed=9)
+    m = W.export_moe_weights(a, layer_index=2, scheme="omega", fused12=True)
+    k12 = "layers.2.feed_forward.experts.1.w12.weight"
+    assert np.asarray(m[k12]).shape == (2 * H, d) and "layers.2.feed_forward.experts.1.w1.weight" not in m
+    assert np.asarray(m["layers.2.feed_forward.experts.1.w3.weight"]).shape == (d, H)
+    lay = FakeLayer(d, H, E, Es)
+    assert W.load_moe_weights(lay, m, layer_index=2, scheme="omega") == ["layers.2.ffn_norm.weight"]
+    for g in range(E + Es):
+        for got, want in zip(lay.experts[g], (a["W1"][g], a["W3"][g], a["W2"][g])):
+            assert got.flags["C_CONTIGUOUS"] and np.array_equal(got, want)
+    # the halves are not interchangeable: the first H rows are the SiLU branch
+    assert np.array_equal(np.asarray(m[k12], np.float32)[:H], a["W1"][1])
+    # a down projection of the wrong shape (the separate form's w3 [H, d]) is refused
+    bad = dict(m)
+    bad["layers.2.feed_forward.experts.0.w3.weight"] = a["W3"][0].tolist()
+    with pytest.raises(RuntimeError, match="Error code"):
+        W.load_moe_weights(FakeLayer(d, H, E, Es), bad, layer_index=2, scheme="omega")
+    # dense names with one expert
+    a1 = _arrays(d, H, 1, 0, False, seed=10)
+    dense = {"layers.0.feed_forward.gate.weight": a1["Wg"].tolist(),
+             "layers.0.feed_forward.w12.weight": np.concatenate([a1["W1"][0], a1["W3"][0]]).tolist(),
+             "layers.0.feed_forward.w3.weight": a1["W2"][0].tolist()}
+    lay1 = FakeLayer(d, H, 1, 0)
+    W.load_moe_weights(lay1, dense, strict=False)
+    assert np.array_equal(lay1.experts[0][0], a1["W1"][0]) and np.array_equal(lay1.experts[0][2], a1["W2"][0])
+    with pytest.raises(ValueError):
+        W.export_moe_weights(a, scheme="mixtral", fused12=True)
