@@ -265,10 +265,15 @@ public:
     void setTraining(bool on) { check(ctx_.get(), omega_moe_set_training(moe_, on ? 1 : 0)); }
     // update() of a layer without an updater: w -= learnRate * diffW (FullyLayer.update, FullyLayer.java:569-590)
     float learnRate = 0.0f;
-    void update() override { check(ctx_.get(), omega_moe_update(moe_, learnRate)); }
+    bool freeze = false;  // Layer.freeze: a frozen layer's update() does nothing (FullyLayer.java:571)
+    void update() override
+    {
+        if (!freeze) check(ctx_.get(), omega_moe_update(moe_, learnRate));
+    }
     // update() under the AdamW updater (AdamW.update, AdamW.java:69-92): trainTime is network.train_time, from 1
     void updateAdamW(float lr, int trainTime, float beta1 = 0.9f, float beta2 = 0.95f, float weightDecay = 1e-4f)
     {
+        if (freeze) return;
         check(ctx_.get(), omega_moe_update_adamw(moe_, lr, beta1, beta2, weightDecay, trainTime));
     }
     void accGrad(float scale) override { check(ctx_.get(), omega_moe_acc_grad(moe_, scale)); }

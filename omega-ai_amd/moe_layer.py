@@ -116,6 +116,7 @@ class MoELayer:
         self.output_buf = None
         self.diff = None
         self.delta = None
+        self.freeze = False
         cfg = L.MoEConfigStruct(T_max, embedDim, nExperts, topK, hidden, nShared, int(renorm), int(bias),
                                 L.DTYPE_BF16 if dtype == "bf16" else L.DTYPE_F32,
                                 L.ROUTER_EXACT if router_mode == "exact" else L.ROUTER_FAST)
@@ -306,12 +307,16 @@ class MoELayer:
         """The update of a layer without an updater: w -= learnRate * diffW (FullyLayer.update,
         J/engine/nn/layer/FullyLayer.java:569-590); bf16 layers step fp32 master copies and re-round.  forward() must run
         again before the next back()."""
+        if self.freeze:      # Layer.freeze: a frozen layer's update() does nothing (FullyLayer.java:571)
+            return
         self.ctx.check(self.lib.omega_moe_update(self.handle, float(learnRate)))
 
     def updateAdamW(self, learnRate, train_time, beta1=0.9, beta2=0.95, weight_decay=1e-4):
         """update() under the AdamW updater (AdamW.update, J/engine/updater/AdamW.java:69-92; adamw_kernel,
         J/engine/updater/gpu/updater.cu:31-52): train_time is network.train_time, starting at 1; the defaults are the
         reference's (AdamWKernel.java:25-26, AdamW.java:27).  forward() must run again before the next back()."""
+        if self.freeze:
+            return
         self.ctx.check(self.lib.omega_moe_update_adamw(self.handle, float(learnRate), float(beta1), float(beta2),
                                                        float(weight_decay), int(train_time)))
 

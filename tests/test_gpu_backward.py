@@ -78,6 +78,12 @@ def test_acc_grad_and_update_fp32():
     layer.back(g1)
     a = {k: layer.grad(w, 1) for k, w in (("W1", L.W_W1), ("W2", L.W_W2))}
     a["Wg"], a["bg"] = layer.grad(L.W_GATE), layer.grad(L.W_GATE_BIAS)
+    layer.freeze = True                     # a frozen layer's update() does nothing (FullyLayer.update)
+    w_frozen = layer._download_weight(L.W_W1, 1, (cfg.H, cfg.d))
+    layer.update(0.25)
+    layer.updateAdamW(0.25, 1)
+    assert np.array_equal(layer._download_weight(L.W_W1, 1, (cfg.H, cfg.d)), w_frozen)
+    layer.freeze = False
     layer.accGrad(1.0)                      # first call: copy
     layer.back(g2)
     layer.accGrad(2.0)                      # then acc += 2 * grad(0.5 dout) = 2 * grad(dout) in total
