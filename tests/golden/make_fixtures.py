@@ -6,7 +6,8 @@ cover its building blocks with expected outputs), so the fixtures freeze what th
   * the fp32 parity configuration (256 tokens, d=128, 8 experts, top-2, H=256) under a fixed seed, and
   * small adversarial cases: ties (all-equal gate rows, duplicated gate rows), empty experts, K == E,
     shared experts without renormalisation.
-The backward pass of four of the cases is frozen the same way (bw_*.npz, see BW_CASES).
+The backward pass of four of the cases is frozen the same way (bw_*.npz, see BW_CASES), and so are five steps of the
+AdamW update (adamw_steps.npz).
 Inputs are regenerated from the seed by the counter-based generator, so only expected outputs are stored:
 routing arrays in full, the layer output as float64 checksums plus a few rows.
 Run from the repository root:  python tests/golden/make_fixtures.py
@@ -84,7 +85,37 @@ def expected_backward(spec):
     return out
 
 
+# AdamW (the updater oracle, pinned against torch.optim.AdamW in float64 and closed forms): 512 parameters, five steps
+# with gradients whose magnitudes span six decades (and exact zeros); stored are the parameters and both moments after
+# every step, bit for bit.  File adamw_steps.npz.
+ADAMW = dict(n=512, steps=5, lr=3e-3, beta1=0.9, beta2=0.95, wd=1e-2, seed=77)
+
+
+def adamw_inputs():
+    n, seed = ADAMW["n"], ADAMW["seed"]
+    w0 = O.fill_normal(n, seed, 1, 0.5)
+    grads = []
+    for t in range(ADAMW["steps"]):
+        g = O.fill_normal(n, seed, 10 + t, 1.0) * (np.float32(10.0) ** np.floor(O.fill_normal(n, seed, 20 + t, 2.0)).clip(-4, 1))
+        g = g.astype(np.float32)
+        g[::17] = 0.0
+        grads.append(g)
+    return w0, grads
+
+
+def expected_adamw():
+    w, grads = adamw_inputs()
+    m, v = np.zeros_like(w), np.zeros_like(w)
+    out = {}
+    for t, g in enumerate(grads, 1):
+        w, m, v = O.adamw(w, g, m, v, ADAMW["lr"], ADAMW["beta1"], ADAMW["beta2"], ADAMW["wd"], t)
+        out[f"w{t}"], out[f"m{t}"], out[f"v{t}"] = w.copy(), m.copy(), v.copy()
+    return out
+
+
 def main():
+    np.savez_compressed(os.path.join(HERE, "adamw_steps.npz"), **expected_adamw())
+    print("wrote adamw_steps")
     for name, spec in CASES.items():
         np.savez_compressed(os.path.join(HERE, name + ".npz"), **expected(spec))
         print("wrote", name)

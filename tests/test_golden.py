@@ -87,3 +87,16 @@ def test_hip_path_reproduces_backward_fixture(name):
     e = int(np.argmax(want["dW_norms"][2]))
     assert N.rel_l2(layer.grad(L.W_W2, e)[0], want["dW2_first_row"]) <= tol
     layer.close()
+
+
+
+def test_oracle_reproduces_adamw_fixture():
+    want, got = load("adamw_steps"), MF.expected_adamw()
+    assert sorted(want) == sorted(got) and len(want) == 3 * MF.ADAMW["steps"]
+    for k in want:
+        assert np.array_equal(want[k].view(np.uint32), got[k].view(np.uint32)), k
+    # the frozen run did something: every parameter with a non-zero first gradient moved by about lr at step 1
+    w0, grads = MF.adamw_inputs()
+    moved = np.abs(want["w1"].astype(np.float64) - w0)
+    nz = grads[0] != 0
+    assert nz.sum() > 400 and np.all(moved[nz] > 0.5 * MF.ADAMW["lr"]) and np.all(moved[~nz] < 0.1 * MF.ADAMW["lr"])
