@@ -203,6 +203,9 @@ static int moe_reserve_backward(omega_moe *m, int T)
         m->dgamma = m->dbg + ((c.E + 3) & ~3);
         m->dW13 = m->dgamma + ((c.d + 3) & ~3);
         m->dW2 = m->dW13 + 2 * (size_t)m->G * HD;
+        OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->bw_zero_state, (size_t)2 * m->G * 4));
+        OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->bw_zero_state, 0, (size_t)2 * m->G * 4, ctx->stream));
+        m->bw_zero_valid = false;
     }
     if (bf && !m->W2T) {
         // one row group of slack behind W2T: the last 256-column tile of a width H = 128 mod 256 reads it (and drops it)
@@ -418,6 +421,7 @@ int omega_moe_destroy(omega_moe *m)
     if (m->dWg) hipFree(m->dWg);
     if (m->acc_grad) hipFree(m->acc_grad);
     if (m->sumsq_part) hipFree(m->sumsq_part);
+    if (m->bw_zero_state) hipFree(m->bw_zero_state);
     if (m->y_slabs) hipFree(m->y_slabs);
     if (m->adam_m) hipFree(m->adam_m);
     if (m->adam_v) hipFree(m->adam_v);
@@ -680,6 +684,10 @@ static int backward_impl(omega_moe *m, const void *x, const void *dout, int T, v
     const void *xin = block ? m->hbuf : x;
     void *dxl = block ? m->bw_dhx : dx;
     OMEGA_HIP_CHECK(ctx, bf ? launch_backward_bf16(m, xin, dout, T, dxl, ctx->stream) : launch_backward_f32(m, xin, dout, T, dxl, ctx->stream));
+    if (bf) {  // the pass wrote the states of the weight-gradient blocks into the other copy
+        m->bw_zero_phase ^= 1;
+        m->bw_zero_valid = true;
+    }
     if (block) OMEGA_HIP_CHECK(ctx, launch_rmsnorm_backward(m, x, m->bw_dhx, dout, T, dx, ctx->stream));
     else OMEGA_HIP_CHECK(ctx, launch_zero_f32(m->dgamma, (size_t)m->cfg.d, ctx->stream));  // the norm took no part
     return OMEGA_OK;
@@ -708,6 +716,10 @@ int omega_moe_time_backward(omega_moe *m, const void *x, const void *dout, int T
     for (int i = 0; i < warmup + iters; ++i) {
         if (i == warmup) OMEGA_HIP_CHECK(ctx, hipEventRecord(m->ev0, ctx->stream));
         OMEGA_HIP_CHECK(ctx, bf ? launch_backward_bf16(m, x, dout, T, dx, ctx->stream) : launch_backward_f32(m, x, dout, T, dx, ctx->stream));
+        if (bf) {
+            m->bw_zero_phase ^= 1;
+            m->bw_zero_valid = true;
+        }
     }
     OMEGA_HIP_CHECK(ctx, hipEventRecord(m->ev1, ctx->stream));
     OMEGA_HIP_CHECK(ctx, hipEventSynchronize(m->ev1));
@@ -793,6 +805,7 @@ int omega_moe_update(omega_moe *m, float lr)
     if (m->acc_valid) {
         OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(m->dWg, m->acc_grad, grad_block_floats(m) * 4, hipMemcpyDeviceToDevice, ctx->stream));
         m->acc_valid = false;
+        m->bw_zero_valid = false;  // the gradient block now holds the accumulators
     }
     if (c.dtype == OMEGA_DTYPE_BF16) {
         // the step is taken on fp32 master copies (made from the weights at the first update after they were set); the
@@ -833,6 +846,7 @@ int omega_moe_update_adamw(omega_moe *m, float lr, float beta1, float beta2, flo
     if (m->acc_valid) {
         OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(m->dWg, m->acc_grad, n * 4, hipMemcpyDeviceToDevice, ctx->stream));
         m->acc_valid = false;
+        m->bw_zero_valid = false;  // the gradient block now holds the accumulators
     }
     if (!m->adam_m) {
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->adam_m, n * 4));

@@ -680,11 +680,20 @@ __global__ __launch_bounds__(256) void bw_combine_bf16_kernel(const uint4 *__res
 }
 
 // The weight gradients of a group without rows are zero; the product kernels have no items for it.
+// A block that this kernel zeroed and nothing has written since (the group stayed without rows) is left alone:
+// st_in[g] == 1 says so; every workgroup writes the group's new state to st_out (a second array, so that no workgroup
+// of this launch reads what another one wrote).  force: the states are not to be trusted (the gradients were
+// overwritten from the accumulators).
 __global__ __launch_bounds__(256) void bw_zero_empty_kernel(const int32_t *__restrict__ counts, int E, int T,
-                                                            float *__restrict__ dW13, float *__restrict__ dW2, size_t HD)
+                                                            float *__restrict__ dW13, float *__restrict__ dW2, size_t HD,
+                                                            const int32_t *__restrict__ st_in, int32_t *__restrict__ st_out,
+                                                            int force)
 {
     const int g = blockIdx.x;
-    if ((g < E ? counts[g] : T) > 0) return;
+    const bool has_rows = (g < E ? counts[g] : T) > 0;
+    const bool known_zero = !has_rows && !force && st_in[g] == 1;
+    if (blockIdx.y == 0 && threadIdx.x == 0) st_out[g] = has_rows ? 0 : 1;
+    if (has_rows || known_zero) return;
     float4 *p13 = (float4 *)(dW13 + (size_t)g * 2 * HD), *p2 = (float4 *)(dW2 + (size_t)g * HD);
     const float4 z = {0.0f, 0.0f, 0.0f, 0.0f};
     for (size_t i = (size_t)blockIdx.y * 256 + threadIdx.x; i < HD / 4; i += (size_t)gridDim.y * 256) {
@@ -723,7 +732,9 @@ hipError_t launch_backward_bf16(const omega_moe *m, const void *x, const void *d
                              m->bw_ksteps_cap * 32, s));
     STEP(launch_product_bf16(m, MODE_WGRAD, m->bw_dhT, nullptr, m->bw_xgT, nullptr, m->dW13, nullptr, nullptr, m->wq_w13, c.d,
                              m->bw_ksteps_cap * 32, s));
-    hipLaunchKernelGGL(bw_zero_empty_kernel, dim3(G, 128), dim3(256), 0, s, m->counts, c.E, T, m->dW13, m->dW2, HD);
+    hipLaunchKernelGGL(bw_zero_empty_kernel, dim3(G, 128), dim3(256), 0, s, m->counts, c.E, T, m->dW13, m->dW2, HD,
+                       (const int32_t *)(m->bw_zero_state + (m->bw_zero_phase ? G : 0)), m->bw_zero_state + (m->bw_zero_phase ? 0 : G),
+                       m->bw_zero_valid ? 0 : 1);
     // router and gate
     hipLaunchKernelGGL(bw_router_kernel, dim3(ceil_div(T, 256)), dim3(256), 0, s, (const float *)m->bw_probs, m->ids, m->w,
                        (const float *)m->bw_dw, T, c.E, c.K, c.renorm, m->bw_dlogits);

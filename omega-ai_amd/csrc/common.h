@@ -101,6 +101,9 @@ struct omega_moe {
     float *dWg = nullptr, *dbg = nullptr, *dgamma = nullptr, *dW13 = nullptr, *dW2 = nullptr;
     float *acc_grad = nullptr;       // accumulators, one block in the order dWg, dbg, dgamma, dW13, dW2
     bool acc_valid = false;          // accGrad has run since the last update
+    int32_t *bw_zero_state = nullptr;  // [2][G]: which groups' weight-gradient blocks are known to be zero (two copies, used in turn)
+    int bw_zero_phase = 0;           // which copy the next backward pass reads
+    bool bw_zero_valid = false;      // false: the gradient block was written from outside the backward pass
     double *sumsq_part = nullptr;    // scratch of the gradient-norm reduction
     float *adam_m = nullptr;         // AdamW moments, each laid out like the gradient block (allocated by the first AdamW update)
     float *adam_v = nullptr;

@@ -402,3 +402,43 @@ def test_grad_norm_and_clipping(name, kw, block):
     assert abs(layer.gradSumSq() - coef * coef * want) <= 1e-5 * want
     assert all(np.array_equal(a, b) for a, b in zip(after, _all_grads(layer, cfg, block)))   # the plain gradients were not touched
     layer.close()
+
+
+def test_empty_expert_gradients_stay_zero_across_passes_bf16():
+    """An expert without rows has zero weight gradients.  The backward pass zeroes such a block once and then leaves
+    it alone for as long as the expert stays empty; whatever writes the block in between - the expert getting rows
+    again, update() bringing the accumulators in - must make the next pass zero it again."""
+    G, cfg, inp, dout, layer = _setup("c2_mixtral", dict(T=96, d=256, H=256, E=4, K=2, zipf_bias=1.2), 41)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = G.P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    shut = inp["bg"].copy()
+    shut[3] = -1e4                       # expert 3 never wins
+    open_ = inp["bg"].copy()
+    open_[:] = 0.0
+
+    def run(bias):
+        layer.set_gate(inp["Wg"], bias)
+        layer.forward(x)
+        layer.back(g)
+        return int(layer.routing()["counts"][3]), layer.grad(L.W_W1, 3), layer.grad(L.W_W2, 3)
+
+    n, g1, g2 = run(shut)
+    assert n == 0 and not g1.any() and not g2.any()
+    n, g1, g2 = run(shut)                # still empty: the block is left alone, and is still zero
+    assert n == 0 and not g1.any() and not g2.any()
+    n, g1, g2 = run(open_)               # rows again: real gradients
+    assert n > 0 and g1.any() and g2.any()
+    n, g1, g2 = run(shut)                # empty again: zero again
+    assert n == 0 and not g1.any() and not g2.any()
+    # accumulators: a pass with rows, then an empty one; update() copies the accumulated (non-zero) gradients into the
+    # gradient block, so the next empty pass has to zero it afresh
+    run(open_)
+    layer.accGrad(1.0)
+    n, g1, _ = run(shut)
+    assert n == 0 and not g1.any()
+    layer.accGrad(1.0)
+    layer.update(1e-3)
+    assert layer.grad(L.W_W1, 3).any()   # the block now holds the accumulated gradient of the pass with rows
+    n, g1, g2 = run(shut)
+    assert n == 0 and not g1.any() and not g2.any()
+    layer.close()
