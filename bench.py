@@ -111,10 +111,15 @@ def main():
     probe = None
     if cfg.dtype == "bf16" and not a.no_mfma_probe:
         import ctypes
+        probe_lib = ctypes.CDLL(os.path.join(ROOT, "bench_probe.so"))   # built by __graft_entry__.build()
+        probe_lib.bench_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+        ctx.sync()
         v = ctypes.c_float()
         probe = {}
         for key, rnd in (("constant_operands_TFLOP/s", 0), ("random_operands_TFLOP/s", 1)):
-            ctx.check(ctx.lib.omega_hip_mfma_probe(ctx.handle, rnd, 400, ctypes.byref(v)))
+            st = probe_lib.bench_probe_mfma(0, rnd, 400, ctypes.byref(v))
+            if st != 0:
+                raise RuntimeError(f"bench_probe_mfma: HIP error {st}")
             probe[key] = v.value
         probe["frac_of_random_operand_rate"] = up_tflops / probe["random_operands_TFLOP/s"]
 

@@ -3,7 +3,8 @@
 // sustains under its power cap when the matrix cores do nothing but multiply realistic data; with constant operands
 // (little switching activity) it reaches the nominal clock.  Used by the benchmark to put the product kernels'
 // MFMA throughput next to what the hardware can hold, not to compute anything.
-#include "common.h"
+// Built into bench_probe.so, which only bench.py loads: the layer library does not contain it.
+#include <hip/hip_runtime.h>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float probe_f32x16_t;
@@ -39,12 +40,40 @@ __global__ __launch_bounds__(512) void mfma_probe_kernel(float *out, int iters, 
     if (s == 12345.678f) out[0] = s;  // keeps the loop alive
 }
 
-// launches the probe `launches` times (about 2.5 ms each at full rate) and returns the FLOP count of one launch
-hipError_t launch_mfma_probe(float *scratch, int num_cus, int random_operands, int launches, hipStream_t s, double *flop_per_launch)
+// Bf16 matrix-core rate in TFLOP/s that `device` sustains over `launches` launches of about 2.5 ms (the first quarter
+// untimed).  random_operands != 0: random bf16 values (the rate under the power cap); 0: constants (the nominal clock).
+// Returns 0, or the HIP error code.
+extern "C" int bench_probe_mfma(int device, int random_operands, int launches, float *tflops)
 {
-    const int iters = 20000;
-    for (int i = 0; i < launches; ++i)
+    if (!tflops || launches < 4) return (int)hipErrorInvalidValue;
+    hipDeviceProp_t prop;
+    hipError_t e = hipSetDevice(device);
+    if (e == hipSuccess) e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return (int)e;
+    const int num_cus = prop.multiProcessorCount, iters = 20000, warm = launches / 4;
+    float *scratch = nullptr;
+    hipStream_t s = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    e = hipMalloc((void **)&scratch, 4);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    for (int i = 0; e == hipSuccess && i < launches; ++i) {
+        if (i == warm) e = hipEventRecord(e0, s);
         hipLaunchKernelGGL(mfma_probe_kernel, dim3(num_cus), dim3(512), 0, s, scratch, iters, random_operands);
-    *flop_per_launch = (double)iters * PROBE_ACC * 8.0 * num_cus * 32768.0;  // 8 waves per workgroup, 2 x 32 x 32 x 16 per MFMA
-    return hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipGetLastError();
+    if (e == hipSuccess) e = hipEventRecord(e1, s);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e0) hipEventDestroy(e0);
+    if (e1) hipEventDestroy(e1);
+    if (s) hipStreamDestroy(s);
+    if (scratch) hipFree(scratch);
+    if (e != hipSuccess) return (int)e;
+    // 8 waves per workgroup, 2 x 32 x 32 x 16 FLOP per MFMA
+    const double flop = (double)iters * PROBE_ACC * 8.0 * num_cus * 32768.0;
+    *tflops = (float)(flop * (launches - warm) / (ms * 1e-3) / 1e12);
+    return 0;
 }

@@ -236,6 +236,10 @@ int omega_moe_get_router_probs(omega_moe *moe, const void *x_dev, int T, float *
  * dtype), 2 y [T*K+Es*T,d] fp32; after omega_moe_backward of a bf16 layer also 3 dh1|dh3 [T*K+Es*T,2H] bf16, and for
  * any layer 4 dlogits [T,E] fp32.  For tests. */
 int omega_moe_get_workspace(omega_moe *moe, int which, int T, void *host_dst);
+/* Fills a whole workspace buffer, padding rows included, with one byte value (which = 1 a, 2 y; Tensor.clearGPU /
+ * Tensor.fill on a layer-owned tensor, J/engine/tensor/Tensor.java:680-685).  For tests: with 0xFF every element reads
+ * as NaN, so a row that a forward pass should have written and did not cannot go unnoticed. */
+int omega_moe_fill_workspace(omega_moe *moe, int which, int byte_value);
 
 /* Average duration in milliseconds of the launches of one stage, measured with events on the
  * context's stream: runs `iters` back-to-back repetitions of the stage (0 router, 1 dispatch,
@@ -249,12 +253,6 @@ int omega_moe_time_stage(omega_moe *moe, int stage, const void *x_dev, int T, vo
  * x_dev and T must have run. */
 int omega_moe_time_backward(omega_moe *moe, const void *x_dev, const void *dout_dev, int T, void *dx_dev, int warmup,
                             int iters, float *ms_avg);
-
-/* Measurement aid, no counterpart in the reference: the bf16 matrix-core rate the device sustains with no memory
- * traffic at all (a loop of independent MFMAs on every SIMD, `launches` launches of about 2.5 ms, the first
- * quarter untimed), in TFLOP/s.  random_operands != 0 feeds random bf16 values (realistic switching activity: the
- * rate under the power cap), 0 feeds constants (the rate at the nominal clock). */
-int omega_hip_mfma_probe(omega_ctx *ctx, int random_operands, int launches, float *tflops);
 
 /* Per-stage timing of omega_moe_forward itself: while profiling is on, every forward records events
  * on the context's stream around its five stages (router, dispatch, experts_up, experts_down,

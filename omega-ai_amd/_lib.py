@@ -40,7 +40,6 @@ SIGNATURES = {
     "omega_moe_destroy": (C.c_int, [C.c_void_p]),
     "omega_moe_set_weights": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
     "omega_moe_get_weights": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
-    "omega_hip_mfma_probe": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_float)]),
     "omega_moe_forward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "omega_moe_forward_block": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "omega_moe_get_norm": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
@@ -69,6 +68,7 @@ SIGNATURES = {
     "omega_moe_get_routing": (C.c_int, [C.c_void_p, C.c_int] + [C.c_void_p] * 6),
     "omega_moe_get_router_probs": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "omega_moe_get_workspace": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "omega_moe_fill_workspace": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "omega_moe_time_stage": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int,
                                        C.POINTER(C.c_float)]),
     "omega_moe_set_profiling": (C.c_int, [C.c_void_p, C.c_int]),

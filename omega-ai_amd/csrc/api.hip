@@ -178,6 +178,7 @@ static void moe_free_workspace(omega_moe *m)
     m->T_cap = 0;
     moe_free_backward_workspace(m);
     m->fwd_T = -1;
+    m->routed_T = m->dispatched_T = -1;
 }
 
 static size_t grad_block_floats(const omega_moe *m)
@@ -470,6 +471,11 @@ int omega_moe_set_weights(omega_moe *m, int which, int expert, const void *src, 
     if (!src || weight_slot(m, which, expert, &p, &bytes) != OMEGA_OK)
         OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "set_weights: bad kind, expert index or source");
     m->master_valid = false;  // fp32 master copies of a bf16 layer are remade from the weights at the next update
+    // the activations (and, in training mode, the h1 / h3 records) of the last forward belong to the old weights: a
+    // backward pass needs a new forward first
+    m->fwd_T = -1;
+    m->fwd_block = false;
+    m->rec_valid = false;
     if (!weight_is_packed(m, which)) {
         OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(p, src, bytes, is_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, ctx->stream));
         OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
@@ -538,11 +544,15 @@ static int stage_router(omega_moe *m, const void *x, int T)
 {
     // training mode (bf16 layers, backward workspace in place): the probabilities are kept for the backward pass
     float *probs = (m->training && m->cfg.dtype == OMEGA_DTYPE_BF16 && m->bw_T_cap >= T) ? m->bw_probs : nullptr;
+    m->routed_T = m->dispatched_T = -1;
     OMEGA_HIP_CHECK(m->ctx, launch_router(m, x, T, nullptr, probs, m->ctx->stream));
+    m->routed_T = T;
     return OMEGA_OK;
 }
 static int stage_dispatch(omega_moe *m, const void *x, int T)
 {
+    if (m->routed_T != T) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: the router has not run for this T");
+    m->dispatched_T = -1;
     const int bm = moe_tile_m(m, T);
     m->bm = bm;
     m->max_m_tiles = moe_max_m_tiles(m, T, bm);
@@ -565,18 +575,21 @@ static int stage_dispatch(omega_moe *m, const void *x, int T)
     if (m->max_m_tiles > m->tiles_cap) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: workspace too small for this T");
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));
+    m->dispatched_T = T;
     return OMEGA_OK;
 }
 // x: the rows the shared experts read in fp32 layers (bf16 layers read the packed copy the gather left in xs)
 static int stage_experts(omega_moe *m, const void *x, int T, int which)
 {
-    if (m->bm != moe_tile_m(m, T)) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "experts: dispatch has not run for this T");
+    if (m->dispatched_T != T || m->bm != moe_tile_m(m, T))
+        OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "experts: dispatch has not run for this T");
     if (m->cfg.dtype == OMEGA_DTYPE_BF16) OMEGA_HIP_CHECK(m->ctx, launch_experts_bf16(m, x, T, which, m->ctx->stream));
     else OMEGA_HIP_CHECK(m->ctx, launch_experts_f32(m, x, T, which, m->ctx->stream));
     return OMEGA_OK;
 }
 static int stage_combine(omega_moe *m, int T, void *out, const void *resid)
 {
+    if (m->dispatched_T != T) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "combine: dispatch has not run for this T");
     OMEGA_HIP_CHECK(m->ctx, launch_combine(m, T, out, resid, m->ctx->stream));
     return OMEGA_OK;
 }
@@ -985,6 +998,7 @@ int omega_moe_get_routing(omega_moe *m, int T, int32_t *ids, float *w, int32_t *
 int omega_moe_get_router_probs(omega_moe *m, const void *x, int T, float *logits, float *probs)
 {
     MOE_ENTER(m);
+    stage_invalidates(m);
     RUN(check_T(m, x, T, true));
     if (T == 0) return OMEGA_OK;
     RUN(moe_reserve(m, T));
@@ -992,7 +1006,9 @@ int omega_moe_get_router_probs(omega_moe *m, const void *x, int T, float *logits
     float *dl = nullptr, *dp = nullptr;
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&dl, n * 4));
     hipError_t e = hipMalloc((void **)&dp, n * 4);
+    m->routed_T = m->dispatched_T = -1;
     if (e == hipSuccess) e = launch_router(m, x, T, dl, dp, ctx->stream);
+    if (e == hipSuccess) m->routed_T = T;
     if (e == hipSuccess && logits) e = hipMemcpyAsync(logits, dl, n * 4, hipMemcpyDeviceToHost, ctx->stream);
     if (e == hipSuccess && probs) e = hipMemcpyAsync(probs, dp, n * 4, hipMemcpyDeviceToHost, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -1049,29 +1065,14 @@ int omega_moe_get_workspace(omega_moe *m, int which, int T, void *host_dst)
     return OMEGA_OK;
 }
 
-int omega_hip_mfma_probe(omega_ctx *ctx, int random_operands, int launches, float *tflops)
+int omega_moe_fill_workspace(omega_moe *m, int which, int byte_value)
 {
-    CTX_ENTER(ctx);
-    if (!tflops || launches < 4) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "mfma_probe: bad argument");
-    float *scratch = nullptr;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&scratch, 4));
-    hipError_t e = hipEventCreate(&e0);
-    if (e == hipSuccess) e = hipEventCreate(&e1);
-    double flop = 0.0;
-    const int warm = launches / 4;
-    if (e == hipSuccess) e = launch_mfma_probe(scratch, ctx->num_cus, random_operands, warm, ctx->stream, &flop);
-    if (e == hipSuccess) e = hipEventRecord(e0, ctx->stream);
-    if (e == hipSuccess) e = launch_mfma_probe(scratch, ctx->num_cus, random_operands, launches - warm, ctx->stream, &flop);
-    if (e == hipSuccess) e = hipEventRecord(e1, ctx->stream);
-    if (e == hipSuccess) e = hipEventSynchronize(e1);
-    float ms = 0.0f;
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    if (e0) hipEventDestroy(e0);
-    if (e1) hipEventDestroy(e1);
-    hipFree(scratch);
-    OMEGA_HIP_CHECK(ctx, e);
-    *tflops = (float)(flop * (launches - warm) / (ms * 1e-3) / 1e12);
+    MOE_ENTER(m);
+    if ((which != 1 && which != 2) || m->rows_cap == 0)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "fill_workspace: selector must be 1 (a) or 2 (y) and the workspace must exist");
+    void *p = which == 1 ? m->a : (void *)m->y;
+    const size_t bytes = which == 1 ? m->rows_cap * m->cfg.H * m->esize : m->rows_cap * m->cfg.d * 4;
+    OMEGA_HIP_CHECK(ctx, hipMemsetAsync(p, byte_value, bytes, ctx->stream));
     return OMEGA_OK;
 }
 
@@ -1094,10 +1095,11 @@ int omega_moe_time_stage(omega_moe *m, int stage, const void *x, int T, void *ou
             case 3: return stage_experts(m, x, T, 1);
             case 4: return stage_combine(m, T, out, nullptr);
             case 6:
-                OMEGA_HIP_CHECK(ctx, launch_dispatch_index(m, T, m->bm, ctx->stream));
-                return OMEGA_OK;
             case 7:
-                OMEGA_HIP_CHECK(ctx, launch_dispatch_gather(m, x, T, ctx->stream));
+                // parts of a dispatch that has already run for this T (same buffers, same result)
+                if (m->dispatched_T != T) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_stage: dispatch has not run for this T");
+                if (stage == 6) OMEGA_HIP_CHECK(ctx, launch_dispatch_index(m, T, m->bm, ctx->stream));
+                else OMEGA_HIP_CHECK(ctx, launch_dispatch_gather(m, x, T, ctx->stream));
                 return OMEGA_OK;
             case 8: return forward_impl(m, x, T, out, 1);
             case 9:

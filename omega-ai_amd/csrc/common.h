@@ -133,6 +133,11 @@ struct omega_moe {
     int bw_T_cap = 0;
     size_t bw_rows_cap = 0;
     int fwd_T = -1;                  // tokens of the last forward (what a backward pass may follow), -1: none
+    // which batch the index buffers describe: ids / w / tile_counts hold the router's result for routed_T tokens, and
+    // dst / dstp / src_row, the tile list and the work queues the dispatch stage's for dispatched_T (-1: none yet, or
+    // the buffers were reallocated).  A stage is refused unless the stage before it ran for the same T, because the
+    // index buffers are what the next stage's addresses are formed from.
+    int routed_T = -1, dispatched_T = -1;
     bool fwd_block = false;          // ... and whether it was the block form
     void *bw_dhx = nullptr;          // [T,d] layer dtype: input gradient of the layer inside the block form
     bool training = false;           // forward keeps h1 / h3 (bf16 layers: as block records in bw_h1 / bw_h3)
@@ -196,8 +201,6 @@ struct omega_adamw {
     float lr, beta1, beta2, b1c, b2c, eps, wd;  // b1c, b2c: 1 - beta^t, formed on the host
 };
 hipError_t launch_update_adamw(const omega_moe *m, float *master, float *mw, float *vw, const omega_adamw &p, hipStream_t s);
-hipError_t launch_mfma_probe(float *scratch, int num_cus, int random_operands, int launches, hipStream_t s,
-                             double *flop_per_launch);
 hipError_t launch_pack_rows(void *dst_packed, const void *src_rowmajor, int R, int Kd, hipStream_t s);
 hipError_t launch_unpack_rows(void *dst_rowmajor, const void *src_packed, int R, int Kd, hipStream_t s);
 int experts_bf16_tile_m(const omega_moe *m, int T);

@@ -379,6 +379,10 @@ class MoELayer:
         self.ctx.check(self.lib.omega_moe_get_workspace(self.handle, idx, T, h.ctypes.data))
         return bf16_bits_to_f32(h) if raw_bf16 else h
 
+    def fill_workspace(self, which, byte_value):
+        """Every byte of the 'a' or 'y' buffer (padding rows included) set to byte_value; 0xFF reads as NaN."""
+        self.ctx.check(self.lib.omega_moe_fill_workspace(self.handle, {"a": 1, "y": 2}[which], int(byte_value)))
+
     # ---- checkpoint: raw LE float32, order gate, (gate bias), then w1,w3,w2 per expert, routed then shared
     def _download_weight(self, which, expert, shape):
         raw_bf16 = self.dtype == "bf16" and which not in (L.W_GATE_BIAS, L.W_NORM)   # those two are fp32 in every layer

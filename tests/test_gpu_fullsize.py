@@ -1,10 +1,14 @@
 """The four bf16 configurations at their full sizes, inputs generated on the device from the seed.
 
 Routing (ids, weights, counts, offsets, permutation) is compared bit for bit with the oracle's router and
-with a stable argsort over ALL tokens; the layer output is compared with the oracle on a sample of tokens
-(1e-2 relative L2, bf16 with fp32 accumulation), and size-independent properties are checked on the whole
-batch: counts sum to T*K, the permutation is a stable bijection, the gathered buffer holds exactly the
-routed rows, every output row is finite."""
+with a stable argsort over ALL tokens.  The grouped products are checked on every work item: the a and y buffers
+are poisoned with NaN before the forward (an unwritten valid row cannot pass), and the first and last row of every
+32-row block of every expert is compared, in two columns of every 128-column group, with float64 dot products of
+the layer's own operands.  The layer output is compared with the oracle (1e-2 relative L2, bf16 with fp32
+accumulation) on a token sample that touches every row tile, and on ALL tokens with the fp32 layer of this library
+holding the same weights (a different product kernel, pinned to the oracle at 1e-5).  Size-independent properties on
+the whole batch: counts sum to T*K, the permutation is a stable bijection, the gathered buffer holds exactly the
+routed rows, a second forward is bit-identical."""
 import numpy as np
 import pytest
 
@@ -27,6 +31,9 @@ def test_full_size_configuration(name):
     layer.init_synthetic(SEED, C, cfg)
     x = P.DeviceBuffer(G.ctx(), (cfg.T, cfg.d), cfg.dtype)
     x.fill_normal(SEED, C.STREAM_X, C.tensor_std(cfg, "x"))
+    layer.forward(x)                       # sizes the index state; its results are thrown away by the poison
+    layer.fill_workspace("a", 0xFF)
+    layer.fill_workspace("y", 0xFF)
     out = layer.forward(x).to_numpy()
     r = layer.routing()
 
@@ -47,20 +54,27 @@ def test_full_size_configuration(name):
     # ---- gathered buffer == routed rows (sampled rows: the full buffer is up to 0.5 GB)
     if cfg.P * cfg.d <= 40_000_000:
         assert np.array_equal(layer.workspace("xg", cfg.T), xh[src])
-    # ---- output on sampled tokens against the oracle
-    tok = np.unique(np.linspace(0, cfg.T - 1, 6).astype(np.int32))
-    need = sorted(set(r["ids"][tok].ravel().tolist()) | set(range(cfg.E, cfg.E + cfg.Es)))
-    remap = {g: i for i, g in enumerate(need)}
-    W1 = np.stack([layer._download_weight(L.W_W1, g, (cfg.H, cfg.d)) for g in need])
-    W3 = np.stack([layer._download_weight(L.W_W3, g, (cfg.H, cfg.d)) for g in need])
-    W2 = np.stack([layer._download_weight(L.W_W2, g, (cfg.d, cfg.H)) for g in need])
-    n_routed = len([g for g in need if g < cfg.E])
-    ids_c = np.vectorize(remap.get)(r["ids"][tok]).astype(np.int32)
-    ref = O.moe_tokens(np.ascontiguousarray(xh[tok]), ids_c, np.ascontiguousarray(r["w"][tok]), W1, W3, W2, n_routed,
-                       cfg.Es, np.arange(len(tok), dtype=np.int32), bf16=True)
-    err = N.rel_l2(out[tok], ref)
-    assert err <= 1e-2, err
+    # ---- every work item of the two products: NaN poison + float64 spot checks on every 32-row block
+    assert G.check_products_every_block(layer, cfg, cfg.T, r, xh) > 0
+    # ---- output against the oracle on a token sample that touches every row tile
+    tok = np.union1d(G.row_tile_tokens(r, cfg, cfg.T), np.linspace(0, cfg.T - 1, 6).astype(np.int32)).astype(np.int32)
+    Gn = cfg.E + cfg.Es
+    W1 = np.stack([layer._download_weight(L.W_W1, g, (cfg.H, cfg.d)) for g in range(Gn)])
+    W3 = np.stack([layer._download_weight(L.W_W3, g, (cfg.H, cfg.d)) for g in range(Gn)])
+    W2 = np.stack([layer._download_weight(L.W_W2, g, (cfg.d, cfg.H)) for g in range(Gn)])
+    ref = G.oracle_tokens_parallel(
+        lambda part: O.moe_tokens(xh, r["ids"], r["w"], W1, W3, W2, cfg.E, cfg.Es, part, bf16=True), tok)
+    del W1, W3, W2
+    G.assert_rows_close(out[tok], ref, 1e-2, 2e-2, "oracle sample")
     assert np.isfinite(out).all()
+    # ---- output of ALL tokens against the fp32 layer with the same weights
+    twin = G.f32_twin(layer, cfg)
+    x32 = G.f32_copy(x)
+    out32 = twin.forward(x32).to_numpy()
+    assert np.array_equal(twin.routing()["ids"], r["ids"])
+    G.assert_rows_close(out, out32, 1e-2, 2e-2, "fp32 twin, all tokens")
+    twin.close()
+    x32.free()
     # a second forward on the same input is bit-identical (no atomics anywhere on the path)
     assert np.array_equal(layer.forward(x).to_numpy(), out)
     layer.close()

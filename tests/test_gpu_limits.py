@@ -144,3 +144,75 @@ def test_two_layers_interleaved_and_device_side_copies():
     assert N.rel_l2(outA, G.oracle_forward(cfgA, inpA)["out"]) < 1e-2
     A.close()
     B.close()
+
+
+def test_stage_calls_out_of_order_are_refused():
+    """The stage entry points form the next stage's addresses from the index buffers the stage before left: a stage is
+    refused (on the host, before any launch) unless the stage before it ran for the same token count."""
+    from tests import gpu_util as G
+    P = G.P
+    cfg = C.MoEConfig("ord", T=96, d=256, E=4, K=2, H=256, dtype="bf16")
+    inp = make_inputs(cfg, 5)
+    layer = G.build_layer(cfg, inp, T_max=cfg.T)          # workspace allocated, index buffers uninitialised
+    lib, h = layer.lib, layer.handle
+    x = P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], "bf16")
+    out = P.DeviceBuffer(G.ctx(), (cfg.T, cfg.d), "bf16")
+    ms = __import__("ctypes").c_float()
+
+    def refused(st):
+        assert st == L.ERR_INVALID_ARG, st
+        assert b"has not run" in lib.omega_hip_last_error(G.ctx().handle)
+
+    # straight after create: nothing has run
+    refused(lib.omega_moe_dispatch(h, x.ptr, cfg.T))
+    refused(lib.omega_moe_experts_up(h, x.ptr, cfg.T))
+    refused(lib.omega_moe_experts_down(h, cfg.T))
+    refused(lib.omega_moe_combine(h, cfg.T, out.ptr))
+    for stage in (L.STAGE_DISPATCH, L.STAGE_UP, L.STAGE_DOWN, L.STAGE_COMBINE, L.STAGE_INDEX, L.STAGE_GATHER):
+        refused(lib.omega_moe_time_stage(h, stage, x.ptr, cfg.T, out.ptr, 0, 1, __import__("ctypes").byref(ms)))
+    # router for a smaller batch, then dispatch for a larger one
+    assert lib.omega_moe_router(h, x.ptr, 32) == L.OK
+    refused(lib.omega_moe_dispatch(h, x.ptr, cfg.T))
+    assert lib.omega_moe_dispatch(h, x.ptr, 32) == L.OK
+    refused(lib.omega_moe_experts(h, x.ptr, cfg.T))
+    refused(lib.omega_moe_combine(h, cfg.T, out.ptr))
+    # a new router run invalidates the dispatch that went before it
+    assert lib.omega_moe_router(h, x.ptr, 32) == L.OK
+    refused(lib.omega_moe_experts_up(h, x.ptr, 32))
+    # the stages in order give the forward's result
+    layer.number = cfg.T
+    for name in ("router", "dispatch", "experts"):
+        layer.stage(name, x)
+    layer.stage("combine", out=out)
+    staged = out.to_numpy()
+    assert np.array_equal(layer.forward(x).to_numpy(), staged)
+    # a forward leaves the stages usable for its T only
+    assert lib.omega_moe_combine(h, cfg.T, out.ptr) == L.OK
+    refused(lib.omega_moe_combine(h, cfg.T - 1, out.ptr))
+    layer.close()
+
+
+@pytest.mark.parametrize("training", [False, True])
+def test_backward_after_set_weights_is_refused(training):
+    """Activations (and the kept h1 / h3 of training mode) belong to the weights they were computed with: after
+    set_weights a backward pass needs a new forward."""
+    from tests import gpu_util as G
+    P = G.P
+    cfg = C.MoEConfig("sw", T=64, d=256, E=4, K=2, H=256, dtype="bf16")
+    inp = make_inputs(cfg, 6)
+    layer = G.build_layer(cfg, inp)
+    layer.set_training(training)
+    x = P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], "bf16")
+    dout = O.round_bf16(O.fill_normal(cfg.T * cfg.d, 6, 900, 1.0).reshape(cfg.T, cfg.d))
+    g = P.DeviceBuffer.from_numpy(G.ctx(), dout, "bf16")
+    layer.forward(x)
+    layer.back(g)
+    inp["W2"][1] = O.round_bf16(inp["W2"][1] * np.float32(0.5))
+    layer.set_expert(1, inp["W1"][1], inp["W3"][1], inp["W2"][1])
+    with pytest.raises(RuntimeError, match="no omega_moe_forward has run"):
+        layer.back(g)
+    layer.forward(x)
+    dx = layer.back(g).to_numpy()
+    bw = O.moe_backward(inp["x"], dout, inp["Wg"], None, inp["W1"], inp["W3"], inp["W2"], cfg.K, True, 0, bf16=True)
+    assert N.rel_l2(dx, bw["dx"]) < 1e-2
+    layer.close()
