@@ -231,6 +231,14 @@ int omega_moe_get_routing(omega_moe *moe, int T, int32_t *ids, float *w, int32_t
 /* Router intermediates, for tests: runs the router on x_dev and copies logits and probabilities
  * [T,E] to host (blocking).  Overwrites the routing state like omega_moe_router. */
 int omega_moe_get_router_probs(omega_moe *moe, const void *x_dev, int T, float *logits, float *probs);
+/* omega_moe_get_router_probs for callers that cannot allocate device memory (code under HIP graph capture around it,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same result and
+ * same effect on the routing state, but it calls no hipMalloc / hipFree: logits and probabilities are staged in a
+ * static device array of the library (2 x 4 MiB per device, held until the process ends) and the layer's workspace is
+ * never grown.  Refused with a message: T above the workspace the layer already holds (create it with T_max >= T), and
+ * T*E above 1048576.  All calls on one device share the array: calls that overlap on one device (two contexts, two
+ * threads) race on it. */
+int omega_moe_get_router_probs_noalloc(omega_moe *moe, const void *x_dev, int T, float *logits, float *probs);
 /* Host copy (blocking) of a workspace buffer of the last call, rows in logical order (row dst[p] of pair p,
  * then T rows per shared expert), row-major: which = 0 xg [T*K,d] (layer dtype), 1 a [T*K+Es*T,H] (layer
  * dtype), 2 y [T*K+Es*T,d] fp32; after omega_moe_backward of a bf16 layer also 3 dh1|dh3 [T*K+Es*T,2H] bf16, and for

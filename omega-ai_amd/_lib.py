@@ -67,6 +67,7 @@ SIGNATURES = {
     "omega_moe_combine": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "omega_moe_get_routing": (C.c_int, [C.c_void_p, C.c_int] + [C.c_void_p] * 6),
     "omega_moe_get_router_probs": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "omega_moe_get_router_probs_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "omega_moe_get_workspace": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "omega_moe_fill_workspace": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "omega_moe_time_stage": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int,

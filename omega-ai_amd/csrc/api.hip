@@ -11,6 +11,16 @@
 
 static thread_local std::string g_create_error;
 
+// Staging area of omega_moe_get_router_probs_noalloc: logits in the first half, probabilities in the second.  Every
+// device the library runs on holds its own copy of the array for the life of the process; host code never uses the
+// array's name as an address - omega_hip_ctx_create asks the runtime for the device's copy (hipGetSymbolAddress) and
+// keeps it per device.
+#define OMEGA_NOALLOC_MAX_FLOATS (1u << 20)  // T * E may not exceed this: 2 x 4 MiB per device
+static __device__ __align__(256) float scratch[2 * (size_t)OMEGA_NOALLOC_MAX_FLOATS];
+#define OMEGA_MAX_DEVICES 64
+static float *g_scratch_ptr[OMEGA_MAX_DEVICES];  // by device ordinal; written under g_scratch_mu
+static std::mutex g_scratch_mu;
+
 int omega_set_error(omega_ctx *ctx, int status, const char *what, hipError_t herr, const char *file, int line)
 {
     char buf[512];
@@ -44,9 +54,22 @@ int omega_hip_ctx_create(int device, omega_ctx **out)
     OMEGA_HIP_CHECK(nullptr, hipGetDeviceProperties(&prop, device));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         OMEGA_FAIL(nullptr, OMEGA_ERR_UNSUPPORTED, "ctx_create: device is not gfx950 (MI355X)");
+    if (device >= OMEGA_MAX_DEVICES) OMEGA_FAIL(nullptr, OMEGA_ERR_UNSUPPORTED, "ctx_create: device ordinal above 63");
+    float *scratch_dev = nullptr;
+    {
+        // once per device, with that device current: the address of its copy of the static scratch array
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        if (!g_scratch_ptr[device]) {
+            void *p = nullptr;
+            OMEGA_HIP_CHECK(nullptr, hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            g_scratch_ptr[device] = (float *)p;
+        }
+        scratch_dev = g_scratch_ptr[device];
+    }
     omega_ctx *c = new (std::nothrow) omega_ctx();
     if (!c) OMEGA_FAIL(nullptr, OMEGA_ERR_OOM, "ctx_create: host allocation failed");
     c->device = device;
+    c->noalloc_scratch = scratch_dev;
     c->num_cus = prop.multiProcessorCount;
     e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = experts_bf16_init();
@@ -1015,6 +1038,31 @@ int omega_moe_get_router_probs(omega_moe *m, const void *x, int T, float *logits
     hipFree(dl);
     if (dp) hipFree(dp);
     OMEGA_HIP_CHECK(ctx, e);
+    return OMEGA_OK;
+}
+
+// omega_moe_get_router_probs without any allocation: the device-side staging of logits and probabilities is the static
+// scratch array (this device's copy, through the pointer kept at ctx_create), and the workspace is never grown.
+// The router kernel writes every element of [T,E] that is copied out, so nothing needs clearing between calls.
+int omega_moe_get_router_probs_noalloc(omega_moe *m, const void *x, int T, float *logits, float *probs)
+{
+    MOE_ENTER(m);
+    stage_invalidates(m);
+    RUN(check_T(m, x, T, true));
+    if (T == 0) return OMEGA_OK;
+    if (T > m->T_cap)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_router_probs_noalloc: T exceeds the workspace the layer holds (create it with T_max >= T); this entry point never allocates");
+    const size_t n = (size_t)T * m->cfg.E;
+    if (n > OMEGA_NOALLOC_MAX_FLOATS)
+        OMEGA_FAIL(ctx, OMEGA_ERR_UNSUPPORTED, "get_router_probs_noalloc: T*E exceeds the static scratch of 1048576 values");
+    if (!ctx->noalloc_scratch) OMEGA_FAIL(ctx, OMEGA_ERR_HIP, "get_router_probs_noalloc: no scratch address for this device");
+    float *dl = ctx->noalloc_scratch, *dp = ctx->noalloc_scratch + OMEGA_NOALLOC_MAX_FLOATS;
+    m->routed_T = m->dispatched_T = -1;
+    OMEGA_HIP_CHECK(ctx, launch_router(m, x, T, dl, dp, ctx->stream));
+    m->routed_T = T;
+    if (logits) OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(logits, dl, n * 4, hipMemcpyDeviceToHost, ctx->stream));
+    if (probs) OMEGA_HIP_CHECK(ctx, hipMemcpyAsync(probs, dp, n * 4, hipMemcpyDeviceToHost, ctx->stream));
+    OMEGA_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
     return OMEGA_OK;
 }
 

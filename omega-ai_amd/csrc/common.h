@@ -17,6 +17,7 @@ struct omega_ctx {
     std::mutex mu;
     std::string last_error;
     int num_cus = 256;
+    float *noalloc_scratch = nullptr;  // this device's copy of the static scratch array of the allocation-free entry point
 };
 
 // One entry per row tile of the grouped products: written on the device by the scan kernel.

@@ -366,6 +366,13 @@ class MoELayer:
         self.ctx.check(self.lib.omega_moe_get_router_probs(self.handle, x.ptr, T, lg.ctypes.data, p.ctypes.data))
         return lg, p
 
+    def router_probs_noalloc(self, x, T):
+        """router_probs through the entry point that allocates nothing (T within T_max, T*E within 2^20)."""
+        lg = np.empty((T, self.nExperts), np.float32)
+        p = np.empty((T, self.nExperts), np.float32)
+        self.ctx.check(self.lib.omega_moe_get_router_probs_noalloc(self.handle, x.ptr, T, lg.ctypes.data, p.ctypes.data))
+        return lg, p
+
     def workspace(self, which, T):
         """Host copy of a workspace buffer in logical row order: 'xg' [T*K,d], 'a' [T*K+Es*T,H],
         'y' [T*K+Es*T,d] (fp32 values); after back() also 'dh' [T*K+Es*T,2H] (dh1 | dh3, bf16 layers) and
