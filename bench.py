@@ -37,6 +37,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c2_mixtral")
     ap.add_argument("--seed", type=int, default=20251)
+    ap.add_argument("--override", default="", help="replace dimensions of the named configuration, e.g. T=1024,K=8 "
+                                                    "(experiments; the default line is the configuration as named)")
     ap.add_argument("--router", default="exact", choices=["exact", "fast"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
@@ -57,6 +59,10 @@ def main():
     L = importlib.import_module("omega-ai_amd._lib")
     C = P.configs
     cfg = C.CONFIGS[a.config]
+    if a.override:
+        import dataclasses
+        kw = {k: int(v) for k, v in (item.split("=") for item in a.override.split(","))}
+        cfg = dataclasses.replace(cfg, name=cfg.name + "[" + a.override + "]", **kw)
     ctx = P.Context(0)
     layer = P.MoELayer(cfg.d, cfg.H, cfg.E, cfg.K, renorm=cfg.renorm, nShared=cfg.Es, bias=cfg.has_gate_bias, ctx=ctx,
                        dtype=cfg.dtype, router_mode=a.router, T_max=cfg.T)

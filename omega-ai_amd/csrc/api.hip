@@ -315,7 +315,7 @@ static int moe_reserve(omega_moe *m, int T)
     moe_free_workspace(m);
     const omega_moe_config &c = m->cfg;
     const size_t P = (size_t)T * c.K;
-    const int n_tok_tiles = ceil_div(T, ROUTER_TOK_TILE);
+    const int n_tok_tiles = ceil_div(T, router_tok_tile(c.E));
     const int bm = moe_tile_m(m, T);
     // every expert's rows start on a row-tile boundary: the buffers hold whole tiles
     m->tiles_cap = moe_max_m_tiles(m, T, bm);

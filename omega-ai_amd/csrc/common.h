@@ -150,7 +150,10 @@ struct omega_moe {
     size_t prof_used = 0;
 };
 
-#define ROUTER_TOK_TILE 32
+// Tokens per router workgroup = per row of tile_counts / tile_base and per workgroup of the rank kernel: 16 for layers
+// with at most 16 experts, else 32 (router.hip).
+int router_tok_tile(int E);
+#define ROUTER_TOK_TILE_MAX 32
 
 __host__ __device__ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 

@@ -3,7 +3,7 @@
 // Pair p = t*K+j goes to logical row dst[p] = offsets[id_p] + #{q<p : id_q == id_p} of the expert-contiguous
 // order (a stable counting sort of the pair list by expert id); src_row[dst[p]] = t.  In the buffers the
 // experts' segments start on row-tile boundaries (physical row dstp[p] = first_tile[id_p]*bm + rank).
-// The router left one histogram row per 32-token tile in tile_counts[tile][e].  Three launches:
+// The router left one histogram row per token tile (16 or 32 tokens, router_tok_tile) in tile_counts[tile][e].  Three launches:
 //   scan    one workgroup per 8 experts: exclusive prefix over the tiles of each expert (tile_base) and
 //           the per-expert totals -> counts[e]
 //   rank    one workgroup per token tile: offsets = exclusive scan of counts, first_tile = exclusive scan of
@@ -18,7 +18,7 @@
 #include "common.h"
 #include "pack.h"
 
-#define TOK_TILE ROUTER_TOK_TILE
+#define TOK_TILE_MAX ROUTER_TOK_TILE_MAX
 #define SCAN_EC 8     // experts per scan workgroup
 #define SCAN_SEG 32   // tile segments per expert
 
@@ -63,6 +63,10 @@ __device__ __forceinline__ int table_k_slices(int Nt, int ks_max, int KT)
     return max(1, min(min(ks_max, 256 / Nt), KT / 8));
 }
 
+// Row tiles of one group that run side by side on an XCD (see dispatch_rank_kernel): a group with more row tiles than
+// this is cut into row blocks of about equal size, each of which walks all column tiles.
+#define OMEGA_ROW_BLOCK_MAX 8
+
 __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ desc, int NT, int ncols, int g, int rows,
                                                   int Mg, int mt0, int total_mt, int bm, bool shared, int ks_max = 1,
                                                   int KT = 0)
@@ -71,17 +75,33 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
     const int Nt = total_mt * NT, r = Nt % 256;
     const int KS = table_k_slices(Nt, ks_max, KT);
     const int S = (r == 0 || r > 128 || KS > 1) ? 1 : min(4, 256 / r);
-    const int nblk = (rows + 31) >> 5;  // 32-row blocks of the group, dealt evenly to its Mg row tiles
+    // the group's rows are dealt evenly, in blocks of 32, to its Mg row tiles (instead of full tiles and a ragged last
+    // one): the same number of tiles and of MFMA blocks, but tiles of nearly one cost.  (Equal tiles in units of 16 rows -
+    // every tile the same number of MFMA blocks, the last one of each half empty - cut the L2 miss traffic of the up
+    // product by a fifth when every expert has 1040 rows, and still lost 4 % of time to the extra blocks.)
+    const int nblk = (rows + 31) >> 5;
+    // order within the group: row blocks of RB row tiles; inside a row block column tile after column tile, the row
+    // tiles of the block fastest
+    const int NB = (Mg + OMEGA_ROW_BLOCK_MAX - 1) / OMEGA_ROW_BLOCK_MAX;
     for (int l = threadIdx.x; l < Mg * NT; l += 256) {
-        const int mt = l % Mg, n = l / Mg;
+        // row block b holds row tiles [b*Mg/NB, (b+1)*Mg/NB); the entries before it number (first tile) * NT
+        int b = min(NB - 1, (l / NT) * NB / Mg);
+        while ((b * Mg) / NB * NT > l) --b;
+        while (b + 1 < NB && ((b + 1) * Mg) / NB * NT <= l) ++b;
+        const int f = (b * Mg) / NB, RB = ((b + 1) * Mg) / NB - f;
+        const int li = l - f * NT;
+        const int mt = f + li % RB, n = li / RB;
         const int at = mt0 * NT + l;
         const int tfirst = 32 * ((mt * nblk) / Mg);
         const int trows = min(32 * (((mt + 1) * nblk) / Mg), rows) - tfirst;
         omega_tile_desc dsc;
         dsc.g = g;
         dsc.n0 = n * ncols;
-        dsc.a_rg = dsc.kt0 = 0;
+        dsc.a_rg = 0;
         dsc.b_rg = ncols == 128 ? 1 : 0;  // read by the plain 256-column products only: a half-width item
+        // (items without k slices: kt0 = first 32 x 32 block record of the item - 8 records per row-tile slot - for the
+        //  products that keep or read h1 / h3 block records)
+        dsc.kt0 = (mt0 + mt) * 8;
         if (KS > 1) {
             // slice ks of KS (a_rg = KS, kt0 = ks) adds its part of the k range into partial result ks; adjacent
             // entries, so the slices of a tile run on one XCD and share its rows
@@ -100,11 +120,13 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
             desc[at] = dsc;
         } else {
             const int tb = (trows + 31) >> 5;  // the tile's 32-row blocks, dealt evenly to the S slices
+            const int rec0 = dsc.kt0;
             for (int sl = 0; sl < S; ++sl) {
                 const int sfirst = 32 * ((sl * tb) / S);
                 dsc.row0 = mt0 * bm + tfirst + sfirst;
                 dsc.rows = max(0, min(32 * (((sl + 1) * tb) / S), trows) - sfirst);  // 0: nothing to do
                 dsc.xrow0 = shared ? tfirst + sfirst : -1;
+                dsc.kt0 = rec0 + (sfirst >> 5);
                 desc[Nt - r + (at - (Nt - r)) * S + sl] = dsc;
             }
         }
@@ -125,8 +147,8 @@ __device__ __forceinline__ int table_entries(int total_mt, int NT, int ks_max = 
 #define MAXE 256
 __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__restrict__ ids,
                                                             const int32_t *__restrict__ tile_base,
-                                                            const int32_t *__restrict__ counts, int T, int K, int E,
-                                                            int Es, int bm, int32_t *__restrict__ offsets,
+                                                            const int32_t *__restrict__ counts, int T, int tok_tile, int K,
+                                                            int E, int Es, int bm, int32_t *__restrict__ offsets,
                                                             int32_t *__restrict__ dst, int32_t *__restrict__ dstp,
                                                             int32_t *__restrict__ src_row,
                                                             omega_tile *__restrict__ tiles,
@@ -137,10 +159,10 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
 {
     __shared__ int off_s[MAXE + 1];        // logical first row of each expert
     __shared__ int mt_s[MAXE + 64 + 1];    // first row tile of each group (routed, then shared)
-    __shared__ int id_s[TOK_TILE * 64];    // K <= 64
+    __shared__ int id_s[TOK_TILE_MAX * 64];    // K <= 64
     const int tid = threadIdx.x, tile = blockIdx.x;
-    const int t0 = tile * TOK_TILE;
-    const int npairs = min(TOK_TILE, T - t0) * K;
+    const int t0 = tile * tok_tile;
+    const int npairs = min(tok_tile, T - t0) * K;
 
     // exclusive scans of the E counts and of their tile counts: one wave, 4 experts per lane
     if (tid < 64) {
@@ -208,7 +230,13 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
 
     // ---- work-item tables of the two grouped products (bf16 layers) ----
     // Tile number first_tile[g]*NT + n*Mg + m = (expert g, column tile n, row tile m): row tiles fastest, so that
-    // tiles that run at the same time share weight tiles.  The rows of a group are dealt evenly (in blocks of 32) to
+    // tiles that run at the same time share weight tiles.  A group with more than OMEGA_ROW_BLOCK_MAX row tiles is cut
+    // into row blocks of at most that many row tiles, each walking all column tiles (row tiles of the block fastest):
+    // the 32 consecutive entries an XCD works on at a time then form a block of about 8 row tiles x 4 column tiles that
+    // fetches each of its operand tiles once, where one column tile x 32 row tiles would fetch the rows again for every
+    // column tile (down product: 8192 tokens, 64 experts + 2 shared, 0.390 -> 0.368 ms; 16384 tokens, 128 skewed
+    // experts, 0.502 -> 0.486 ms).
+    // The rows of a group are dealt evenly (in blocks of 32) to
     // its row tiles, instead of full tiles and a ragged last one: the same number of tiles and of MFMA blocks, but
     // tiles of one cost, so that the workgroups of an XCD, which share operand tiles through its L2, stay in step.
     // The compute units take 256 tiles at a time; when the
@@ -425,12 +453,13 @@ __global__ __launch_bounds__(256) void dispatch_gather_bytes_kernel(const unsign
 hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
-    const int n_tiles = ceil_div(T, TOK_TILE);
+    const int tok_tile = router_tok_tile(c.E);
+    const int n_tiles = ceil_div(T, tok_tile);
     hipLaunchKernelGGL(dispatch_scan_kernel, dim3(ceil_div(c.E, SCAN_EC)), dim3(256), 0, s, m->tile_counts,
                        m->tile_base, n_tiles, c.E, m->counts);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(dispatch_rank_kernel, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_base, m->counts, T, c.K,
+    hipLaunchKernelGGL(dispatch_rank_kernel, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_base, m->counts, T, tok_tile, c.K,
                        c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles, m->tile_meta, m->desc_up, c.H / 128, 128,
                        m->desc_down, c.d / m->down_cols, m->down_cols, m->down_ks_max, c.H / 32);
     return hipGetLastError();

@@ -94,6 +94,7 @@ struct TileCtx {
     int kt;                   // k steps of the item
     int half;                 // plain 256-column products: the item covers the first 128 columns only
     int slab;                 // MODE_DOWNK: which partial result the item writes
+    int rec0;                 // products that write or read h1 / h3 block records: record of the item's first 32-row block
 };
 
 __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char *p)
@@ -118,6 +119,8 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
         const size_t k0 = (size_t)d.kt0 * 8192;
         c.kt = d.xrow0;
         c.half = 0;
+        c.slab = 0;
+        c.rec0 = 0;
         c.A = uniform_ptr((const unsigned char *)Axg + (size_t)d.a_rg * rg_bytes + k0);
         c.B0 = uniform_ptr((const unsigned char *)Wa + (size_t)d.b_rg * rg_bytes + k0);
         c.B1 = uniform_ptr(c.B0 + rg_bytes);
@@ -127,6 +130,7 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
     }
     c.kt = KT;
     c.slab = 0;
+    c.rec0 = d.kt0;
     c.half = FUSED ? 0 : d.b_rg;
     // k slices (tables of small batches, items with a_rg = KS > 1 and kt0 = ks): MODE_DOWNK runs slice ks over its own
     // part of the k range; a launch that knows nothing of partial results (MODE_DOWN) computes the whole range in the
@@ -195,6 +199,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     ctx.n0 = __builtin_amdgcn_readfirstlane(ctx_in.n0);
     ctx.half = __builtin_amdgcn_readfirstlane(ctx_in.half);
     ctx.slab = __builtin_amdgcn_readfirstlane(ctx_in.slab);
+    ctx.rec0 = __builtin_amdgcn_readfirstlane(ctx_in.rec0);
     int cur = __builtin_amdgcn_readfirstlane(cur_io);
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -213,16 +218,17 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     // ---- MFMA operand addressing ----
     // Row (2i + wm)*32 + l32 of A, row j*128 + wn*32 + l32 (up: block 0 = 32 columns of W1, block 1 = the same 32
     // columns of W3) or wn*64 + j*32 + l32 (down) of B.  The chunk swizzle depends on the row only through l32
-    // (rows differ by multiples of 32), so one swizzled k offset serves every block and the blocks are constant
-    // byte offsets.
+    // (rows differ by multiples of 32), so one swizzled k offset per operand serves every block and the blocks are
+    // constant byte offsets.
+    // (An item may start 16 rows into a 32-row unit of the packed image: the swizzle of the A rows follows the
+    //  physical row, i.e. l32 with bit 4 flipped.)
     const int l32 = lane & 31, lhi = lane >> 5;
-    const int sw = swz(l32);
+    const int sw = swz(l32), swa = swz(l32 ^ (MODE == MODE_WGRAD ? 0 : (ctx.row0 & 16)));
     uint32_t pa[2], pb[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-        const uint32_t ko = (uint32_t)((ks * 2 + lhi) ^ sw) << 4;
-        pa[ks] = (uint32_t)(wm * 32 + l32) * (BK * 2) + ko;
-        pb[ks] = TILE_BYTES + (uint32_t)((FUSED ? wn * 32 : wn * 64) + l32) * (BK * 2) + ko;
+        pa[ks] = (uint32_t)(wm * 32 + l32) * (BK * 2) + ((uint32_t)((ks * 2 + lhi) ^ swa) << 4);
+        pb[ks] = TILE_BYTES + (uint32_t)((FUSED ? wn * 32 : wn * 64) + l32) * (BK * 2) + ((uint32_t)((ks * 2 + lhi) ^ sw) << 4);
     }
     constexpr uint32_t A_BLK = 64 * BK * 2, B_BLK = (FUSED ? 128 : 32) * BK * 2;
 #define READ_FRAGS(AF, BF, stage, ks)                                                                       \
@@ -339,7 +345,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         float *r1 = (float *)(MODE == MODE_UPRAW ? Cout : Aux1), *r3 = (float *)(MODE == MODE_UPRAW ? Aux1 : Aux2);
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
-            const size_t rb = (size_t)(ctx.row0 >> 5) + 2 * i + wm;
+            const size_t rb = (size_t)ctx.rec0 + 2 * i + wm;
             float *o1 = r1 + (rb * ncb + cb) * 1024 + lane, *o3 = r3 + (rb * ncb + cb) * 1024 + lane;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -356,7 +362,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
             const int row = (2 * i + wm) * 32 + l32;
-            const size_t rb = (size_t)(ctx.row0 >> 5) + 2 * i + wm;
+            const size_t rb = (size_t)ctx.rec0 + 2 * i + wm;
             const int prow = ctx.row0 + row;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {

@@ -1,6 +1,8 @@
 // Router: gate projection, row softmax, wave-level top-k, per-token-tile expert histogram.
 //
-// One workgroup (256 threads) routes a tile of 32 tokens.
+// One workgroup routes a tile of TT tokens: 32 (256 threads), or 16 for layers with at most 16 experts (one thread per
+// token and expert, 128 or 256 threads: the sums are bound by LDS reads per compute unit, so such a layer spreads its
+// tokens over twice as many workgroups).
 //  phase 1  logits[t,e] = sum_k x[t,k]*Wg[e,k] (+bg[e]): one lane per (token, expert); x and Wg are
 //           staged through LDS in chunks of 64..256 k.  EXACT mode adds the products one k at a time with
 //           a separate multiply and add (this file is compiled with -ffp-contract=off), which is the
@@ -16,8 +18,15 @@
 // FAST mode of bf16 layers with more than 16 experts takes phase 1 to the matrix cores (router_mfma_kernel below).
 #include "common.h"
 
-#define TOK_TILE ROUTER_TOK_TILE
 #define ROUTER_EPT(EP) ((EP) >= 128 ? 4 : (EP) >= 32 ? 2 : 1)
+// token tile and threads per workgroup for EP (padded) experts
+#define ROUTER_TT(EP) ((EP) <= 16 ? 16 : 32)
+#define ROUTER_NTHR(EP) ((EP) <= 8 ? 128 : 256)
+// k per staged chunk for at most 16 experts: with 16-token tiles the sums of a 256-k chunk take less time than the
+// next chunk's loads need to arrive, and the kernel is bound by one memory latency per chunk: 512-k chunks halve their
+// number (Mixtral shape, 4096 tokens: 32-token tiles 42 us; 16-token tiles 54 us with 256-k chunks, 34 us with 512)
+#define ROUTER_KC_SMALL 512
+int router_tok_tile(int E) { return E <= 16 ? 16 : 32; }
 
 // Phase 1 for the tokens t0.. of one workgroup: acc[x*NT + i] = logit of (token tg + i*TPP, expert e1 + x*EL), bias
 // not yet added.  A thread owns EPT experts (2 from 128 experts on: each x value read from LDS then feeds two sums,
@@ -31,20 +40,24 @@
 template <int EP, int KC, bool EXACT, bool XBF, bool FAST_IO>
 __device__ __forceinline__ void router_sums(const void *__restrict__ x, const void *__restrict__ Wg, int T, int d, int E,
                                             int t0, float (*xs)[KC + 4], float (*ws)[KC + 4],
-                                            float (&acc)[TOK_TILE * EP / 256])
+                                            float (&acc)[ROUTER_TT(EP) * EP / ROUTER_NTHR(EP)])
 {
+    constexpr int TOK_TILE = ROUTER_TT(EP), NTHR = ROUTER_NTHR(EP);
     constexpr int EPT = ROUTER_EPT(EP);           // experts per thread
     constexpr int EL = EP / EPT;                  // threads across the experts
-    constexpr int NT = TOK_TILE * EL / 256;       // tokens per thread
-    constexpr int TPP = 256 / EL;                 // tokens per pass
+    constexpr int NT = TOK_TILE * EL / NTHR;      // tokens per thread
+    constexpr int TPP = NTHR / EL;                // tokens per pass
+    static_assert(NT >= 1 && NT * NTHR == TOK_TILE * EL, "every thread owns whole (token, expert) sums");
+    constexpr int TPR = NTHR / TOK_TILE;          // staging threads per token row (8 or 16)
+    static_assert(TPR * TOK_TILE == NTHR && KC % (8 * TPR) == 0, "whole staging vectors per thread");
     const int tid = threadIdx.x;
     const int e1 = tid % EL, tg = tid / EL;
     // staging: every thread carries 8 consecutive k of one token and of WCH gate rows from global memory to LDS;
     // the next chunk is fetched into registers while the current one is being summed
-    constexpr int XCH = KC / 64;
-    constexpr int WCH = EP * (KC / 8) / 256;
-    static_assert(EP * (KC / 8) % 256 == 0, "every thread stages the same number of gate vectors");
-    const int x_tt = tid >> 3, x_ks = (tid & 7) * 8;
+    constexpr int XCH = KC / (8 * TPR);
+    constexpr int WCH = EP * (KC / 8) / NTHR;
+    static_assert(EP * (KC / 8) % NTHR == 0, "every thread stages the same number of gate vectors");
+    const int x_tt = tid / TPR, x_ks = (tid % TPR) * 8;
     // raw staging registers: 8 k of bf16 = one uint4, 8 k of fp32 = two; conversion happens when they are
     // written to LDS, so the global loads stay in flight during the sums of the current chunk
     uint4 xr[XCH][2], wr[WCH][2];
@@ -93,19 +106,19 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
     };
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int c = 0; c < XCH; ++c) load8(x, t0 + x_tt, T, k0 + x_ks + 64 * c, xr[c]);
+        for (int c = 0; c < XCH; ++c) load8(x, t0 + x_tt, T, k0 + x_ks + 8 * TPR * c, xr[c]);
 #pragma unroll
         for (int c = 0; c < WCH; ++c) {
-            const int idx = tid + c * 256;
+            const int idx = tid + c * NTHR;
             load8(Wg, idx / (KC / 8), E, k0 + (idx % (KC / 8)) * 8, wr[c]);
         }
     };
     auto stash = [&]() {
 #pragma unroll
-        for (int c = 0; c < XCH; ++c) widen(xr[c], &xs[x_tt][x_ks + 64 * c]);
+        for (int c = 0; c < XCH; ++c) widen(xr[c], &xs[x_tt][x_ks + 8 * TPR * c]);
 #pragma unroll
         for (int c = 0; c < WCH; ++c) {
-            const int idx = tid + c * 256;
+            const int idx = tid + c * NTHR;
             widen(wr[c], &ws[idx / (KC / 8)][(idx % (KC / 8)) * 8]);
         }
     };
@@ -169,7 +182,7 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
 // and visible on entry).  RELAXED (the matrix-core FAST path only, tolerance mode): exponentials in single precision
 // and the softmax sum as a butterfly over the lanes instead of the reference's order - the ordered sum is a chain of
 // EP dependent cross-lane reads per token and dominates that path otherwise.
-template <int EP, bool RELAXED = false>
+template <int EP, bool RELAXED = false, int TOK_TILE = 32, int NTHR = 256>
 __device__ __forceinline__ void router_select(float (*lg)[EP], int *hist, int t0, int tile, int T, int E, int K, int renorm,
                                               int32_t *__restrict__ ids, float *__restrict__ wout,
                                               int32_t *__restrict__ tile_counts, float *__restrict__ probs_out)
@@ -185,7 +198,7 @@ __device__ __forceinline__ void router_select(float (*lg)[EP], int *hist, int t0
     for (int pass = 0; pass < PASSES; ++pass) {
         const int tt = wave * 8 + pass * TOK_PER_PASS + grp;
         const int t = t0 + tt;
-        if (t >= T) continue;  // uniform over the GS lanes that exchange data
+        if (t >= T || tt >= TOK_TILE) continue;  // uniform over the GS lanes that exchange data
         float v[VPL], p[VPL];
         float mx = -INFINITY;
 #pragma unroll
@@ -253,19 +266,20 @@ __device__ __forceinline__ void router_select(float (*lg)[EP], int *hist, int t0
         }
     }
     __syncthreads();
-    for (int e = tid; e < E; e += 256) tile_counts[(size_t)tile * E + e] = hist[e];
+    for (int e = tid; e < E; e += NTHR) tile_counts[(size_t)tile * E + e] = hist[e];
 }
 
 template <int EP, int KC, bool EXACT>
-__global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
+__global__ __launch_bounds__(ROUTER_NTHR(EP)) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
                                                      const float *__restrict__ bg, int T, int d, int E, int K,
                                                      int renorm, int32_t *__restrict__ ids,
                                                      float *__restrict__ wout, int32_t *__restrict__ tile_counts,
                                                      float *__restrict__ logits_out, float *__restrict__ probs_out)
 {
+    constexpr int TOK_TILE = ROUTER_TT(EP), NTHR = ROUTER_NTHR(EP);
     constexpr int EPT = ROUTER_EPT(EP), EL = EP / EPT;  // phase 1: experts per thread, threads across the experts
-    constexpr int NT = TOK_TILE * EL / 256;             // tokens per thread in phase 1
-    constexpr int TPP = 256 / EL;                       // tokens per pass
+    constexpr int NT = TOK_TILE * EL / NTHR;            // tokens per thread in phase 1
+    constexpr int TPP = NTHR / EL;                      // tokens per pass
     constexpr int LDW = KC + 4;  // LDS row stride in floats: rows stay 16-byte aligned and bank-staggered
     __shared__ __attribute__((aligned(16))) float xs[TOK_TILE][LDW];
     __shared__ __attribute__((aligned(16))) float ws[EP][LDW];
@@ -309,7 +323,7 @@ __global__ __launch_bounds__(256) void router_kernel(const void *__restrict__ x,
     }
     __syncthreads();
 
-    router_select<EP>(lg, hist, t0, tile, T, E, K, renorm, ids, wout, tile_counts, probs_out);
+    router_select<EP, false, TOK_TILE, NTHR>(lg, hist, t0, tile, T, E, K, renorm, ids, wout, tile_counts, probs_out);
 }
 
 // FAST mode of bf16 layers with 32 experts or more: the gate projection on the matrix cores.  x and Wg are bf16, so
@@ -328,6 +342,7 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t *__restri
                                                           int32_t *__restrict__ tile_counts, float *__restrict__ logits_out,
                                                           float *__restrict__ probs_out)
 {
+    constexpr int TOK_TILE = 32;                // only layers with more than 16 experts take this kernel
     constexpr int NB = EP / 32;                 // expert blocks
     // up to 64 experts every wave takes all blocks and a quarter of k; from 128 on the waves split the blocks (measured:
     // 64 experts 0.064 -> 0.058 ms with the k split at T = 8192, d = 2048; 128 experts 0.125 -> 0.157 ms at T = 16384)
@@ -410,7 +425,7 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t *__restri
 hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
-    const int tiles = ceil_div(T, TOK_TILE);
+    const int tiles = ceil_div(T, router_tok_tile(c.E));
     const int exact = c.router_mode == OMEGA_ROUTER_EXACT;
     const float *bg = c.has_gate_bias ? m->bg : nullptr;
     if (!exact && c.dtype == OMEGA_DTYPE_BF16 && c.E > 16 && ((uintptr_t)x % 16) == 0) {
@@ -427,15 +442,15 @@ hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits
 #define ROUTER_LAUNCH(EPV, KCV)                                                                                    \
     do {                                                                                                           \
         if (exact)                                                                                                 \
-            hipLaunchKernelGGL((router_kernel<EPV, KCV, true>), dim3(tiles), dim3(256), 0, s, x, c.dtype, m->Wg, bg, \
+            hipLaunchKernelGGL((router_kernel<EPV, KCV, true>), dim3(tiles), dim3(ROUTER_NTHR(EPV)), 0, s, x, c.dtype, m->Wg, bg, \
                                T, c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out, probs_out);   \
         else                                                                                                       \
-            hipLaunchKernelGGL((router_kernel<EPV, KCV, false>), dim3(tiles), dim3(256), 0, s, x, c.dtype, m->Wg,    \
+            hipLaunchKernelGGL((router_kernel<EPV, KCV, false>), dim3(tiles), dim3(ROUTER_NTHR(EPV)), 0, s, x, c.dtype, m->Wg,    \
                                bg, T, c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out,           \
                                probs_out);                                                                         \
     } while (0)
-    if (c.E <= 8) ROUTER_LAUNCH(8, 256);
-    else if (c.E <= 16) ROUTER_LAUNCH(16, 256);
+    if (c.E <= 8) ROUTER_LAUNCH(8, ROUTER_KC_SMALL);
+    else if (c.E <= 16) ROUTER_LAUNCH(16, ROUTER_KC_SMALL);
     else if (c.E <= 32) ROUTER_LAUNCH(32, 128);
     else if (c.E <= 64) ROUTER_LAUNCH(64, 64);
     else if (c.E <= 128) ROUTER_LAUNCH(128, 64);
