@@ -337,7 +337,11 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
                 // needs no dealing - it adds the same work to every queue: each workgroup takes the entry of its place
                 const unsigned long long act = __ballot(lane < wpx);
                 const int c0 = __builtin_amdgcn_readfirstlane(c);
+#ifdef SCHED_NODEAL
+                if (true) {
+#else
                 if (__ballot(lane < wpx && c == c0) == act) {
+#endif
                     ce = c;
                     src = lane;
                 } else {
