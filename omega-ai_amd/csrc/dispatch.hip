@@ -80,8 +80,11 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
     // every tile the same number of MFMA blocks, the last one of each half empty - cut the L2 miss traffic of the up
     // product by a fifth when every expert has 1040 rows, and still lost 4 % of time to the extra blocks.)
     const int nblk = (rows + 31) >> 5;
+    const int qblk = nblk / Mg, nhi = nblk % Mg;  // the first nhi row tiles hold qblk + 1 blocks, the others qblk
     // order within the group: row blocks of RB row tiles; inside a row block column tile after column tile, the row
-    // tiles of the block fastest
+    // tiles of the block fastest.  (Walking the column tiles twice, first with the taller row tiles and then with the
+    // others, makes most rounds of 32 entries cost the same, so that the queue builder has nothing to deal: dispatch
+    // 50 -> 39 us at the Mixtral shape, but its up product 1.529 -> 1.544 ms - each weight tile is then fetched twice.)
     const int NB = (Mg + OMEGA_ROW_BLOCK_MAX - 1) / OMEGA_ROW_BLOCK_MAX;
     for (int l = threadIdx.x; l < Mg * NT; l += 256) {
         // row block b holds row tiles [b*Mg/NB, (b+1)*Mg/NB); the entries before it number (first tile) * NT
@@ -92,8 +95,8 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
         const int li = l - f * NT;
         const int mt = f + li % RB, n = li / RB;
         const int at = mt0 * NT + l;
-        const int tfirst = 32 * ((mt * nblk) / Mg);
-        const int trows = min(32 * (((mt + 1) * nblk) / Mg), rows) - tfirst;
+        const int tfirst = 32 * (mt * qblk + min(mt, nhi));
+        const int trows = min(32 * ((mt + 1) * qblk + min(mt + 1, nhi)), rows) - tfirst;
         omega_tile_desc dsc;
         dsc.g = g;
         dsc.n0 = n * ncols;
@@ -337,11 +340,7 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
                 // needs no dealing - it adds the same work to every queue: each workgroup takes the entry of its place
                 const unsigned long long act = __ballot(lane < wpx);
                 const int c0 = __builtin_amdgcn_readfirstlane(c);
-#ifdef SCHED_NODEAL
-                if (true) {
-#else
                 if (__ballot(lane < wpx && c == c0) == act) {
-#endif
                     ce = c;
                     src = lane;
                 } else {

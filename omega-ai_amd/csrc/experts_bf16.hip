@@ -85,11 +85,23 @@ __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t
                  : "memory");
 }
 
+// The same with only the lanes of `mask` taking part: a wave whose 16-row block of the A tile holds no valid row keeps
+// its place in the load sequence (the waits count instructions) but moves 16 bytes instead of 1 KiB.
+__device__ __forceinline__ void dma16_masked(const void *sbase, uint32_t voff, uint32_t lds_base, uint64_t mask)
+{
+    uint64_t saved;
+    asm volatile("s_mov_b32 m0, %3\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\tglobal_load_lds_dwordx4 %2, %1\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "s"(sbase), "v"(voff), "s"(lds_base), "s"(mask)
+                 : "memory");
+}
+
 // Everything the loads of one work item need (uniform over the workgroup except the two lane offsets).
 // A: packed row group of the tile's first row; B0/B1: packed row groups of the two 128-row halves of the B tile.
 struct TileCtx {
     const unsigned char *A, *B0, *B1;
     uint32_t a_off0, a_off1;  // this lane's byte offsets of its two A blocks within a k step
+    uint64_t a_mask0, a_mask1;  // lanes that take part in the two A loads: all, or lane 0 alone for a block without valid rows
     int row0, rows, n0;
     int kt;                   // k steps of the item
     int half;                 // plain 256-column products: the item covers the first 128 columns only
@@ -102,6 +114,12 @@ __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char 
     const uint64_t v = (uint64_t)p;
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (const unsigned char *)(((uint64_t)hi << 32) | lo);
+}
+
+__device__ __forceinline__ uint64_t uniform_u64(uint64_t v)
+{
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
 }
 
 template <int MODE>
@@ -126,6 +144,7 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
         c.B1 = uniform_ptr(c.B0 + rg_bytes);
         c.a_off0 = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
         c.a_off1 = (uint32_t)KT * 8192u + c.a_off0;
+        c.a_mask0 = c.a_mask1 = ~0ull;
         return c;
     }
     c.kt = KT;
@@ -160,16 +179,23 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
     const int qa0 = blk0 + (16 * wave < d.rows ? wave : 0), qa1 = blk0 + (16 * (wave + 8) < d.rows ? wave + 8 : 0);
     c.a_off0 = (uint32_t)(qa0 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa0 & 7) * 1024u + (uint32_t)lane * 16u;
     c.a_off1 = (uint32_t)(qa1 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa1 & 7) * 1024u + (uint32_t)lane * 16u;
+    c.a_mask0 = 16 * wave < c.rows ? ~0ull : 1ull;
+    c.a_mask1 = 16 * (wave + 8) < c.rows ? ~0ull : 1ull;
     return c;
 }
 
 // direct load n (0..3) of k step `kstep` of a work item into ring stage `stage`: n -> (operand, row group) =
 // (n & 1 ? B : A, n >> 1)
+// MASKED: A blocks without valid rows move 16 bytes (every product but the k-sliced one of small batches, whose items
+// are bound by the weight stream and whose kernel has no registers to spare)
+#define LOADS_MASKED(M) ((M) != MODE_DOWNK)
+template <bool MASKED>
 __device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, uint32_t blk_off, int stage, int kstep, int n)
 {
     const uint32_t sb = lds_wave + stage * STAGE_BYTES;
     const uint32_t kb = (uint32_t)kstep * 8192u;
-    if ((n & 1) == 0) dma16(c.A, kb + ((n >> 1) ? c.a_off1 : c.a_off0), sb + (n >> 1) * 8192);
+    if ((n & 1) == 0 && MASKED) dma16_masked(c.A, kb + ((n >> 1) ? c.a_off1 : c.a_off0), sb + (n >> 1) * 8192, (n >> 1) ? c.a_mask1 : c.a_mask0);
+    else if ((n & 1) == 0) dma16(c.A, kb + ((n >> 1) ? c.a_off1 : c.a_off0), sb + (n >> 1) * 8192);
     else dma16((n >> 1) == 0 ? c.B0 : c.B1, kb + blk_off, sb + TILE_BYTES + (n >> 1) * 8192);
 }
 
@@ -200,6 +226,10 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     ctx.half = __builtin_amdgcn_readfirstlane(ctx_in.half);
     ctx.slab = __builtin_amdgcn_readfirstlane(ctx_in.slab);
     ctx.rec0 = __builtin_amdgcn_readfirstlane(ctx_in.rec0);
+    if (LOADS_MASKED(MODE)) {
+        ctx.a_mask0 = uniform_u64(ctx_in.a_mask0);
+        ctx.a_mask1 = uniform_u64(ctx_in.a_mask1);
+    }
     int cur = __builtin_amdgcn_readfirstlane(cur_io);
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -211,8 +241,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 // load n of virtual k step v: steps beyond this item's last belong to the next item
 #define ISSUE_V(stage, v, n)                                                              \
     do {                                                                                  \
-        if ((v) < KT) issue_load(ctx, lds_wave, blk_off, stage, v, n);                    \
-        else if (has_next) issue_load(nx, lds_wave, blk_off, stage, (v) - KT, n);          \
+        if ((v) < KT) issue_load<LOADS_MASKED(MODE)>(ctx, lds_wave, blk_off, stage, v, n);                    \
+        else if (has_next) issue_load<LOADS_MASKED(MODE)>(nx, lds_wave, blk_off, stage, (v) - KT, n);          \
     } while (0)
 
     // ---- MFMA operand addressing ----
@@ -280,7 +310,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         {                                                                                                   \
             if ((i & 1) == 0) {                                                                             \
                 if (GEN) ISSUE_V(prv, kt - 1 + NSTAGE, 2 + (i >> 1));                                       \
-                else issue_load(ctx, lds_wave, blk_off, prv, kt - 1 + NSTAGE, 2 + (i >> 1));                \
+                else issue_load<LOADS_MASKED(MODE)>(ctx, lds_wave, blk_off, prv, kt - 1 + NSTAGE, 2 + (i >> 1));                \
             }                                                                                               \
             MFMA2(af0, bf0, i);                                                                             \
         }                                                                                                   \
@@ -294,7 +324,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         {                                                                                                   \
             if ((i & 1) == 0) {                                                                             \
                 if (GEN) ISSUE_V(cur, kt + NSTAGE, i >> 1);                                                 \
-                else issue_load(ctx, lds_wave, blk_off, cur, kt + NSTAGE, i >> 1);                          \
+                else issue_load<LOADS_MASKED(MODE)>(ctx, lds_wave, blk_off, cur, kt + NSTAGE, i >> 1);                          \
             }                                                                                               \
             MFMA2(af1, bf1, i);                                                                             \
         }                                                                                                   \
@@ -438,10 +468,10 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
         const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
         for (int st = 0; st < NSTAGE - 1; ++st) {
 #pragma unroll
-            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load(cur_ctx, lds_wave, blk_off, st, st, n);
+            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<LOADS_MASKED(MODE)>(cur_ctx, lds_wave, blk_off, st, st, n);
         }
-        issue_load(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 0);
-        issue_load(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 1);
+        issue_load<LOADS_MASKED(MODE)>(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 0);
+        issue_load<LOADS_MASKED(MODE)>(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 1);
         asm volatile("s_waitcnt vmcnt(14)" ::: "memory");  // all but steps 1.. : LOADS_PER_STEP * (NSTAGE - 2) + 2
         __syncthreads();
     }
