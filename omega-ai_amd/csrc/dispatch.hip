@@ -3,13 +3,15 @@
 // Pair p = t*K+j goes to logical row dst[p] = offsets[id_p] + #{q<p : id_q == id_p} of the expert-contiguous
 // order (a stable counting sort of the pair list by expert id); src_row[dst[p]] = t.  In the buffers the
 // experts' segments start on row-tile boundaries (physical row dstp[p] = first_tile[id_p]*bm + rank).
-// The router left one histogram row per token tile (16 or 32 tokens, router_tok_tile) in tile_counts[tile][e].  Three launches:
-//   scan    one workgroup per 8 experts: exclusive prefix over the tiles of each expert (tile_base) and
-//           the per-expert totals -> counts[e]
-//   rank    one workgroup per token tile: offsets = exclusive scan of counts, first_tile = exclusive scan of
-//           ceil(counts/bm); rank of each pair among the earlier pairs of its tile with the same expert;
-//           dst/dstp/src_row; workgroup 0 also publishes offsets and the row-tile list that schedules the
-//           grouped products
+// The router left one histogram row per token tile (16 or 32 tokens, router_tok_tile) in tile_counts[tile][e].  Two
+// launches - three when the histogram is large:
+//   scan    (histograms above 16384 cells only) one workgroup per 8 experts: exclusive prefix over the tiles of each
+//           expert (tile_base) and the per-expert totals -> counts[e]
+//   rank    one workgroup per token tile: the prefix of its tile and the totals (summed from the histogram rows in the
+//           same pass unless a scan launch left them); offsets = exclusive scan of counts, first_tile = exclusive scan
+//           of ceil(counts/bm); rank of each pair among the earlier pairs of its tile with the same expert (ballots
+//           within 64-pair chunks, per-chunk counts across them); dst/dstp/src_row; workgroup g (mod grid) writes the
+//           row tiles and the work items of group g, workgroup 0 publishes counts, offsets and the totals
 //   gather  one wave per token: the row of x is read once with 16-byte accesses and written to its K
 //           destination rows (gather semantics as img_token_drop,
 //           J/engine/nn/layer/dit/kernel/TokenDropKernel.cu:147-160); fp32 layers keep rows contiguous,
@@ -148,10 +150,16 @@ __device__ __forceinline__ int table_entries(int total_mt, int NT, int ks_max = 
 
 // MAXE: experts are limited to 256 per layer by the router kernels.
 #define MAXE 256
+#define RANK_CHUNKS (TOK_TILE_MAX * 64 / 64)  // 64-pair chunks of the largest token tile (K <= 64)
+// FUSED: the workgroup forms the prefix of its token tile over the tiles before it, and the per-expert totals, from
+// the router's histogram rows itself (a single pass: no scan launch in front; used while the histogram is small enough
+// for every workgroup to read all of it); else tile_base / counts come from dispatch_scan_kernel.
+template <bool FUSED>
 __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__restrict__ ids,
+                                                            const int32_t *__restrict__ tile_counts,
                                                             const int32_t *__restrict__ tile_base,
-                                                            const int32_t *__restrict__ counts, int T, int tok_tile, int K,
-                                                            int E, int Es, int bm, int32_t *__restrict__ offsets,
+                                                            int32_t *__restrict__ counts, int n_tiles, int T, int tok_tile,
+                                                            int K, int E, int Es, int bm, int32_t *__restrict__ offsets,
                                                             int32_t *__restrict__ dst, int32_t *__restrict__ dstp,
                                                             int32_t *__restrict__ src_row,
                                                             omega_tile *__restrict__ tiles,
@@ -163,9 +171,61 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     __shared__ int off_s[MAXE + 1];        // logical first row of each expert
     __shared__ int mt_s[MAXE + 64 + 1];    // first row tile of each group (routed, then shared)
     __shared__ int id_s[TOK_TILE_MAX * 64];    // K <= 64
-    const int tid = threadIdx.x, tile = blockIdx.x;
+    __shared__ int base_s[MAXE];           // pairs of each expert in the token tiles before this one
+    __shared__ int tot_s[MAXE];            // pairs of each expert in the whole batch
+    __shared__ int part_s[2][256];
+    __shared__ int ccount[RANK_CHUNKS][MAXE];  // pairs of each expert in each 64-pair chunk of this tile
+    const int tid = threadIdx.x, tile = blockIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t0 = tile * tok_tile;
     const int npairs = min(tok_tile, T - t0) * K;
+    const int nchunks = (npairs + 63) >> 6;
+
+    for (int i = tid; i < npairs; i += 256) id_s[i] = ids[(size_t)t0 * K + i];
+    for (int i = tid; i < nchunks * E; i += 256) ccount[i / E][i % E] = 0;
+    if (FUSED) {
+        // thread (segment s of the tiles, expert e): pairs of e in its tiles, and in those of them before this tile
+        int ES = 1;
+        while (ES < E) ES <<= 1;
+        const int segs = 256 / ES, sg = tid / ES, e = tid % ES;
+        const int per = (n_tiles + segs - 1) / segs;
+        const int b = min(sg * per, n_tiles), en = min(b + per, n_tiles);
+        int before = 0, all = 0;
+        if (e < E) {
+            int t = b;
+            for (; t + 4 <= en; t += 4) {  // four independent loads in flight
+                int c[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) c[u] = tile_counts[(size_t)(t + u) * E + e];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    all += c[u];
+                    before += t + u < tile ? c[u] : 0;
+                }
+            }
+            for (; t < en; ++t) {
+                const int c = tile_counts[(size_t)t * E + e];
+                all += c;
+                before += t < tile ? c : 0;
+            }
+        }
+        part_s[0][tid] = before;
+        part_s[1][tid] = all;
+        __syncthreads();
+        if (tid < E) {
+            int bsum = 0, asum = 0;
+            for (int q = 0; q < segs; ++q) {
+                bsum += part_s[0][q * ES + tid];
+                asum += part_s[1][q * ES + tid];
+            }
+            base_s[tid] = bsum;
+            tot_s[tid] = asum;
+            if (tile == 0) counts[tid] = asum;
+        }
+    } else if (tid < E) {
+        base_s[tid] = tile_base[(size_t)tile * E + tid];
+        tot_s[tid] = counts[tid];
+    }
+    __syncthreads();
 
     // exclusive scans of the E counts and of their tile counts: one wave, 4 experts per lane
     if (tid < 64) {
@@ -173,7 +233,7 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int e = tid * 4 + i;
-            c[i] = e < E ? counts[e] : 0;
+            c[i] = e < E ? tot_s[e] : 0;
             run += c[i];
             runt += (c[i] + bm - 1) / bm;
         }
@@ -198,37 +258,67 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
             for (int s = 0; s <= Es; ++s) mt_s[E + s] = inclt + s * per_shared;
         }
     }
-    for (int i = tid; i < npairs; i += 256) id_s[i] = ids[(size_t)t0 * K + i];
-    __syncthreads();
 
-    for (int i = tid; i < npairs; i += 256) {
-        const int e = id_s[i];
-        int rank = 0;
-        for (int q = 0; q < i; ++q) rank += (id_s[q] == e) ? 1 : 0;
-        rank += tile_base[(size_t)tile * E + e];
+    // Stable rank of every pair among the pairs of its expert.  Within a 64-pair chunk (one wave): the lanes with one
+    // expert find each other by ballot, a lane's rank is the number of them below it; across chunks: per-chunk counts
+    // in LDS.  Each wave takes every fourth chunk.
+    int my_rank[RANK_CHUNKS / 4], my_e[RANK_CHUNKS / 4];
+#pragma unroll
+    for (int cq = 0; cq < RANK_CHUNKS / 4; ++cq) {
+        const int ch = wave + 4 * cq;
+        my_rank[cq] = 0;
+        my_e[cq] = -1;
+        if (ch >= nchunks) continue;  // uniform over the wave
+        const int i = ch * 64 + lane;
+        const bool valid = i < npairs;
+        const int e = valid ? id_s[i] : -1;
+        unsigned long long todo = __ballot(valid), mine = 0;
+        while (todo) {
+            const int leader = __ffsll((long long)todo) - 1;
+            const int le = __builtin_amdgcn_readlane(e, leader);
+            const unsigned long long m = __ballot(e == le);
+            if (e == le) mine = m;
+            todo &= ~m;
+        }
+        if (valid) {
+            const unsigned long long below = mine & ((1ull << lane) - 1ull);
+            my_rank[cq] = __popcll(below);
+            my_e[cq] = e;
+            if (below == 0) ccount[ch][e] = __popcll(mine);  // the lowest lane of each expert of the chunk
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int cq = 0; cq < RANK_CHUNKS / 4; ++cq) {
+        const int ch = wave + 4 * cq, e = my_e[cq];
+        if (ch >= nchunks || e < 0) continue;
+        const int i = ch * 64 + lane;
+        int rank = base_s[e] + my_rank[cq];
+        for (int c2 = 0; c2 < ch; ++c2) rank += ccount[c2][e];
         const int r = off_s[e] + rank;
         dst[(size_t)t0 * K + i] = r;
         dstp[(size_t)t0 * K + i] = mt_s[e] * bm + rank;
         src_row[r] = t0 + i / K;
     }
 
+    const int G = E + Es;
     if (tile == 0) {
         for (int e = tid; e <= E; e += 256) offsets[e] = off_s[e];
-        const int G = E + Es;
-        for (int g = 0; g < G; ++g) {
-            const int rows = g < E ? off_s[g + 1] - off_s[g] : T;
-            const int nm = mt_s[g + 1] - mt_s[g];
-            for (int mt = tid; mt < nm; mt += 256) {
-                omega_tile tl;
-                tl.g = g;
-                tl.row0 = (mt_s[g] + mt) * bm;
-                tl.rows = min(bm, rows - mt * bm);
-                tl.xrow0 = g < E ? -1 : mt * bm;
-                tiles[mt_s[g] + mt] = tl;
-            }
-        }
         if (tid == 0) tile_meta[0] = mt_s[G];
         for (int g = tid; g <= G; g += 256) tile_meta[1 + g] = mt_s[g];
+    }
+    // row-tile list: group g is written by workgroup g (mod grid), like the work-item tables below
+    for (int g = tile; g < G; g += gridDim.x) {
+        const int rows = g < E ? off_s[g + 1] - off_s[g] : T;
+        const int nm = mt_s[g + 1] - mt_s[g];
+        for (int mt = tid; mt < nm; mt += 256) {
+            omega_tile tl;
+            tl.g = g;
+            tl.row0 = (mt_s[g] + mt) * bm;
+            tl.rows = min(bm, rows - mt * bm);
+            tl.xrow0 = g < E ? -1 : mt * bm;
+            tiles[mt_s[g] + mt] = tl;
+        }
     }
 
     // ---- work-item tables of the two grouped products (bf16 layers) ----
@@ -247,7 +337,6 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     // slices of its 32-row blocks (adjacent entries, so that the slices of a tile run side by side on one XCD and share
     // the weight tile in its L2).  Group g is written by workgroup g (mod grid).
     if (desc_up != nullptr || desc_down != nullptr) {
-        const int G = E + Es;
         if (tile == 0 && tid == 0) {
             tile_meta[G + 2] = table_entries(mt_s[G], nt_up);
             tile_meta[G + 3] = table_entries(mt_s[G], nt_down, ks_max_down, kt_down);
@@ -453,18 +542,30 @@ __global__ __launch_bounds__(256) void dispatch_gather_bytes_kernel(const unsign
     }
 }
 
+// Largest histogram (token tiles x experts) for which every rank workgroup sums all of it itself instead of reading
+// the prefix a scan launch left: 64 KiB per workgroup out of the L2.
+#define RANK_FUSED_MAX_CELLS 16384
+
 hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
     const int tok_tile = router_tok_tile(c.E);
     const int n_tiles = ceil_div(T, tok_tile);
-    hipLaunchKernelGGL(dispatch_scan_kernel, dim3(ceil_div(c.E, SCAN_EC)), dim3(256), 0, s, m->tile_counts,
-                       m->tile_base, n_tiles, c.E, m->counts);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(dispatch_rank_kernel, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_base, m->counts, T, tok_tile, c.K,
-                       c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles, m->tile_meta, m->desc_up, c.H / 128, 128,
-                       m->desc_down, c.d / m->down_cols, m->down_cols, m->down_ks_max, c.H / 32);
+    const bool fused = (size_t)n_tiles * c.E <= RANK_FUSED_MAX_CELLS;
+    if (!fused) {
+        hipLaunchKernelGGL(dispatch_scan_kernel, dim3(ceil_div(c.E, SCAN_EC)), dim3(256), 0, s, m->tile_counts,
+                           m->tile_base, n_tiles, c.E, m->counts);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+#define RANK_LAUNCH(F)                                                                                                      \
+    hipLaunchKernelGGL(dispatch_rank_kernel<F>, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_counts, m->tile_base, m->counts, \
+                       n_tiles, T, tok_tile, c.K, c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles,          \
+                       m->tile_meta, m->desc_up, c.H / 128, 128, m->desc_down, c.d / m->down_cols, m->down_cols,             \
+                       m->down_ks_max, c.H / 32)
+    if (fused) RANK_LAUNCH(true);
+    else RANK_LAUNCH(false);
+#undef RANK_LAUNCH
     return hipGetLastError();
 }
 
