@@ -18,7 +18,13 @@
 // FAST mode of bf16 layers with more than 16 experts takes phase 1 to the matrix cores (router_mfma_kernel below).
 #include "common.h"
 
+typedef __attribute__((ext_vector_type(8))) __bf16 rt_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float rt_f32x16;
+
 #define ROUTER_EPT(EP) ((EP) >= 128 ? 4 : (EP) >= 32 ? 2 : 1)
+// MFMA form of the exact sums (bf16 layers with more than 16 experts): a unit = 16 tokens x 64 experts, one
+// v_mfma_f32_16x16x1_4b_f32 per k; a workgroup of 32 tokens has 2 * ceil(EP/64) units, dealt to its 4 waves
+#define ROUTER_MU(EP) ((EP) > 128 ? 2 : 1)
 // token tile and threads per workgroup for EP (padded) experts
 #define ROUTER_TT(EP) ((EP) <= 16 ? 16 : 32)
 #define ROUTER_NTHR(EP) ((EP) <= 8 ? 128 : 256)
@@ -37,10 +43,16 @@ int router_tok_tile(int E) { return E <= 16 ? 16 : 32; }
 // every load is a whole 16-byte vector; rows beyond T or E are redirected to the last valid row (their sums are
 // never used), which keeps the loads free of branches - and with that really asynchronous: a load issued inside
 // a divergent branch makes the compiler wait for all earlier ones first.
-template <int EP, int KC, bool EXACT, bool XBF, bool FAST_IO>
+// MFMA: the sums run on the matrix cores instead (macc; acc is not touched): v_mfma_f32_16x16x1_4b_f32 takes ONE k per
+// instruction - D = C + a*b per element, one product and one addition - so a chain of them over k = 0, 1, 2, ... is
+// the sequential sum, term for term: with bf16 operands every product is exact in fp32 and the addition rounds once,
+// exactly as the fused multiply-add of the vector path does.  A unit of 16 tokens x 64 experts is four 16 x 16 blocks
+// (lane l supplies x[token l % 16][k] and Wg[expert l of the unit][k]); the chain of one unit keeps a SIMD's matrix
+// pipe busy at twice the rate of the vector units, and a lane reads 32 bytes of LDS per 4 k instead of 128.
+template <int EP, int KC, bool EXACT, bool XBF, bool FAST_IO, bool MFMA = false>
 __device__ __forceinline__ void router_sums(const void *__restrict__ x, const void *__restrict__ Wg, int T, int d, int E,
                                             int t0, float (*xs)[KC + 4], float (*ws)[KC + 4],
-                                            float (&acc)[ROUTER_TT(EP) * EP / ROUTER_NTHR(EP)])
+                                            float (&acc)[ROUTER_TT(EP) * EP / ROUTER_NTHR(EP)], rt_f32x16 (&macc)[ROUTER_MU(EP)])
 {
     constexpr int TOK_TILE = ROUTER_TT(EP), NTHR = ROUTER_NTHR(EP);
     constexpr int EPT = ROUTER_EPT(EP);           // experts per thread
@@ -163,7 +175,31 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
             }                                                                          \
         }                                                                              \
     } while (0)
-        if (!wave_live) {
+        if (MFMA) {
+            constexpr int UNITS = 2 * ((EP + 63) / 64), MU = ROUTER_MU(EP);
+            const int lane = tid & 63, wave = tid >> 6;
+            const float *xrow[MU], *wrow[MU];
+#pragma unroll
+            for (int j = 0; j < MU; ++j) {
+                const int u = min(wave + 4 * j, UNITS - 1);  // (waves without a unit do not enter the loop below)
+                xrow[j] = &xs[(u & 1) * 16 + (lane & 15)][0];
+                wrow[j] = &ws[min((u >> 1) * 64 + lane, EP - 1)][0];
+            }
+            if (wave < UNITS) {  // uniform over the wave
+#pragma unroll 4
+                for (int k4 = 0; k4 < KC / 4; ++k4) {  // (beyond d the staged chunk is zero: a +0 term changes nothing)
+#pragma unroll
+                    for (int j = 0; j < MU; ++j) {
+                        if (wave + 4 * j >= UNITS) continue;
+                        const float4 xv = *(const float4 *)(xrow[j] + k4 * 4), wv = *(const float4 *)(wrow[j] + k4 * 4);
+                        macc[j] = __builtin_amdgcn_mfma_f32_16x16x1f32(xv.x, wv.x, macc[j], 0, 0, 0);
+                        macc[j] = __builtin_amdgcn_mfma_f32_16x16x1f32(xv.y, wv.y, macc[j], 0, 0, 0);
+                        macc[j] = __builtin_amdgcn_mfma_f32_16x16x1f32(xv.z, wv.z, macc[j], 0, 0, 0);
+                        macc[j] = __builtin_amdgcn_mfma_f32_16x16x1f32(xv.w, wv.w, macc[j], 0, 0, 0);
+                    }
+                }
+            }
+        } else if (!wave_live) {
             // every token of this wave lies beyond T: it only stages and keeps the barriers
         } else if (FAST_IO || kend == KC) {
             // whole chunk: no exit test inside, so the LDS reads of later steps are issued ahead of the sums
@@ -178,98 +214,96 @@ __device__ __forceinline__ void router_sums(const void *__restrict__ x, const vo
     }
 }
 
-// Phases 2 and 3 for the 32 tokens of one workgroup, from the logits in lg (all 256 threads; lg and hist are complete
-// and visible on entry).  RELAXED (the matrix-core FAST path only, tolerance mode): exponentials in single precision
-// and the softmax sum as a butterfly over the lanes instead of the reference's order - the ordered sum is a chain of
-// EP dependent cross-lane reads per token and dominates that path otherwise.
+// Phases 2 and 3 for the tokens of one workgroup, from the logits in lg (all threads; lg and hist are complete and
+// visible on entry; lg is overwritten).  LPT = NTHR / TOK_TILE lanes (8 or 16) share a token; lane j of them owns the
+// experts j, j + LPT, ...  Softmax in the reference's order (J/engine/gpu/SoftmaxKernel.cu:4-24): the row maximum
+// (any order gives the same value), e = (float)exp((double)(z - max)) written back to LDS, then ONE lane per token adds
+// the E values in expert order - the reference's thread-per-row loop, run for all tokens of the tile side by side - and
+// every lane divides.  Top-k: K rounds; a lane scans its own experts in ascending order with a strict comparison, the
+// LPT lanes combine by a butterfly on (value, index) with "greater value, or equal value and lower index", so ties go
+// to the lowest expert; the winner is masked out.  RELAXED (the matrix-core FAST path, tolerance mode) takes the
+// exponentials in single precision.
 template <int EP, bool RELAXED = false, int TOK_TILE = 32, int NTHR = 256>
 __device__ __forceinline__ void router_select(float (*lg)[EP], int *hist, int t0, int tile, int T, int E, int K, int renorm,
                                               int32_t *__restrict__ ids, float *__restrict__ wout,
                                               int32_t *__restrict__ tile_counts, float *__restrict__ probs_out)
 {
-    constexpr int GS = EP < 64 ? EP : 64;    // lanes that share one token
-    constexpr int VPL = EP / GS;             // experts per lane
+    constexpr int LPT = NTHR / TOK_TILE;            // lanes per token
+    constexpr int VPL = (EP + LPT - 1) / LPT;       // experts per lane
+    constexpr int KPL = (64 + LPT - 1) / LPT;       // slots per lane (K <= 64)
+    static_assert(LPT == 8 || LPT == 16, "a token's lanes lie in one wave");
     const int tid = threadIdx.x;
-    // ---- phase 2: each wave owns 8 tokens; GS lanes share a token ----
-    const int lane = tid & 63, wave = tid >> 6;
-    const int sub = lane % GS, grp = lane / GS;
-    constexpr int TOK_PER_PASS = 64 / GS;
-    constexpr int PASSES = 8 / TOK_PER_PASS;
-    for (int pass = 0; pass < PASSES; ++pass) {
-        const int tt = wave * 8 + pass * TOK_PER_PASS + grp;
-        const int t = t0 + tt;
-        if (t >= T || tt >= TOK_TILE) continue;  // uniform over the GS lanes that exchange data
-        float v[VPL], p[VPL];
-        float mx = -INFINITY;
+    const int tt = tid / LPT, sub = tid % LPT;
+    const int t = t0 + tt;
+    const bool live = t < T;  // uniform over the LPT lanes that exchange data
+    float p[VPL];
+    float mx = -INFINITY;
 #pragma unroll
-        for (int q = 0; q < VPL; ++q) {
-            const int e = sub + q * GS;
-            v[q] = e < E ? lg[tt][e] : -INFINITY;
-            mx = fmaxf(mx, v[q]);
+    for (int q = 0; q < VPL; ++q) {
+        const int e = sub + q * LPT;
+        p[q] = (e < E && e < EP) ? lg[tt][e] : -INFINITY;
+        mx = fmaxf(mx, p[q]);
+    }
+#pragma unroll
+    for (int m = LPT / 2; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, LPT));
+#pragma unroll
+    for (int q = 0; q < VPL; ++q) {
+        const int e = sub + q * LPT;
+        p[q] = (e < E && e < EP) ? (RELAXED ? __expf(p[q] - mx) : (float)exp((double)(p[q] - mx))) : 0.0f;
+        if (e < EP) lg[tt][e] = p[q];
+    }
+    __syncthreads();
+    float s = 0.0f;
+    if (sub == 0 && live)
+        for (int e = 0; e < E; ++e) s = s + lg[tt][e];
+    s = __shfl(s, 0, LPT);
+#pragma unroll
+    for (int q = 0; q < VPL; ++q) {
+        const int e = sub + q * LPT;
+        p[q] = p[q] / s;
+        if (probs_out != nullptr && live && e < E) probs_out[(size_t)t * E + e] = p[q];
+        if (e >= E) p[q] = -1.0f;  // never selected: probabilities are >= 0
+    }
+    // lane `sub` keeps the winners of the rounds j = sub, sub + LPT, ...
+    int myid[KPL];
+    float myw[KPL];
+#pragma unroll
+    for (int u = 0; u < KPL; ++u) { myid[u] = 0; myw[u] = 0.0f; }
+    float rs = 0.0f;  // sum of the selected weights in slot order, the same in all lanes of the token
+    for (int j = 0; j < K; ++j) {
+        float bv = p[0];
+        int bi = sub;
+#pragma unroll
+        for (int q = 1; q < VPL; ++q)
+            if (p[q] > bv) { bv = p[q]; bi = sub + q * LPT; }
+#pragma unroll
+        for (int m = LPT / 2; m >= 1; m >>= 1) {
+            const float ov = __shfl_xor(bv, m, LPT);
+            const int oi = __shfl_xor(bi, m, LPT);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
         }
+        rs = rs + bv;
 #pragma unroll
-        for (int m = GS / 2; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, GS));
+        for (int u = 0; u < KPL; ++u)
+            if (j == sub + u * LPT) { myid[u] = bi; myw[u] = bv; }
 #pragma unroll
-        for (int q = 0; q < VPL; ++q) {
-            const int e = sub + q * GS;
-            p[q] = e < E ? (RELAXED ? __expf(v[q] - mx) : (float)exp((double)(v[q] - mx))) : 0.0f;
-        }
-        float s = 0.0f;
-        if (RELAXED) {
+        for (int q = 0; q < VPL; ++q)
+            if (bi == sub + q * LPT) p[q] = -1.0f;
+    }
 #pragma unroll
-            for (int q = 0; q < VPL; ++q) s = s + p[q];
-#pragma unroll
-            for (int m = GS / 2; m >= 1; m >>= 1) s = s + __shfl_xor(s, m, GS);
-        } else {
-#pragma unroll
-            for (int q = 0; q < VPL; ++q)
-                for (int l = 0; l < GS; ++l) {
-                    const float ev = __shfl(p[q], l, GS);
-                    if (l + q * GS < E) s = s + ev;
-                }
-        }
-#pragma unroll
-        for (int q = 0; q < VPL; ++q) {
-            const int e = sub + q * GS;
-            p[q] = p[q] / s;
-            if (probs_out != nullptr && e < E) probs_out[(size_t)t * E + e] = p[q];
-            if (e >= E) p[q] = -1.0f;  // never selected: probabilities are >= 0
-        }
-        int myid = 0;
-        float myw = 0.0f;
-        for (int j = 0; j < K; ++j) {
-            float bv = p[0];
-            int bi = sub;
-#pragma unroll
-            for (int q = 1; q < VPL; ++q)
-                if (p[q] > bv) { bv = p[q]; bi = sub + q * GS; }
-#pragma unroll
-            for (int m = GS / 2; m >= 1; m >>= 1) {
-                const float ov = __shfl_xor(bv, m, GS);
-                const int oi = __shfl_xor(bi, m, GS);
-                if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-            }
-            if (sub == j) { myid = bi; myw = bv; }
-#pragma unroll
-            for (int q = 0; q < VPL; ++q)
-                if (bi == sub + q * GS) p[q] = -1.0f;
-        }
-        if (renorm) {
-            float rs = 0.0f;
-            for (int j = 0; j < K; ++j) rs = rs + __shfl(myw, j, GS);
-            myw = myw / rs;
-        }
-        if (sub < K) {
-            ids[(size_t)t * K + sub] = myid;
-            wout[(size_t)t * K + sub] = myw;
-            atomicAdd(&hist[myid], 1);
+    for (int u = 0; u < KPL; ++u) {
+        const int j = sub + u * LPT;
+        if (j < K && live) {
+            ids[(size_t)t * K + j] = myid[u];
+            wout[(size_t)t * K + j] = renorm ? myw[u] / rs : myw[u];
+            atomicAdd(&hist[myid[u]], 1);
         }
     }
     __syncthreads();
     for (int e = tid; e < E; e += NTHR) tile_counts[(size_t)tile * E + e] = hist[e];
 }
 
-template <int EP, int KC, bool EXACT>
+template <int EP, int KC, bool EXACT, bool MFMA = false>
 __global__ __launch_bounds__(ROUTER_NTHR(EP)) void router_kernel(const void *__restrict__ x, int dtype, const void *__restrict__ Wg,
                                                      const float *__restrict__ bg, int T, int d, int E, int K,
                                                      int renorm, int32_t *__restrict__ ids,
@@ -301,16 +335,48 @@ __global__ __launch_bounds__(ROUTER_NTHR(EP)) void router_kernel(const void *__r
 #pragma unroll
     for (int i = 0; i < NT * EPT; ++i) acc[i] = 0.0f;
 
+    rt_f32x16 macc[ROUTER_MU(EP)];
+#pragma unroll
+    for (int j = 0; j < ROUTER_MU(EP); ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) macc[j][r] = 0.0f;
+
     const bool fast_io = (d % KC == 0) && (((uintptr_t)x | (uintptr_t)Wg) % 16 == 0);
-    if (dtype == OMEGA_DTYPE_BF16) {
-        if (fast_io) router_sums<EP, KC, EXACT, true, true>(x, Wg, T, d, E, t0, xs, ws, acc);
-        else router_sums<EP, KC, EXACT, true, false>(x, Wg, T, d, E, t0, xs, ws, acc);
+    if (MFMA) {  // bf16 layers only (the launcher sees to it)
+        if (fast_io) router_sums<EP, KC, EXACT, true, true, true>(x, Wg, T, d, E, t0, xs, ws, acc, macc);
+        else router_sums<EP, KC, EXACT, true, false, true>(x, Wg, T, d, E, t0, xs, ws, acc, macc);
+    } else if (dtype == OMEGA_DTYPE_BF16) {
+        if (fast_io) router_sums<EP, KC, EXACT, true, true>(x, Wg, T, d, E, t0, xs, ws, acc, macc);
+        else router_sums<EP, KC, EXACT, true, false>(x, Wg, T, d, E, t0, xs, ws, acc, macc);
     } else {
-        if (fast_io) router_sums<EP, KC, EXACT, false, true>(x, Wg, T, d, E, t0, xs, ws, acc);
-        else router_sums<EP, KC, EXACT, false, false>(x, Wg, T, d, E, t0, xs, ws, acc);
+        if (fast_io) router_sums<EP, KC, EXACT, false, true>(x, Wg, T, d, E, t0, xs, ws, acc, macc);
+        else router_sums<EP, KC, EXACT, false, false>(x, Wg, T, d, E, t0, xs, ws, acc, macc);
+    }
+    if (MFMA) {
+        // unit u = (token half u % 2, expert group u / 2); lane: expert l % 16 of block b, register 4*b + r -> token 4*(l/16) + r
+        constexpr int UNITS = 2 * ((EP + 63) / 64);
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int j = 0; j < ROUTER_MU(EP); ++j) {
+            const int u = wave + 4 * j;
+            if (u >= UNITS) continue;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int e = (u >> 1) * 64 + 16 * b + (lane & 15);
+                if (e >= EP) continue;
+                const float bias = (bg != nullptr && e < E) ? bg[e] : 0.0f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int tt = (u & 1) * 16 + 4 * (lane >> 4) + r;
+                    const float z = bg != nullptr ? macc[j][4 * b + r] + bias : macc[j][4 * b + r];
+                    lg[tt][e] = z;
+                    if (logits_out != nullptr && t0 + tt < T && e < E) logits_out[(size_t)(t0 + tt) * E + e] = z;
+                }
+            }
+        }
     }
 #pragma unroll
-    for (int x_ = 0; x_ < EPT; ++x_) {
+    for (int x_ = 0; x_ < (MFMA ? 0 : EPT); ++x_) {
         const int e = e1 + x_ * EL;
         const float b = (bg != nullptr && e < E) ? bg[e] : 0.0f;
 #pragma unroll
@@ -332,9 +398,6 @@ __global__ __launch_bounds__(ROUTER_NTHR(EP)) void router_kernel(const void *__r
 // waves split the k range (partial sums are added in a fixed order through LDS) or, from 128 experts on, the blocks.  Operand fragments come straight from memory (16 bytes per lane; the 64 bytes a lane pair
 // needs of a row per 32 k are fetched by consecutive loads, so every line is read once): the kernel moves x once
 // (Wg stays in the L2) and has almost no arithmetic, it lives on loads in flight.
-typedef __attribute__((ext_vector_type(8))) __bf16 rt_bf16x8;
-typedef __attribute__((ext_vector_type(16))) float rt_f32x16;
-
 template <int EP>
 __global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ Wg,
                                                           const float *__restrict__ bg, int T, int d, int E, int K,
@@ -439,9 +502,14 @@ hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits
 #undef ROUTER_MFMA_LAUNCH
         return hipGetLastError();
     }
+    // exact sums of bf16 layers with more than 16 experts: on the matrix cores, one k per instruction
+    const bool exact_mfma = exact && c.dtype == OMEGA_DTYPE_BF16 && c.E > 16;
 #define ROUTER_LAUNCH(EPV, KCV)                                                                                    \
     do {                                                                                                           \
-        if (exact)                                                                                                 \
+        if (exact_mfma)                                                                                            \
+            hipLaunchKernelGGL((router_kernel<EPV, KCV, true, (EPV > 16)>), dim3(tiles), dim3(ROUTER_NTHR(EPV)), 0, s, x, c.dtype, m->Wg, bg, \
+                               T, c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out, probs_out);   \
+        else if (exact)                                                                                            \
             hipLaunchKernelGGL((router_kernel<EPV, KCV, true>), dim3(tiles), dim3(ROUTER_NTHR(EPV)), 0, s, x, c.dtype, m->Wg, bg, \
                                T, c.d, c.E, c.K, c.renorm, m->ids, m->w, m->tile_counts, logits_out, probs_out);   \
         else                                                                                                       \
