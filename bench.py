@@ -25,9 +25,24 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3
 PEAK_HBM_GBPS = 8000.0
 
-# HBM traffic per launch of the dominant kernel from the committed rocprofv3 --pmc runs
-# (profiles/experts_bf16_c2_mixtral_pmc.txt): FETCH_SIZE + WRITE_SIZE in bytes, scaled by the copy-kernel factor.
-TRAFFIC_BYTES = {"c2_mixtral": 4.98e9}
+
+
+def profiled_traffic(cfg_name):
+    """HBM / fabric bytes per launch of the dominant kernel (the up product) from the tracked rocprofv3 --pmc summary of
+    this workload, profiles/experts_bf16_<workload>_pmc.txt: the line `traffic_bytes_per_launch up <bytes>`
+    (FETCH_SIZE x copy-kernel factor + WRITE_SIZE).  The counters cannot be read inside a timed run, so the figure
+    belongs to the commit the summary was made at; None when there is no summary for the workload."""
+    path = os.path.join(ROOT, "profiles", f"experts_bf16_{cfg_name}_pmc.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == "up":
+                    return float(parts[2]), os.path.relpath(path, ROOT)
+    except OSError:
+        pass
+    return None, None
+
 
 
 def main():
@@ -104,6 +119,11 @@ def main():
     router_bytes = cfg.T * cfg.d * b + cfg.E * cfg.d * b + cfg.P * 8
     dispatch_bytes = 2 * cfg.P * cfg.d * b + cfg.P * 12
     combine_bytes = cfg.P * cfg.d * b + cfg.T * cfg.d * b + cfg.P * 8
+    # bytes these kernels cannot avoid moving as the path is specified (not the algorithmic figures above): the gather
+    # reads every token row once and writes it K times (+ once per batch for the shared experts' packed copy); the
+    # combine reads the expert outputs as the fp32 rows the composition keeps them in
+    dispatch_real = cfg.T * cfg.d * b + cfg.P * cfg.d * b + (cfg.T * cfg.d * b if cfg.Es else 0) + cfg.P * 12
+    combine_real = rows * cfg.d * 4 + cfg.T * cfg.d * b + cfg.P * 8
     gather_ms = layer.time_stage(L.STAGE_GATHER, x, cfg.T, warmup=2, iters=20)
     # block form (out = x + layer(rmsnorm(x)), the widening next to the path): whole call and its pre-norm kernel
     outb = P.DeviceBuffer(ctx, (cfg.T, cfg.d), cfg.dtype)
@@ -167,6 +187,7 @@ def main():
         gbuf.free()
         dxb.free()
 
+    traffic, traffic_src = profiled_traffic(C.CONFIGS[a.config].name if not a.override else "")
     res = {
         "metric": "MoE-layer fwd tokens/s (Mixtral shape, bf16); MFMA util %; dispatch GB/s",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -178,7 +199,7 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "experts_bf16_kernel<0> (up): a = silu(xg W1^T) * (xg W3^T)",
                      "achieved": up_tflops, "peak": peak, "unit": "TFLOP/s", "frac": up_tflops / peak,
                      "algorithmic_flops_per_launch": up_flops, "avg_launch_ms": stage_ms["experts_up"],
-                     "traffic": TRAFFIC_BYTES.get(cfg.name),
+                     "traffic": traffic, "traffic_source": traffic_src,
                      "mfma_only_probe": probe},
         "block_form": {"what": "out = x + layer(rmsnorm(x)) in one call (omega_moe_forward_block)", "ms_per_step": block_ms,
                        "tokens/s": cfg.T / (block_ms * 1e-3), "prenorm_kernel_ms": rms_ms},
@@ -190,10 +211,12 @@ def main():
             "router": {"GB/s": router_bytes / (stage_ms["router"] * 1e-3) / 1e9, "frac_hbm": router_bytes / (stage_ms["router"] * 1e-3) / 1e9 / PEAK_HBM_GBPS},
             "dispatch": {"GB/s": dispatch_bytes / (stage_ms["dispatch"] * 1e-3) / 1e9,
                          "frac_hbm": dispatch_bytes / (stage_ms["dispatch"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                         "frac_hbm_real_traffic": dispatch_real / (stage_ms["dispatch"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                          "gather_only_ms": gather_ms, "gather_only_GB/s": 2 * cfg.P * cfg.d * b / (gather_ms * 1e-3) / 1e9,
                          "index_only_ms": index_ms},
             "combine": {"GB/s": combine_bytes / (stage_ms["combine"] * 1e-3) / 1e9,
-                        "frac_hbm": combine_bytes / (stage_ms["combine"] * 1e-3) / 1e9 / PEAK_HBM_GBPS},
+                        "frac_hbm": combine_bytes / (stage_ms["combine"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                        "frac_hbm_real_traffic": combine_real / (stage_ms["combine"] * 1e-3) / 1e9 / PEAK_HBM_GBPS},
         },
     }
 
@@ -219,8 +242,25 @@ def main():
             p = O.softmax(O.gate(xh, Wg, bg))
             ids, w = O.topk(p, cfg.K, cfg.renorm)
             counts, offsets, dst, src = O.dispatch(ids, cfg.E)
-            tok = np.unique(np.linspace(0, cfg.T - 1, 16).astype(np.int32))
-            ref = O.moe_tokens(xh, ids, w, W1, W3, W2, cfg.E, cfg.Es, tok, bf16=bf)
+            # a token of every row tile of every expert (first row of the tile, last row of the expert), so that the
+            # sample touches every row tile the grouped products schedule, plus 16 evenly spaced tokens
+            bm = 256 if bf else 64
+            pick = set(np.linspace(0, cfg.T - 1, 16).astype(np.int64).tolist())
+            for e in range(cfg.E):
+                n, l0 = int(counts[e]), int(offsets[e])
+                if n:
+                    Mg, nblk = -(-n // bm), -(-n // 32)
+                    qb, nhi = divmod(nblk, Mg)
+                    pick.update(int(src[l0 + 32 * (mt * qb + min(mt, nhi))]) for mt in range(Mg))
+                    pick.add(int(src[l0 + n - 1]))
+            if cfg.Es:
+                pick.update(range(0, cfg.T, bm))
+            tok = np.array(sorted(pick), np.int32)
+            from concurrent.futures import ThreadPoolExecutor
+            parts = [p for p in np.array_split(tok, min(8, len(tok))) if len(p)]
+            with ThreadPoolExecutor(len(parts)) as ex:
+                ref = np.concatenate(list(ex.map(
+                    lambda part: O.moe_tokens(xh, ids, w, W1, W3, W2, cfg.E, cfg.Es, part, bf16=bf), parts)))
             res["parity"] = {
                 "ids_bit_exact": bool(np.array_equal(r["ids"], ids)), "weights_bit_exact": bool(np.array_equal(r["w"], w)),
                 "counts_bit_exact": bool(np.array_equal(r["counts"], counts)),

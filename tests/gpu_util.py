@@ -55,15 +55,16 @@ def assert_routing_bit_exact(r, ref):
 def row_tile_tokens(r, cfg, T, bm=256):
     """One token per row tile of every group (its first row; for a group's last tile also its last row), so that a
     token sample touches every row tile the grouped products schedule.  Row tiles of a group are its 32-row blocks
-    dealt evenly to ceil(rows / bm) tiles."""
+    dealt evenly to ceil(rows / bm) tiles, the taller tiles first."""
     toks = set()
     for e in range(cfg.E):
         n, l0 = int(r["counts"][e]), int(r["offsets"][e])
         if n == 0:
             continue
         Mg, nblk = -(-n // bm), -(-n // 32)
+        qb, nhi = divmod(nblk, Mg)                   # the first nhi row tiles hold qb + 1 blocks of 32 rows, the others qb
         for mt in range(Mg):
-            toks.add(int(r["src_row"][l0 + 32 * ((mt * nblk) // Mg)]))
+            toks.add(int(r["src_row"][l0 + 32 * (mt * qb + min(mt, nhi))]))
         toks.add(int(r["src_row"][l0 + n - 1]))
     if cfg.Es > 0:                                   # shared experts: row t of a shared group is token t
         toks.update(range(0, T, bm))

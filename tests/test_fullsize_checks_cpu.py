@@ -98,7 +98,8 @@ def test_row_tile_tokens_touch_every_row_tile(case):
     for e in range(cfg.E):
         n, l0 = int(r["counts"][e]), int(r["offsets"][e])
         Mg, nblk = -(-n // 256), -(-n // 32)
+        qb, nhi = divmod(nblk, Mg)
         for mt in range(Mg):
-            lo, hi = l0 + 32 * ((mt * nblk) // Mg), l0 + min(32 * (((mt + 1) * nblk) // Mg), n)
+            lo, hi = l0 + 32 * (mt * qb + min(mt, nhi)), l0 + min(32 * ((mt + 1) * qb + min(mt + 1, nhi)), n)
             assert any(lo <= q < hi for q in touched), (e, mt)
     assert 0 in tok and cfg.T - 1 in tok                # shared experts: first and last row tile
