@@ -155,6 +155,9 @@ struct omega_moe {
 int router_tok_tile(int E);
 #define ROUTER_TOK_TILE_MAX 32
 
+// Size of the last-level (memory-side) cache of the device: streams larger than this are written / read around it.
+#define OMEGA_LLC_BYTES ((size_t)256 << 20)
+
 __host__ __device__ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 int omega_set_error(omega_ctx *ctx, int status, const char *what, hipError_t herr, const char *file, int line);
