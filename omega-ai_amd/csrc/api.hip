@@ -73,6 +73,7 @@ int omega_hip_ctx_create(int device, omega_ctx **out)
     c->num_cus = prop.multiProcessorCount;
     e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = experts_bf16_init();
+    if (e == hipSuccess) e = router_init();
     if (e != hipSuccess) {
         delete c;
         return omega_set_error(nullptr, OMEGA_ERR_HIP, "ctx_create: stream / kernel attribute setup", e, __FILE__, __LINE__);

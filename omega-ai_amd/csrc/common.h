@@ -213,6 +213,7 @@ hipError_t launch_unpack_rows(void *dst_rowmajor, const void *src_packed, int R,
 int experts_bf16_tile_m(const omega_moe *m, int T);
 int experts_f32_tile_m(void);
 hipError_t experts_bf16_init(void);
+hipError_t router_init(void);  // kernel attributes of the router (LDS beyond 64 KiB), once per device
 
 // ---- device helpers ----
 #ifdef __HIPCC__

@@ -16,6 +16,10 @@
 //           value and lower index" so ties go to the lowest expert; winners are masked out.
 //  phase 3  LDS-atomic histogram of the selected experts, flushed as row `tile` of tile_counts[.,E].
 // FAST mode of bf16 layers with more than 16 experts takes phase 1 to the matrix cores (router_mfma_kernel below).
+// bf16 layers with at most 16 experts and at most one tile per compute unit take router_pipe_kernel: phase 1 is then as
+// long as one chain of d dependent multiply-adds, and separate staging waves keep everything else out of the waves that
+// run the chains (Mixtral shape: 4096 tokens 33 -> 29 us, 64 tokens 27 -> 22 us; of the 22, 11 are the chain itself at
+// 6.25 clocks a term and 6.5 are launch, the first loads and phases 2 and 3).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 rt_bf16x8;
@@ -485,6 +489,140 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(const bf16_t *__restri
     router_select<EP, true>(lg, hist, t0, tile, T, E, K, renorm, ids, wout, tile_counts, probs_out);
 }
 
+// Batches of at most one 16-token tile per compute unit, bf16, at most 16 experts, d a multiple of 512: the whole
+// kernel is as long as ONE chain of d dependent multiply-adds (about 6 clocks a term on a SIMD that has no second wave
+// to fill them), so everything else is taken out of the waves that run the chains.  The workgroup has two kinds of
+// waves: 16*EP/64 sum waves, one lane per (token, expert), that only read LDS and add; and two staging waves that
+// carry the NEXT 512-k chunk of x and Wg from memory to a second LDS buffer as fp32 while the current one is summed.
+// One barrier per chunk, executed by every wave of both kinds (B_c: chunk c is staged, and chunk c-1 is summed - so
+// its buffer may take chunk c+1).  The terms are the exact fp32 products of bf16 operands, added in k order by
+// fused multiply-adds: the same bits as the separate multiply and add of the sequential sum, in either router mode.
+#define RP_KC 512
+#define RP_LDW (RP_KC + 4)
+#define RP_STAGERS 128
+template <int EP>
+__global__ __launch_bounds__(16 * EP + RP_STAGERS) void router_pipe_kernel(
+    const bf16_t *__restrict__ x, const bf16_t *__restrict__ Wg, const float *__restrict__ bg, int T, int d, int E, int K,
+    int renorm, int32_t *__restrict__ ids, float *__restrict__ wout, int32_t *__restrict__ tile_counts,
+    float *__restrict__ logits_out, float *__restrict__ probs_out)
+{
+    constexpr int TT = 16, CT = 16 * EP, ST = RP_STAGERS, KC = RP_KC, LDW = RP_LDW;
+    extern __shared__ __attribute__((aligned(16))) float rp_smem[];
+    float(*xs)[TT][LDW] = (float(*)[TT][LDW])rp_smem;                  // [2][TT][LDW]
+    float(*ws)[EP][LDW] = (float(*)[EP][LDW])(rp_smem + 2 * TT * LDW);  // [2][EP][LDW]
+    __shared__ float lg[TT][EP];
+    __shared__ int hist[EP];
+    const int tid = threadIdx.x, tile = blockIdx.x, t0 = tile * TT;
+    if (tid < EP) hist[tid] = 0;
+    const int nch = d / KC;
+    if (tid >= CT) {
+        // staging wave: thread st carries 8 consecutive k (16 bytes of bf16) of one row per load
+        const int st = tid - CT;
+        constexpr int XCH = TT * (KC / 8) / ST, WCH = EP * (KC / 8) / ST;
+        static_assert(TT * (KC / 8) % ST == 0 && EP * (KC / 8) % ST == 0, "whole vectors per staging thread");
+        // (a second chunk of loads in flight gained nothing: the sum waves, bound by their LDS reads, set the pace)
+        uint4 xr[XCH], wr[WCH];
+        auto fetch = [&](int k0) {
+#pragma unroll
+            for (int c = 0; c < XCH; ++c) {
+                const int idx = st + c * ST;
+                xr[c] = *(const uint4 *)(x + (size_t)min(t0 + idx / (KC / 8), T - 1) * d + k0 + (idx % (KC / 8)) * 8);
+            }
+#pragma unroll
+            for (int c = 0; c < WCH; ++c) {
+                const int idx = st + c * ST;
+                wr[c] = *(const uint4 *)(Wg + (size_t)min(idx / (KC / 8), E - 1) * d + k0 + (idx % (KC / 8)) * 8);
+            }
+        };
+        auto widen = [&](const uint4 &v, float *dst) {
+            *(float4 *)dst = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                                         __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+            *(float4 *)(dst + 4) = make_float4(__uint_as_float(v.z << 16), __uint_as_float(v.z & 0xffff0000u),
+                                               __uint_as_float(v.w << 16), __uint_as_float(v.w & 0xffff0000u));
+        };
+        fetch(0);
+        for (int c = 0; c < nch; ++c) {
+            const int b = c & 1;
+#pragma unroll
+            for (int q = 0; q < XCH; ++q) {
+                const int idx = st + q * ST;
+                widen(xr[q], &xs[b][idx / (KC / 8)][(idx % (KC / 8)) * 8]);
+            }
+#pragma unroll
+            for (int q = 0; q < WCH; ++q) {
+                const int idx = st + q * ST;
+                widen(wr[q], &ws[b][idx / (KC / 8)][(idx % (KC / 8)) * 8]);
+            }
+            if (c + 1 < nch) fetch((c + 1) * KC);
+            __syncthreads();  // B_c
+        }
+    } else {
+        const int e1 = tid % EP, tg = tid / EP;
+        // a wave whose lowest token is past the end of the batch forms no sum; it keeps the barriers
+        const bool wave_live = t0 + (tid & ~63) / EP < T;
+        float a_ = 0.0f;
+        for (int c = 0; c < nch; ++c) {
+            __syncthreads();  // B_c
+            if (!wave_live) continue;
+            const float4 *wp = (const float4 *)&ws[c & 1][e1][0], *xp = (const float4 *)&xs[c & 1][tg][0];
+            float4 wa[8], xa[8], wb[8], xb[8];
+#define ROUTER_LD(W, X, g)                                    \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j)             \
+    {                                                         \
+        W[j] = wp[(g) * 8 + j];                               \
+        X[j] = xp[(g) * 8 + j];                               \
+    }
+#define ROUTER_FM(W, X)                                       \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j)             \
+    {                                                         \
+        a_ = fmaf(X[j].x, W[j].x, a_);                        \
+        a_ = fmaf(X[j].y, W[j].y, a_);                        \
+        a_ = fmaf(X[j].z, W[j].z, a_);                        \
+        a_ = fmaf(X[j].w, W[j].w, a_);                        \
+    }
+            // the LDS reads of the next 32 k are in flight while the terms of the current 32 are added (the fences
+            // keep the reads where they are written: ahead of the other set's terms)
+            ROUTER_LD(wa, xa, 0)
+            for (int g = 0; g < KC / 32; g += 2) {
+                __builtin_amdgcn_sched_barrier(0);
+                ROUTER_LD(wb, xb, g + 1)
+                __builtin_amdgcn_sched_barrier(0);
+                ROUTER_FM(wa, xa)
+                __builtin_amdgcn_sched_barrier(0);
+                if (g + 2 < KC / 32) {
+                    ROUTER_LD(wa, xa, g + 2)
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                ROUTER_FM(wb, xb)
+            }
+#undef ROUTER_LD
+#undef ROUTER_FM
+        }
+        const float z = (bg != nullptr && e1 < E) ? a_ + bg[e1] : a_;
+        lg[tg][e1] = z;
+        if (logits_out != nullptr && t0 + tg < T && e1 < E) logits_out[(size_t)(t0 + tg) * E + e1] = z;
+    }
+    __syncthreads();
+    if (tid < CT) {
+        router_select<EP, false, TT, CT>(lg, hist, t0, tile, T, E, K, renorm, ids, wout, tile_counts, probs_out);
+    } else {
+        __syncthreads();  // the staging waves keep the two barriers of the selection
+        __syncthreads();
+    }
+}
+
+int router_pipe_smem_bytes(int EP) { return 2 * (16 + EP) * RP_LDW * (int)sizeof(float); }
+
+hipError_t router_init(void)
+{
+    hipError_t e = hipFuncSetAttribute((const void *)router_pipe_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       router_pipe_smem_bytes(8));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute((const void *)router_pipe_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                router_pipe_smem_bytes(16));
+    return e;
+}
+
 hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
@@ -500,6 +638,19 @@ hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits
         else if (c.E <= 128) ROUTER_MFMA_LAUNCH(128);
         else ROUTER_MFMA_LAUNCH(256);
 #undef ROUTER_MFMA_LAUNCH
+        return hipGetLastError();
+    }
+    // at most 16 experts, bf16, at most one tile per compute unit: chains fed by staging waves (either mode: same bits)
+    if (c.dtype == OMEGA_DTYPE_BF16 && c.E <= 16 && tiles <= m->ctx->num_cus && c.d % RP_KC == 0 &&
+        (((uintptr_t)x | (uintptr_t)m->Wg) % 16) == 0) {
+        if (c.E <= 8)
+            hipLaunchKernelGGL(router_pipe_kernel<8>, dim3(tiles), dim3(16 * 8 + RP_STAGERS), router_pipe_smem_bytes(8), s,
+                               (const bf16_t *)x, (const bf16_t *)m->Wg, bg, T, c.d, c.E, c.K, c.renorm, m->ids, m->w,
+                               m->tile_counts, logits_out, probs_out);
+        else
+            hipLaunchKernelGGL(router_pipe_kernel<16>, dim3(tiles), dim3(16 * 16 + RP_STAGERS), router_pipe_smem_bytes(16), s,
+                               (const bf16_t *)x, (const bf16_t *)m->Wg, bg, T, c.d, c.E, c.K, c.renorm, m->ids, m->w,
+                               m->tile_counts, logits_out, probs_out);
         return hipGetLastError();
     }
     // exact sums of bf16 layers with more than 16 experts: on the matrix cores, one k per instruction

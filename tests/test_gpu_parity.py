@@ -167,6 +167,33 @@ def test_bf16_small_batches_slice_the_down_product(G, T, d, H, E, K, Es):
     layer.close()
 
 
+@pytest.mark.parametrize("T,d,E,K,zipf", [
+    (37, 1536, 8, 2, 0.0),     # ragged tile whose second wave holds no token, three chunks of 512 k (odd count)
+    (16, 512, 5, 2, 1.1),      # fewer experts than lanes across them, gate bias, a single chunk
+    (130, 1024, 12, 3, 0.7),   # 12 of 16 expert lanes, bias, two tokens in the last tile
+    (4096, 512, 16, 4, 0.0),   # one tile per compute unit: the largest batch of the small-batch kernel
+    (4112, 512, 8, 2, 0.0),    # one tile more: the same layer through the general kernel
+])
+def test_bf16_small_batch_router_bit_exact(G, T, d, E, K, zipf):
+    """bf16 layers with at most 16 experts and at most one 16-token tile per compute unit route through a kernel of
+    their own (staging waves feed the waves that form the sums): logits, probabilities and the routing against the
+    oracle, bit for bit, and the fast router mode gives the same bits (its terms are exact products either way)."""
+    cfg = scaled(C.CONFIGS["c2_mixtral"], T=T, d=d, H=256, E=E, K=K, zipf_bias=zipf)
+    layer, x, out, r, ref, inp = G.run_case(cfg, seed=9000 + T)
+    G.assert_routing_bit_exact(r, ref)
+    lg, p = layer.router_probs(x, T)
+    assert np.array_equal(lg.view(np.uint32), ref["logits"].view(np.uint32))
+    assert np.array_equal(p.view(np.uint32), ref["p"].view(np.uint32))
+    assert N.rel_l2(out, ref["out"]) <= BF16_TOL
+    layer.close()
+    fast = G.build_layer(cfg, inp, "fast")
+    fast.forward(x)
+    lgf, pf = fast.router_probs(x, T)
+    assert np.array_equal(lgf.view(np.uint32), lg.view(np.uint32))
+    assert np.array_equal(pf.view(np.uint32), p.view(np.uint32))
+    fast.close()
+
+
 def test_bf16_fast_router_agrees(G):
     cfg = scaled(C.CONFIGS["c2_mixtral"], T=512, d=512, H=1024)
     layer, x, out, r, ref, inp = G.run_case(cfg, seed=4242, router_mode="fast")
