@@ -492,9 +492,10 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
 // One wave per token; 16-byte chunks; up to 8 chunks in flight per lane.  PACKED: destination rows are in the
 // packed tile image (chunk index = 4*kstep + c); when xs != nullptr, the token is also copied to row t of xs.
 // The first n_sched workgroups build the product kernels' queues instead (see schedule_queues).
-// NT: the rows are written with non-temporal stores.  Worth 23 % when the gathered buffer is larger than the last-level
-// cache of 256 MiB (16384 tokens x 8 slots x 2048: 0.204 -> 0.158 ms, and the products that follow gain 2 %); a buffer
-// that fits is better left to it (8192 x 6 x 2048: the launch alone gains, the forward pass loses).
+// NT: the rows are written with non-temporal stores, from half the last-level cache (256 MiB) of gathered rows on.
+// 16384 tokens x 8 slots x 2048 (512 MiB): launch 0.204 -> 0.158 ms and the products that follow gain 2 %;
+// 8192 x 6 x 2048 (192 MiB): launch 0.090 -> 0.073 ms, forward pass 1.332 -> 1.321 ms; 4096 x 2 x 4096 (64 MiB): launch
+// -2.5 us, up product +3 us, the forward pass the same - left to the cache.
 template <bool PACKED, bool NT>
 __global__ __launch_bounds__(256) void dispatch_gather_kernel(const uint4 *__restrict__ x, const int32_t *__restrict__ dstp,
                                                               int T, int K, int chunks_per_row,
@@ -586,7 +587,7 @@ hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipS
         const int G = c.E + c.Es;
         sched_args sa = {{m->desc_up, m->desc_down, nullptr}, {m->wq_up, m->wq_down, nullptr}, {G + 2, G + 3, 0}, {0, 0, 0},
                          m->tile_meta, m->n_wg};
-        if ((size_t)T * c.K * row_bytes > OMEGA_LLC_BYTES)
+        if ((size_t)T * c.K * row_bytes > OMEGA_LLC_BYTES / 2)
             hipLaunchKernelGGL((dispatch_gather_kernel<true, true>), dim3(ceil_div(T, 4) + SCHED_WGS), dim3(256), 0, s, (const uint4 *)x,
                                m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs, SCHED_WGS, sa);
         else
