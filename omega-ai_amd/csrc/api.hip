@@ -400,7 +400,7 @@ int omega_moe_create(omega_ctx *ctx, const omega_moe_config *cfg, omega_moe **ou
     alloc0(&m->W2, wsz);
     alloc0((void **)&m->counts, (size_t)c.E * 4);
     alloc0((void **)&m->offsets, (size_t)(c.E + 1) * 4);
-    alloc0((void **)&m->tile_meta, (size_t)(m->G + 8) * 4);
+    alloc0((void **)&m->tile_meta, (size_t)(m->G + 10) * 4);
     if (e == hipSuccess) e = hipEventCreate(&m->ev0);
     if (e == hipSuccess) e = hipEventCreate(&m->ev1);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -592,9 +592,13 @@ static int stage_dispatch(omega_moe *m, const void *x, int T)
         const bool small = m->max_m_tiles * (c.d / 256) <= m->n_wg / 2;
         m->down_ks_max = min_tiles * (c.d / 256) <= m->n_wg / 2 && c.H >= 512 ? 8 : 1;
         m->down_cols = small && m->down_ks_max == 1 ? 128 : 256;
-        // slices x tiles never exceed n_wg, so all partial results together are smaller than n_wg tiles of 256 x 256
-        if (m->down_ks_max > 1 && !m->y_slabs)
-            OMEGA_HIP_CHECK(m->ctx, hipMalloc((void **)&m->y_slabs, (size_t)m->n_wg * 256 * 256 * 4));
+        // A large batch whose last round of output tiles would occupy at most half of the compute units: those tiles
+        // are cut into up to 4 k slices (rather than row slices, which stream the whole weight tile for a quarter of
+        // the rows and are bound by that stream), if a slice keeps at least 64 k steps.
+        m->down_tail_ks = (m->down_ks_max == 1 && !small && c.H >= 2 * 64 * 32) ? 4 : 1;
+        // sliced entries never exceed 256, so there are at most 256 partial results, each a tile of 256 x 256
+        if ((m->down_ks_max > 1 || m->down_tail_ks > 1) && !m->y_slabs)
+            OMEGA_HIP_CHECK(m->ctx, hipMalloc((void **)&m->y_slabs, (size_t)256 * 256 * 256 * 4));
     }
     if (m->max_m_tiles > m->tiles_cap) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: workspace too small for this T");
     OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));

@@ -77,7 +77,8 @@ struct omega_moe {
     omega_tile *tiles = nullptr;     // [max_m_tiles]
     int32_t *tile_meta = nullptr;    // [0] = number of row tiles; [1+g] = first row tile of group g (G+1 entries);
                                      // [G+2], [G+3] = entries of desc_up, desc_down; [G+4..G+6] = entries of the
-                                     // backward tables desc_da, desc_w2, desc_w13
+                                     // backward tables desc_da, desc_w2, desc_w13; [G+7] = k slices per tile of a
+                                     // small batch; [G+8], [G+9] = first k-sliced entry of desc_down and their number
     omega_tile_desc *desc_up = nullptr;    // bf16: [tiles_cap * H/128] output tiles of the up product
     omega_tile_desc *desc_down = nullptr;  // bf16: [tiles_cap * d/256] output tiles of the down product
     // bf16: the same work items as one queue per workgroup of the (persistent) product kernels, entry q of workgroup w
@@ -87,8 +88,9 @@ struct omega_moe {
     // columns of a work item of the down product: 256, or 128 when 256-column tiles would leave at least half of the
     // compute units without an item (a few tokens: the product is bound by streaming W2, which every unit must share)
     int down_cols = 256;
-    int down_ks_max = 1;             // > 1: the down table of this batch may hold k slices (small batches)
-    float *y_slabs = nullptr;        // their partial results 1 .. KS-1, each laid out like the rows of y in use
+    int down_ks_max = 1;             // > 1: the down table of this batch may hold k slices of every tile (small batches)
+    int down_tail_ks = 1;            // > 1: the last tiles of the down table may be cut into up to this many k slices
+    float *y_slabs = nullptr;        // partial results of the k slices: 256 tiles of 256 x 256 floats, one per sliced entry
     void *xg = nullptr;              // [rows_cap,d]  gathered tokens (bf16: packed tile image, see pack.h)
     void *xs = nullptr;              // bf16 with shared experts: packed copy of x, [ceil(T/bm)*bm,d]
     void *a = nullptr;               // [rows_cap,H]  (bf16: packed tile image)
@@ -195,7 +197,7 @@ hipError_t launch_transpose_groups(const omega_moe *m, const void *src, const vo
 hipError_t launch_transpose_images(const void *src, int R, int cols, void *dst, int KTd, int k0, int n, size_t src_stride,
                                    size_t dst_stride, hipStream_t s);
 // products of the matrix-core kernel (experts_bf16.hip describes each)
-enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4, MODE_UPREC = 5, MODE_DOWNK = 6 };
+enum { MODE_UP = 0, MODE_DOWN = 1, MODE_UPRAW = 2, MODE_DA = 3, MODE_WGRAD = 4, MODE_UPREC = 5 };
 hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, const void *Aalt, const void *Wa, const void *Wb,
                                void *Cout, void *Aux1, void *Aux2, const omega_tile_desc *wq, int N, int Kd, hipStream_t s);
 hipError_t launch_update_bf16(const omega_moe *m, float *master, float lr, int init, hipStream_t s);
@@ -213,6 +215,7 @@ hipError_t launch_unpack_rows(void *dst_rowmajor, const void *src_packed, int R,
 int experts_bf16_tile_m(const omega_moe *m, int T);
 int experts_f32_tile_m(void);
 hipError_t experts_bf16_init(void);
+hipError_t launch_down_slab_reduce(const omega_moe *m, float *y, hipStream_t s);  // y += partial results of k-sliced items
 hipError_t router_init(void);  // kernel attributes of the router (LDS beyond 64 KiB), once per device
 
 // ---- device helpers ----

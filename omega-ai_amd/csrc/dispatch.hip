@@ -65,18 +65,32 @@ __device__ __forceinline__ int table_k_slices(int Nt, int ks_max, int KT)
     return max(1, min(min(ks_max, 256 / Nt), KT / 8));
 }
 
+// K slices of the last r tiles of a large launch (r = Nt mod 256 <= 128: they would leave at least half of the compute
+// units idle): as many as fill the units, at most tail_ks, each at least 64 k steps long; 1 = none (row slices instead).
+// Row slices stream the whole weight tile for a quarter of the rows and are bound by that stream; k slices are not, but
+// their partial results have to be added up behind the product.  4096 tokens, 8 experts, k = 14336 (448 steps, 64 of 576
+// tiles in 4 slices): product 0.834 -> 0.784 ms, adding up 0.020 ms; k = 1408 (44 steps, 2 slices): 0.369 -> 0.386 ms,
+// hence the minimum length.
+__device__ __forceinline__ int table_tail_k_slices(int Nt, int tail_ks, int KT)
+{
+    const int r = Nt % 256;
+    if (tail_ks <= 1 || r == 0 || r > 128) return 1;
+    return max(1, min(min(tail_ks, 256 / r), KT / 64));
+}
+
 // Row tiles of one group that run side by side on an XCD (see dispatch_rank_kernel): a group with more row tiles than
 // this is cut into row blocks of about equal size, each of which walks all column tiles.
 #define OMEGA_ROW_BLOCK_MAX 8
 
 __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ desc, int NT, int ncols, int g, int rows,
                                                   int Mg, int mt0, int total_mt, int bm, bool shared, int ks_max = 1,
-                                                  int KT = 0)
+                                                  int KT = 0, int tail_ks = 1)
 {
     if (desc == nullptr) return;
     const int Nt = total_mt * NT, r = Nt % 256;
     const int KS = table_k_slices(Nt, ks_max, KT);
-    const int S = (r == 0 || r > 128 || KS > 1) ? 1 : min(4, 256 / r);
+    const int TKS = KS > 1 ? 1 : table_tail_k_slices(Nt, tail_ks, KT);
+    const int S = (r == 0 || r > 128 || KS > 1 || TKS > 1) ? 1 : min(4, 256 / r);
     // the group's rows are dealt evenly, in blocks of 32, to its Mg row tiles (instead of full tiles and a ragged last
     // one): the same number of tiles and of MFMA blocks, but tiles of nearly one cost.  (Equal tiles in units of 16 rows -
     // every tile the same number of MFMA blocks, the last one of each half empty - cut the L2 miss traffic of the up
@@ -108,14 +122,14 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
         //  products that keep or read h1 / h3 block records)
         dsc.kt0 = (mt0 + mt) * 8;
         if (KS > 1) {
-            // slice ks of KS (a_rg = KS, kt0 = ks) adds its part of the k range into partial result ks; adjacent
-            // entries, so the slices of a tile run on one XCD and share its rows
+            // slice ks of KS (a_rg = KS, kt0 = ks, xrow0 = number of the sliced entry = of its partial result) runs over
+            // its part of the k range; adjacent entries, so the slices of a tile run on one XCD and share its rows
             dsc.row0 = mt0 * bm + tfirst;
             dsc.rows = trows;
-            dsc.xrow0 = shared ? tfirst : -1;
             dsc.a_rg = KS;
             for (int ks = 0; ks < KS; ++ks) {
                 dsc.kt0 = ks;
+                dsc.xrow0 = at * KS + ks;
                 desc[at * KS + ks] = dsc;
             }
         } else if (at < Nt - r) {
@@ -123,6 +137,17 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
             dsc.rows = trows;
             dsc.xrow0 = shared ? tfirst : -1;
             desc[at] = dsc;
+        } else if (TKS > 1) {
+            // one of the last r tiles of a large launch, as TKS k slices (fields as above)
+            const int ti = at - (Nt - r);
+            dsc.row0 = mt0 * bm + tfirst;
+            dsc.rows = trows;
+            dsc.a_rg = TKS;
+            for (int ks = 0; ks < TKS; ++ks) {
+                dsc.kt0 = ks;
+                dsc.xrow0 = ti * TKS + ks;
+                desc[Nt - r + ti * TKS + ks] = dsc;
+            }
         } else {
             const int tb = (trows + 31) >> 5;  // the tile's 32-row blocks, dealt evenly to the S slices
             const int rec0 = dsc.kt0;
@@ -139,11 +164,13 @@ __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ 
 }
 
 // entries of a table whose launch has total_mt row tiles and NT column tiles (with the last tiles sliced)
-__device__ __forceinline__ int table_entries(int total_mt, int NT, int ks_max = 1, int KT = 0)
+__device__ __forceinline__ int table_entries(int total_mt, int NT, int ks_max = 1, int KT = 0, int tail_ks = 1)
 {
     const int Nt = total_mt * NT, r = Nt % 256;
     const int KS = table_k_slices(Nt, ks_max, KT);
     if (KS > 1) return Nt * KS;
+    const int TKS = table_tail_k_slices(Nt, tail_ks, KT);
+    if (TKS > 1) return Nt - r + r * TKS;
     const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
     return Nt - r + r * S;
 }
@@ -166,7 +193,7 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
                                                             int32_t *__restrict__ tile_meta,
                                                             omega_tile_desc *__restrict__ desc_up, int nt_up, int ncols_up,
                                                             omega_tile_desc *__restrict__ desc_down, int nt_down,
-                                                            int ncols_down, int ks_max_down, int kt_down)
+                                                            int ncols_down, int ks_max_down, int kt_down, int tail_ks_down)
 {
     __shared__ int off_s[MAXE + 1];        // logical first row of each expert
     __shared__ int mt_s[MAXE + 64 + 1];    // first row tile of each group (routed, then shared)
@@ -339,14 +366,19 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     if (desc_up != nullptr || desc_down != nullptr) {
         if (tile == 0 && tid == 0) {
             tile_meta[G + 2] = table_entries(mt_s[G], nt_up);
-            tile_meta[G + 3] = table_entries(mt_s[G], nt_down, ks_max_down, kt_down);
-            tile_meta[G + 7] = table_k_slices(mt_s[G] * nt_down, ks_max_down, kt_down);  // partial results of the down product
+            tile_meta[G + 3] = table_entries(mt_s[G], nt_down, ks_max_down, kt_down, tail_ks_down);
+            const int Nt = mt_s[G] * nt_down, KS = table_k_slices(Nt, ks_max_down, kt_down);
+            const int TKS = KS > 1 ? 1 : table_tail_k_slices(Nt, tail_ks_down, kt_down);
+            tile_meta[G + 7] = KS;
+            // the k-sliced entries of the down table (their partial results are added up behind the product)
+            tile_meta[G + 8] = KS > 1 ? 0 : Nt - Nt % 256;
+            tile_meta[G + 9] = KS > 1 ? Nt * KS : TKS > 1 ? (Nt % 256) * TKS : 0;
         }
         for (int g = tile; g < G; g += gridDim.x) {
             const int rows = g < E ? off_s[g + 1] - off_s[g] : T;
             const int Mg = mt_s[g + 1] - mt_s[g];
             write_group_items(desc_up, nt_up, ncols_up, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E);
-            write_group_items(desc_down, nt_down, ncols_down, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E, ks_max_down, kt_down);
+            write_group_items(desc_down, nt_down, ncols_down, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E, ks_max_down, kt_down, tail_ks_down);
         }
     }
 }
@@ -572,7 +604,7 @@ hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t 
     hipLaunchKernelGGL(dispatch_rank_kernel<F>, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_counts, m->tile_base, m->counts, \
                        n_tiles, T, tok_tile, c.K, c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles,          \
                        m->tile_meta, m->desc_up, c.H / 128, 128, m->desc_down, c.d / m->down_cols, m->down_cols,             \
-                       m->down_ks_max, c.H / 32)
+                       m->down_ks_max, c.H / 32, m->down_tail_ks)
     if (fused) RANK_LAUNCH(true);
     else RANK_LAUNCH(false);
 #undef RANK_LAUNCH

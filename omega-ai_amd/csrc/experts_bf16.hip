@@ -37,7 +37,7 @@
 
 // What one instantiation of the product kernel computes (tile shape, operand order, epilogue):
 //   UP     tile 256 x (128 of Wa + 128 of Wb), silu(h1)*h3 -> packed bf16 a
-//   DOWN   tile 256 x 256, fp32 row-major output
+//   DOWN   tile 256 x 256, fp32 row-major output; an item may be a k slice of a tile (see make_ctx)
 //   UPRAW  as UP, but h1 and h3 are stored as they sit in the accumulators (Cout = h1, Aux1 = h3): one 4 KiB record
 //          per 32x32 MFMA block, [row block][column block][register 0..15][lane 0..63]
 //   UPREC  UP and UPRAW in one: the forward pass of a layer in training mode (a -> Cout, h1 -> Aux1, h3 -> Aux2)
@@ -47,9 +47,9 @@
 //          whose K axis is the experts' rows; the item names its operand row groups, first k step and k steps
 //          (a_rg, b_rg, kt0, xrow0); fp32 row-major output, row0 = expert * M + first row
 #define FUSED_TILE(M) ((M) == MODE_UP || (M) == MODE_UPRAW || (M) == MODE_UPREC)
-#define PLAIN_DOWN(M) ((M) == MODE_DOWN || (M) == MODE_DOWNK)
+#define PLAIN_DOWN(M) ((M) == MODE_DOWN)
 #define SWAPPED(M) (!PLAIN_DOWN(M) && (M) != MODE_WGRAD)
-#define ITEM_K(M) ((M) == MODE_WGRAD || (M) == MODE_DOWNK)  // the k range belongs to the item, not to the launch
+#define ITEM_K(M) ((M) == MODE_WGRAD || PLAIN_DOWN(M))  // the k range belongs to the item, not to the launch
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -113,7 +113,7 @@ struct TileCtx {
     int row0, rows, n0;
     int kt;                   // k steps of the item
     int half;                 // plain 256-column products: the item covers the first 128 columns only
-    int slab;                 // MODE_DOWNK: which partial result the item writes
+    int slab;                 // down products: 0 = the item writes the output, > 0 = partial result `slab` of those behind Aux1
     int rec0;                 // products that write or read h1 / h3 block records: record of the item's first 32-row block
 };
 
@@ -130,9 +130,10 @@ __device__ __forceinline__ uint64_t uniform_u64(uint64_t v)
     return ((uint64_t)hi << 32) | lo;
 }
 
+// slices: the launch has room for partial results (Aux1), so items that are k slices run as such
 template <int MODE>
 __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa,
-                                            const bf16_t *Wb, int N, int Kd, int wave, int lane)
+                                            const bf16_t *Wb, int N, int Kd, int wave, int lane, bool slices)
 {
     constexpr bool FUSED = FUSED_TILE(MODE);
     TileCtx c;
@@ -159,17 +160,22 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
     c.slab = 0;
     c.rec0 = d.kt0;
     c.half = FUSED ? 0 : d.b_rg;
-    // k slices (tables of small batches, items with a_rg = KS > 1 and kt0 = ks): MODE_DOWNK runs slice ks over its own
-    // part of the k range; a launch that knows nothing of partial results (MODE_DOWN) computes the whole range in the
-    // item of slice 0 and only keeps the other slices' workgroups in step (no rows: loads and barriers, no results)
+    // k slices of a down product (items with a_rg = KS > 1, kt0 = ks, xrow0 = number of the partial result: every tile of
+    // a small batch, or the last tiles of a launch that would leave most compute units idle): slice ks runs over its own
+    // part of the k range; slice 0 writes the output, the others partial results that down_slab_reduce_kernel adds to
+    // it.  A launch without room for partial results computes the whole range in the item of slice 0 and only keeps
+    // the other slices' workgroups in step (no rows: loads and barriers, no results).
     size_t k0 = 0;
-    if (MODE == MODE_DOWNK && d.a_rg > 1) {
-        const int first = (d.kt0 * KT) / d.a_rg;  // even parts: every slice has at least KT / KS >= 8 steps
-        c.kt = ((d.kt0 + 1) * KT) / d.a_rg - first;
-        c.slab = d.kt0;
-        k0 = (size_t)first * 8192;
+    if (PLAIN_DOWN(MODE) && d.a_rg > 1) {
+        if (slices) {
+            const int first = (d.kt0 * KT) / d.a_rg;  // even parts: every slice has at least KT / KS >= 8 steps
+            c.kt = ((d.kt0 + 1) * KT) / d.a_rg - first;
+            c.slab = d.kt0 > 0 ? d.xrow0 : 0;
+            k0 = (size_t)first * 8192;
+        } else if (d.kt0 > 0) {
+            c.rows = 0;
+        }
     }
-    if (MODE == MODE_DOWN && d.a_rg > 1 && d.kt0 > 0) c.rows = 0;
     c.A = uniform_ptr(((!PLAIN_DOWN(MODE) && Ax != nullptr && d.xrow0 >= 0)
                            ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
                            : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes) + k0);
@@ -194,16 +200,13 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
 
 // direct load n (0..3) of k step `kstep` of a work item into ring stage `stage`: n -> (operand, row group) =
 // (n & 1 ? B : A, n >> 1)
-// MASKED: A blocks without valid rows move 16 bytes (every product but the k-sliced one of small batches, whose items
-// are bound by the weight stream and whose kernel has no registers to spare)
-#define LOADS_MASKED(M) ((M) != MODE_DOWNK)
-template <bool MASKED, bool WNT = false>
+// A blocks without valid rows move 16 bytes (a_mask0 / a_mask1).
+template <bool WNT = false>
 __device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, uint32_t blk_off, int stage, int kstep, int n)
 {
     const uint32_t sb = lds_wave + stage * STAGE_BYTES;
     const uint32_t kb = (uint32_t)kstep * 8192u;
-    if ((n & 1) == 0 && MASKED) dma16_masked(c.A, kb + ((n >> 1) ? c.a_off1 : c.a_off0), sb + (n >> 1) * 8192, (n >> 1) ? c.a_mask1 : c.a_mask0);
-    else if ((n & 1) == 0) dma16(c.A, kb + ((n >> 1) ? c.a_off1 : c.a_off0), sb + (n >> 1) * 8192);
+    if ((n & 1) == 0) dma16_masked(c.A, kb + ((n >> 1) ? c.a_off1 : c.a_off0), sb + (n >> 1) * 8192, (n >> 1) ? c.a_mask1 : c.a_mask0);
     else if (WNT) dma16_nt((n >> 1) == 0 ? c.B0 : c.B1, kb + blk_off, sb + TILE_BYTES + (n >> 1) * 8192);
     else dma16((n >> 1) == 0 ? c.B0 : c.B1, kb + blk_off, sb + TILE_BYTES + (n >> 1) * 8192);
 }
@@ -235,10 +238,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     ctx.half = __builtin_amdgcn_readfirstlane(ctx_in.half);
     ctx.slab = __builtin_amdgcn_readfirstlane(ctx_in.slab);
     ctx.rec0 = __builtin_amdgcn_readfirstlane(ctx_in.rec0);
-    if (LOADS_MASKED(MODE)) {
-        ctx.a_mask0 = uniform_u64(ctx_in.a_mask0);
-        ctx.a_mask1 = uniform_u64(ctx_in.a_mask1);
-    }
+    ctx.a_mask0 = uniform_u64(ctx_in.a_mask0);
+    ctx.a_mask1 = uniform_u64(ctx_in.a_mask1);
     int cur = __builtin_amdgcn_readfirstlane(cur_io);
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -250,8 +251,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 // load n of virtual k step v: steps beyond this item's last belong to the next item
 #define ISSUE_V(stage, v, n)                                                              \
     do {                                                                                  \
-        if ((v) < KT) issue_load<LOADS_MASKED(MODE), WNT>(ctx, lds_wave, blk_off, stage, v, n);                    \
-        else if (has_next) issue_load<LOADS_MASKED(MODE), WNT>(nx, lds_wave, blk_off, stage, (v) - KT, n);          \
+        if ((v) < KT) issue_load<WNT>(ctx, lds_wave, blk_off, stage, v, n);                    \
+        else if (has_next) issue_load<WNT>(nx, lds_wave, blk_off, stage, (v) - KT, n);          \
     } while (0)
 
     // ---- MFMA operand addressing ----
@@ -319,7 +320,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         {                                                                                                   \
             if ((i & 1) == 0) {                                                                             \
                 if (GEN) ISSUE_V(prv, kt - 1 + NSTAGE, 2 + (i >> 1));                                       \
-                else issue_load<LOADS_MASKED(MODE), WNT>(ctx, lds_wave, blk_off, prv, kt - 1 + NSTAGE, 2 + (i >> 1));                \
+                else issue_load<WNT>(ctx, lds_wave, blk_off, prv, kt - 1 + NSTAGE, 2 + (i >> 1));                \
             }                                                                                               \
             MFMA2(af0, bf0, i);                                                                             \
         }                                                                                                   \
@@ -333,7 +334,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         {                                                                                                   \
             if ((i & 1) == 0) {                                                                             \
                 if (GEN) ISSUE_V(cur, kt + NSTAGE, i >> 1);                                                 \
-                else issue_load<LOADS_MASKED(MODE), WNT>(ctx, lds_wave, blk_off, cur, kt + NSTAGE, i >> 1);                          \
+                else issue_load<WNT>(ctx, lds_wave, blk_off, cur, kt + NSTAGE, i >> 1);                          \
             }                                                                                               \
             MFMA2(af1, bf1, i);                                                                             \
         }                                                                                                   \
@@ -342,7 +343,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 
     int kt = 0;
     for (; kt < KT - NSTAGE; ++kt) K_STEP(false);
-    nx = make_ctx<MODE>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
+    nx = make_ctx<MODE>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr);
     for (; kt < KT; ++kt) K_STEP(true);
 #undef K_STEP
     cur_io = cur;
@@ -429,11 +430,13 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
             }
         }
     } else if ((PLAIN_DOWN(MODE) || MODE == MODE_WGRAD) && !(ctx.half && wn >= 2)) {
-        // MODE_DOWNK: slice 0 writes the output itself, slice s > 0 partial result s - 1 of those behind Aux1, each laid
-        // out like the rows of the output that are in use (Aux2[0] row tiles)
-        float *Cbase = (float *)Cout;
-        if (MODE == MODE_DOWNK && ctx.slab > 0)
-            Cbase = (float *)Aux1 + (size_t)(ctx.slab - 1) * ((size_t)((const int32_t *)Aux2)[0] * BM * N);
+        // a k slice other than the first writes partial result ctx.slab of those behind Aux1: a tile of BM x 256 of its own
+        float *Cbase = PLAIN_DOWN(MODE) ? (float *)Cout + (size_t)ctx.row0 * N + ctx.n0 : (float *)Cout;
+        int ld = N;
+        if (PLAIN_DOWN(MODE) && ctx.slab > 0) {
+            Cbase = (float *)Aux1 + (size_t)ctx.slab * (BM * 256);
+            ld = 256;
+        }
         // lane: column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
@@ -443,7 +446,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
                 if (row >= ctx.rows) continue;
                 // (32 lanes x 4 bytes = one 128-byte line per store; 16-byte stores of a transposed accumulator layout
                 //  write 32-byte pieces of 32 different lines and were 8 % slower on short-K shapes)
-                float *out = Cbase + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l32;
+                float *out = PLAIN_DOWN(MODE) ? Cbase + (size_t)row * ld + wn * 64 + l32
+                                              : Cbase + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l32;
 #pragma unroll
                 for (int j = 0; j < 2; ++j)  // (non-temporal stores of the weight gradients were 10 % slower)
                     if (PLAIN_DOWN(MODE) || ctx.n0 + wn * 64 + j * 32 < N) out[j * 32] = acc[i][j][r];
@@ -470,7 +474,7 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
 
     omega_tile_desc d = wq[wg];
     if (d.rows <= 0) return;
-    TileCtx cur_ctx = make_ctx<MODE>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane);
+    TileCtx cur_ctx = make_ctx<MODE>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr);
     {
         // first item: k steps 0..NSTAGE-2 and the first half of step NSTAGE-1 into stages 0..NSTAGE-1
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -478,10 +482,10 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
         const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
         for (int st = 0; st < NSTAGE - 1; ++st) {
 #pragma unroll
-            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<LOADS_MASKED(MODE), WNT>(cur_ctx, lds_wave, blk_off, st, st, n);
+            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<WNT>(cur_ctx, lds_wave, blk_off, st, st, n);
         }
-        issue_load<LOADS_MASKED(MODE), WNT>(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 0);
-        issue_load<LOADS_MASKED(MODE), WNT>(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 1);
+        issue_load<WNT>(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 0);
+        issue_load<WNT>(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 1);
         asm volatile("s_waitcnt vmcnt(14)" ::: "memory");  // all but steps 1.. : LOADS_PER_STEP * (NSTAGE - 2) + 2
         __syncthreads();
     }
@@ -506,27 +510,56 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
     }
 }
 
-// y += partial results 1 .. KS-1 of a k-sliced down product, in that order; KS comes from the table builder
-// (tile_meta[ks_slot]).  Workgroup (t, c): the valid rows of row tile t, columns c*1024 .. (16 bytes per lane and trip).
+// y += the partial results of the k-sliced items of a down product, in slice order.  The sliced items are the
+// tile_meta[meta_slot + 1] table entries from entry tile_meta[meta_slot] on (slices of a tile adjacent, slice 0 first);
+// partial result i belongs to the i-th of them and is a tile of BM x 256 floats.  Workgroup (i, j): rows 32 j .. of the
+// tile whose slice 0 is sliced entry i (one workgroup per tile moved 1.3 MB alone and took 40 us for 64 tiles).
 __global__ __launch_bounds__(256) void down_slab_reduce_kernel(float *__restrict__ y, const float *__restrict__ slabs,
-                                                               const omega_tile *__restrict__ tiles,
-                                                               const int32_t *__restrict__ tile_meta, int ks_slot, int d)
+                                                               const omega_tile_desc *__restrict__ desc,
+                                                               const int32_t *__restrict__ tile_meta, int meta_slot, int d)
 {
-    const int KS = tile_meta[ks_slot];
-    if (KS <= 1 || (int)blockIdx.x >= tile_meta[0]) return;
-    const size_t slab_floats = (size_t)tile_meta[0] * BM * d;
-    const omega_tile tl = tiles[blockIdx.x];
-    const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
-    if (c >= d) return;
-    for (int r = 0; r < tl.rows; ++r) {
-        const size_t o = (size_t)(tl.row0 + r) * d + c;
-        float4 v = *(const float4 *)(y + o);
-        for (int s = 0; s < KS - 1; ++s) {
-            const float4 u = *(const float4 *)(slabs + (size_t)s * slab_floats + o);
-            v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
+    const int first = tile_meta[meta_slot], n = tile_meta[meta_slot + 1], i = blockIdx.x;
+    if (i >= n) return;
+    const omega_tile_desc e = desc[first + i];
+    if (e.a_rg <= 1 || e.kt0 != 0) return;
+    const int c = (threadIdx.x & 63) * 4;
+    const int rend = min(e.rows, (int)(blockIdx.y + 1) * 32);
+    for (int r0 = blockIdx.y * 32 + (threadIdx.x >> 6); r0 < rend; r0 += 8) {
+        // two rows per trip: up to 8 independent 16-byte loads in flight per thread
+        const int r1 = r0 + 4;
+        const bool two = r1 < rend;
+        float *o0 = y + (size_t)(e.row0 + r0) * d + e.n0 + c, *o1 = y + (size_t)(e.row0 + (two ? r1 : r0)) * d + e.n0 + c;
+        float4 v0 = *(const float4 *)o0, v1 = *(const float4 *)o1;
+        float4 u0[3], u1[3];
+#pragma unroll
+        for (int s = 1; s < 4; ++s) {
+            const int ss = min(s, e.a_rg - 1);
+            u0[s - 1] = *(const float4 *)(slabs + (size_t)(i + ss) * (BM * 256) + r0 * 256 + c);
+            u1[s - 1] = *(const float4 *)(slabs + (size_t)(i + ss) * (BM * 256) + (two ? r1 : r0) * 256 + c);
         }
-        *(float4 *)(y + o) = v;
+#pragma unroll
+        for (int s = 1; s < 4; ++s) {
+            if (s < e.a_rg) {
+                v0.x += u0[s - 1].x; v0.y += u0[s - 1].y; v0.z += u0[s - 1].z; v0.w += u0[s - 1].w;
+                v1.x += u1[s - 1].x; v1.y += u1[s - 1].y; v1.z += u1[s - 1].z; v1.w += u1[s - 1].w;
+            }
+        }
+        for (int s = 4; s < e.a_rg; ++s) {  // (small batches: up to 8 slices)
+            const float4 w0 = *(const float4 *)(slabs + (size_t)(i + s) * (BM * 256) + r0 * 256 + c);
+            const float4 w1 = *(const float4 *)(slabs + (size_t)(i + s) * (BM * 256) + (two ? r1 : r0) * 256 + c);
+            v0.x += w0.x; v0.y += w0.y; v0.z += w0.z; v0.w += w0.w;
+            v1.x += w1.x; v1.y += w1.y; v1.z += w1.z; v1.w += w1.w;
+        }
+        *(float4 *)o0 = v0;
+        if (two) *(float4 *)o1 = v1;
     }
+}
+
+hipError_t launch_down_slab_reduce(const omega_moe *m, float *y, hipStream_t s)
+{
+    hipLaunchKernelGGL(down_slab_reduce_kernel, dim3(256, BM / 32), dim3(256), 0, s, y, (const float *)m->y_slabs, m->desc_down, m->tile_meta,
+                       m->G + 8, m->cfg.d);
+    return hipGetLastError();
 }
 
 hipError_t experts_bf16_init(void)
@@ -534,8 +567,7 @@ hipError_t experts_bf16_init(void)
     const void *fns[] = {(const void *)experts_bf16_kernel<MODE_UP>, (const void *)experts_bf16_kernel<MODE_DOWN>,
                          (const void *)experts_bf16_kernel<MODE_UPRAW>, (const void *)experts_bf16_kernel<MODE_DA>,
                          (const void *)experts_bf16_kernel<MODE_WGRAD>, (const void *)experts_bf16_kernel<MODE_UPREC>,
-                         (const void *)experts_bf16_kernel<MODE_DOWNK>, (const void *)experts_bf16_kernel<MODE_UP, true>,
-                         (const void *)experts_bf16_kernel<MODE_DOWN, true>, (const void *)experts_bf16_kernel<MODE_DOWNK, true>};
+                         (const void *)experts_bf16_kernel<MODE_UP, true>, (const void *)experts_bf16_kernel<MODE_DOWN, true>};
     for (const void *f : fns) {
         hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
         if (e != hipSuccess) return e;
@@ -568,29 +600,23 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
             hipLaunchKernelGGL(experts_bf16_kernel<MODE_UP>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
                                (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
                                (void *)nullptr, m->wq_up, c.H, c.d);
-    } else if (m->down_ks_max > 1) {
-        // small batch: the table may hold k slices; their partial results are added into y right behind the product
-        if (wnt)
-            hipLaunchKernelGGL((experts_bf16_kernel<MODE_DOWNK, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
-                               (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y,
-                               (void *)m->y_slabs, (void *)m->tile_meta, m->wq_down, c.d, c.H);
-        else
-            hipLaunchKernelGGL(experts_bf16_kernel<MODE_DOWNK>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
-                               (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y,
-                               (void *)m->y_slabs, (void *)m->tile_meta, m->wq_down, c.d, c.H);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(down_slab_reduce_kernel, dim3(m->max_m_tiles, ceil_div(c.d, 1024)), dim3(256), 0, s, m->y,
-                           (const float *)m->y_slabs, m->tiles, m->tile_meta, m->G + 7, c.d);
     } else {
+        // the table may hold k slices (every tile of a small batch, or the last tiles of a large one): their partial
+        // results go to y_slabs and are added into y right behind the product
+        void *slabs = (m->down_ks_max > 1 || m->down_tail_ks > 1) ? (void *)m->y_slabs : nullptr;
         if (wnt)
             hipLaunchKernelGGL((experts_bf16_kernel<MODE_DOWN, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
                                (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y,
-                               (void *)nullptr, (void *)nullptr, m->wq_down, c.d, c.H);
+                               slabs, (void *)nullptr, m->wq_down, c.d, c.H);
         else
             hipLaunchKernelGGL(experts_bf16_kernel<MODE_DOWN>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
                                (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y,
-                               (void *)nullptr, (void *)nullptr, m->wq_down, c.d, c.H);
+                               slabs, (void *)nullptr, m->wq_down, c.d, c.H);
+        if (slabs != nullptr) {
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+            return launch_down_slab_reduce(m, m->y, s);
+        }
     }
     return hipGetLastError();
 }
@@ -610,7 +636,6 @@ hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, cons
         case MODE_DA: LAUNCH(MODE_DA); break;
         case MODE_WGRAD: LAUNCH(MODE_WGRAD); break;
         case MODE_UPREC: LAUNCH(MODE_UPREC); break;
-        case MODE_DOWNK: LAUNCH(MODE_DOWNK); break;
         default: return hipErrorInvalidValue;
     }
 #undef LAUNCH
