@@ -1,4 +1,5 @@
-// Grouped expert SwiGLU products in bf16 on the CDNA4 matrix cores (v_mfma_f32_32x32x16_bf16, fp32 accumulate).
+// Grouped expert SwiGLU products in bf16 on the CDNA4 matrix cores (v_mfma_f32_16x16x32_bf16, fp32 accumulate; four of
+// them per 32x32 block and 32-k step: measured 3.5 % faster than one v_mfma_f32_32x32x16_bf16 pair at the same LDS traffic).
 //   up    a[r,h] = silu(xg[r,:].W1g[h,:]) * (xg[r,:].W3g[h,:])   -> bf16      (one pass over xg for both weights)
 //   down  y[r,c] = a[r,:].W2g[c,:]                                -> fp32
 // (J/engine/nn/layer/llama/LlamaMLPLayer.java:117-130; y = x W^T with W [out,in], J/engine/nn/layer/FullyLayer.java:181,235.)
@@ -52,7 +53,7 @@
 #define ITEM_K(M) ((M) == MODE_WGRAD || PLAIN_DOWN(M))  // the k range belongs to the item, not to the launch
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 #define BM 256
 #define BK 32
@@ -256,53 +257,66 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     } while (0)
 
     // ---- MFMA operand addressing ----
-    // Row (2i + wm)*32 + l32 of A, row j*128 + wn*32 + l32 (up: block 0 = 32 columns of W1, block 1 = the same 32
-    // columns of W3) or wn*64 + j*32 + l32 (down) of B.  The chunk swizzle depends on the row only through l32
-    // (rows differ by multiples of 32), so one swizzled k offset per operand serves every block and the blocks are
-    // constant byte offsets.
-    // (An item may start 16 rows into a 32-row unit of the packed image: the swizzle of the A rows follows the
-    //  physical row, i.e. l32 with bit 4 flipped.)
-    const int l32 = lane & 31, lhi = lane >> 5;
-    const int sw = swz(l32), swa = swz(l32 ^ (MODE == MODE_WGRAD ? 0 : (ctx.row0 & 16)));
+    // Row (2i + wm)*32 + 16 rh + l16 of A, row j*128 + wn*32 + 16 ch + l16 (up: block 0 = 32 columns of W1, block 1 = the
+    // same 32 columns of W3) or wn*64 + j*32 + 16 ch + l16 (down) of B.  The chunk swizzle depends on the row through
+    // l16 and bit 4 only (rows differ by multiples of 32 otherwise), so one swizzled offset per half serves every block
+    // and the blocks are constant byte offsets.  (An item may start 16 rows into a 32-row unit of the packed image: the
+    // swizzle of the A rows follows the physical row, i.e. bit 4 flipped.)
+    // Fragments of v_mfma_f32_16x16x32_bf16: 16 rows x 32 k = one 1 KiB block of the tile image; lane l supplies row
+    // l % 16, chunk l / 16.  rh / ch = which 16-row half of a 32-row block of A / 32-column block of B.
+    const int l16 = lane & 15, lq = lane >> 4;
     uint32_t pa[2], pb[2];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-        pa[ks] = (uint32_t)(wm * 32 + l32) * (BK * 2) + ((uint32_t)((ks * 2 + lhi) ^ swa) << 4);
-        pb[ks] = TILE_BYTES + (uint32_t)((FUSED ? wn * 32 : wn * 64) + l32) * (BK * 2) + ((uint32_t)((ks * 2 + lhi) ^ sw) << 4);
+    for (int h = 0; h < 2; ++h) {
+        const int par_a = MODE == MODE_WGRAD ? h : (h ^ ((ctx.row0 >> 4) & 1));  // bit 4 of the physical row
+        pa[h] = (uint32_t)(wm * 32 + 16 * h + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | (par_a << 4))) << 4);
+        pb[h] = TILE_BYTES + (uint32_t)((FUSED ? wn * 32 : wn * 64) + 16 * h + l16) * (BK * 2) +
+                ((uint32_t)(lq ^ swz(l16 | (h << 4))) << 4);
     }
     constexpr uint32_t A_BLK = 64 * BK * 2, B_BLK = (FUSED ? 128 : 32) * BK * 2;
-#define READ_FRAGS(AF, BF, stage, ks)                                                                       \
+// the rh-th 16-row halves of this wave's row blocks
+#define READ_A(AF, stage, rh)                                                                               \
     do {                                                                                                    \
         if (NBLK > 0) {                                                                                     \
             const unsigned char *sp = smem + (stage) * STAGE_BYTES;                                          \
             _Pragma("unroll") for (int i = 0; i < NB; ++i)                                                   \
-                AF[i] = *(const bf16x8_t *)(sp + pa[ks] + i * A_BLK);                                        \
-            _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                    \
-                BF[j] = *(const bf16x8_t *)(sp + pb[ks] + j * B_BLK);                                        \
+                AF[i] = *(const bf16x8_t *)(sp + pa[rh] + i * A_BLK);                                        \
         }                                                                                                   \
     } while (0)
-// the two MFMAs of row block i.  The up product feeds the weights as the first operand, so that a lane ends
-// up with 4 consecutive output columns of one row (8 bytes of the packed `a`), the down product the rows, so
-// that 32 lanes hold 32 consecutive columns of one row of y.
-#define MFMA2(AF, BF, i)                                                                                     \
+// the four 16-column pieces of this wave's two column blocks: BF[2 * j + ch]
+#define READ_B(BF, stage)                                                                                   \
+    do {                                                                                                    \
+        if (NBLK > 0) {                                                                                     \
+            const unsigned char *sp = smem + (stage) * STAGE_BYTES;                                          \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                    \
+                BF[q] = *(const bf16x8_t *)(sp + pb[q & 1] + (q >> 1) * B_BLK);                              \
+        }                                                                                                   \
+    } while (0)
+// the four MFMAs of half rh of row block i.  The up product feeds the weights as the first operand, so that a lane
+// ends up with 4 consecutive output columns of one row (8 bytes of the packed `a`), the down product the rows, so
+// that 16 lanes hold 16 consecutive columns of one row of y.
+#define MFMA4(AF, BF, i, rh)                                                                                 \
     do {                                                                                                    \
         if ((i) < NBLK) {                                                                                   \
-            _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                    \
-                acc[i][j] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(BF[j], AF[i], acc[i][j], 0, 0, 0) \
-                                 : __builtin_amdgcn_mfma_f32_32x32x16_bf16(AF[i], BF[j], acc[i][j], 0, 0, 0); \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                    \
+                acc[i][q >> 1][rh][q & 1] =                                                                  \
+                    SWAP ? __builtin_amdgcn_mfma_f32_16x16x32_bf16(BF[q], AF[i], acc[i][q >> 1][rh][q & 1], 0, 0, 0) \
+                         : __builtin_amdgcn_mfma_f32_16x16x32_bf16(AF[i], BF[q], acc[i][q >> 1][rh][q & 1], 0, 0, 0); \
         }                                                                                                   \
     } while (0)
 
-    f32x16_t acc[NB][2];
+    // acc[i][j][rh][ch]: 16 x 16 piece (rh, ch) of the 32 x 32 block (row block i, column block j)
+    f32x4_t acc[NB][2][2][2];
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int q = 0; q < 8; ++q)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+            for (int r = 0; r < 4; ++r) acc[i][q >> 2][(q >> 1) & 1][q & 1][r] = 0.0f;
 
-    bf16x8_t af0[NB], bf0[2], af1[NB], bf1[2];
-    READ_FRAGS(af0, bf0, cur, 0);
+    bf16x8_t af0[NB], af1[NB], bq[4], bn[4];
+    READ_A(af0, cur, 0);
+    READ_B(bq, cur);
 
     // One 32-k step on stage `cur`.  The 4 direct loads a wave owes per step are issued one per pair of row blocks:
     //   before the barrier: second half of the loads of step kt-1+NSTAGE, into the stage the previous step released
@@ -315,29 +329,33 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;                                                    \
         const int prv = cur == 0 ? NSTAGE - 1 : cur - 1;                                                    \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
-        READ_FRAGS(af1, bf1, cur, 1);                                                                       \
+        READ_A(af1, cur, 1);                                                                                \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
             if ((i & 1) == 0) {                                                                             \
                 if (GEN) ISSUE_V(prv, kt - 1 + NSTAGE, 2 + (i >> 1));                                       \
                 else issue_load<WNT>(ctx, lds_wave, blk_off, prv, kt - 1 + NSTAGE, 2 + (i >> 1));                \
             }                                                                                               \
-            MFMA2(af0, bf0, i);                                                                             \
+            MFMA4(af0, bq, i, 0);                                                                           \
         }                                                                                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         /* every wave has taken its last fragments of this stage; the next stage must have landed */        \
         if (!GEN || has_next || kt + NSTAGE <= KT) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory"); \
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                                    \
         __syncthreads();                                                                                    \
-        if (!GEN || kt + 1 < KT) READ_FRAGS(af0, bf0, nxt, 0);                                              \
+        if (!GEN || kt + 1 < KT) {                                                                          \
+            READ_A(af0, nxt, 0);                                                                            \
+            READ_B(bn, nxt);                                                                                \
+        }                                                                                                   \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
             if ((i & 1) == 0) {                                                                             \
                 if (GEN) ISSUE_V(cur, kt + NSTAGE, i >> 1);                                                 \
                 else issue_load<WNT>(ctx, lds_wave, blk_off, cur, kt + NSTAGE, i >> 1);                          \
             }                                                                                               \
-            MFMA2(af1, bf1, i);                                                                             \
+            MFMA4(af1, bq, i, 1);                                                                           \
         }                                                                                                   \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) bq[q] = bn[q];                                        \
         cur = nxt;                                                                                          \
     } while (0)
 
@@ -350,30 +368,28 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 
     // ---- epilogue ----
     if (MODE == MODE_UP || MODE == MODE_UPREC) {
-        // lane: row l32 of block i; register r -> column 8*(r/4) + 4*lhi + r%4 of the wave's 32 columns, which are
-        // one k step of the packed `a` (K dimension = N): chunk r/4, bytes lhi*8 .. lhi*8+7
+        // lane: row 16 rh + l16 of block i; piece (rh, ch), register r -> column 16 ch + 4 lq + r of the wave's 32
+        // columns, which are one k step of the packed `a` (K dimension = N): chunk 2 ch + lq / 2, bytes (lq % 2) * 8 ..
         const int KTa = N / BK;
         const int kba = (ctx.n0 >> 5) + wn;
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
-            const int row = (2 * i + wm) * 32 + l32;
-            if (row < ctx.rows) {
-                const int prow = ctx.row0 + row;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    uint32_t pk[2];
+            for (int rh = 0; rh < 2; ++rh) {
+                const int row = (2 * i + wm) * 32 + 16 * rh + l16;
+                if (row < ctx.rows) {
+                    const int prow = ctx.row0 + row;
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        float v[2];
+                    for (int ch = 0; ch < 2; ++ch) {
+                        float v[4];
 #pragma unroll
-                        for (int u = 0; u < 2; ++u) {
-                            const float h1 = acc[i][0][t * 4 + h * 2 + u], h3 = acc[i][1][t * 4 + h * 2 + u];
-                            v[u] = h1 * __builtin_amdgcn_rcpf(1.0f + __expf(-h1)) * h3;  // v_exp_f32, v_rcp_f32: 1 ulp each
+                        for (int r = 0; r < 4; ++r) {
+                            const float h1 = acc[i][0][rh][ch][r], h3 = acc[i][1][rh][ch][r];
+                            v[r] = h1 * __builtin_amdgcn_rcpf(1.0f + __expf(-h1)) * h3;  // v_exp_f32, v_rcp_f32: 1 ulp each
                         }
-                        pk[h] = pack_bf16x2(v[0], v[1]);
+                        const uint2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+                        *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, kba, 2 * ch + (lq >> 1), KTa) + (lq & 1) * 8) = o;
                     }
-                    uint2 o = {pk[0], pk[1]};
-                    *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, kba, t, KTa) + lhi * 8) = o;
                 }
             }
         }
@@ -389,42 +405,47 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
             float *o1 = r1 + (rb * ncb + cb) * 1024 + lane, *o3 = r3 + (rb * ncb + cb) * 1024 + lane;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                o1[r * 64] = acc[i][0][r];
-                o3[r * 64] = acc[i][1][r];
+                o1[r * 64] = acc[i][0][(r >> 3) & 1][(r >> 2) & 1][r & 3];
+                o3[r * 64] = acc[i][1][(r >> 3) & 1][(r >> 2) & 1][r & 3];
             }
         }
     } else if (MODE == MODE_DA) {
-        // acc = d(a) of (row l32 of block i, columns 8*(r/4) + 4*lhi + r%4 of column block j); h1, h3 of the same
+        // acc = d(a) of (row 16 rh + l16 of block i, columns 16 ch + 4 lq + r of column block j); h1, h3 of the same
         // elements come from their records.  dh3 = da * silu(h1); dh1 = da*h3 * s*(1 + h1*(1-s)), s = sigmoid(h1)
         // (silu_backward, J/engine/nn/layer/active/gpu/activeFunction.cu:182-190).  Output: packed image with 2N
         // columns, dh1 in k steps 0..N/32-1, dh3 behind them.
         const int ncb = N >> 5, KTa = 2 * ncb;
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
-            const int row = (2 * i + wm) * 32 + l32;
             const size_t rb = (size_t)ctx.rec0 + 2 * i + wm;
-            const int prow = ctx.row0 + row;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int cb = (ctx.n0 >> 5) + wn * 2 + j;
                 if (cb >= ncb) continue;  // last column tile of a width that is not a multiple of 256
                 const float *p1 = (const float *)Aux1 + (rb * ncb + cb) * 1024 + lane;
                 const float *p3 = (const float *)Aux2 + (rb * ncb + cb) * 1024 + lane;
-                float g1[16], g3[16];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float h1 = p1[r * 64], h3 = p3[r * 64], da = acc[i][j][r];
-                    const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-h1));
-                    g3[r] = da * (h1 * sg);
-                    g1[r] = (da * h3) * sg * (1.0f + h1 * (1.0f - sg));
-                }
-                if (row < ctx.rows) {
+                for (int rh = 0; rh < 2; ++rh) {
+                    const int row = (2 * i + wm) * 32 + 16 * rh + l16;
+                    const int prow = ctx.row0 + row;
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const uint2 o1 = {pack_bf16x2(g1[t * 4], g1[t * 4 + 1]), pack_bf16x2(g1[t * 4 + 2], g1[t * 4 + 3])};
-                        const uint2 o3 = {pack_bf16x2(g3[t * 4], g3[t * 4 + 1]), pack_bf16x2(g3[t * 4 + 2], g3[t * 4 + 3])};
-                        *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, cb, t, KTa) + lhi * 8) = o1;
-                        *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, ncb + cb, t, KTa) + lhi * 8) = o3;
+                    for (int ch = 0; ch < 2; ++ch) {
+                        float g1[4], g3[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int rr = (rh * 2 + ch) * 4 + r;
+                            const float h1 = p1[rr * 64], h3 = p3[rr * 64], da = acc[i][j][rh][ch][r];
+                            const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-h1));
+                            g3[r] = da * (h1 * sg);
+                            g1[r] = (da * h3) * sg * (1.0f + h1 * (1.0f - sg));
+                        }
+                        if (row < ctx.rows) {
+                            const uint2 o1 = {pack_bf16x2(g1[0], g1[1]), pack_bf16x2(g1[2], g1[3])};
+                            const uint2 o3 = {pack_bf16x2(g3[0], g3[1]), pack_bf16x2(g3[2], g3[3])};
+                            const int t = 2 * ch + (lq >> 1);
+                            *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, cb, t, KTa) + (lq & 1) * 8) = o1;
+                            *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, ncb + cb, t, KTa) + (lq & 1) * 8) = o3;
+                        }
                     }
                 }
             }
@@ -437,26 +458,29 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
             Cbase = (float *)Aux1 + (size_t)ctx.slab * (BM * 256);
             ld = 256;
         }
-        // lane: column l32 of each 32x32 block; register r -> row 8*(r/4) + 4*lhi + r%4
+        // lane: column 16 ch + l16 of each 32x32 block; piece (rh, ch), register r -> row 16 rh + 4 lq + r
 #pragma unroll
         for (int i = 0; i < NBLK; ++i) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = (2 * i + wm) * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            for (int q = 0; q < 8; ++q) {
+                const int rh = q >> 2, r = q & 3;
+                const int row = (2 * i + wm) * 32 + 16 * rh + 4 * lq + r;
                 if (row >= ctx.rows) continue;
-                // (32 lanes x 4 bytes = one 128-byte line per store; 16-byte stores of a transposed accumulator layout
-                //  write 32-byte pieces of 32 different lines and were 8 % slower on short-K shapes)
-                float *out = PLAIN_DOWN(MODE) ? Cbase + (size_t)row * ld + wn * 64 + l32
-                                              : Cbase + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l32;
+                // (16 lanes x 4 bytes = half a 128-byte line per row and store)
+                float *out = PLAIN_DOWN(MODE) ? Cbase + (size_t)row * ld + wn * 64 + l16
+                                              : Cbase + (size_t)(ctx.row0 + row) * N + ctx.n0 + wn * 64 + l16;
 #pragma unroll
                 for (int j = 0; j < 2; ++j)  // (non-temporal stores of the weight gradients were 10 % slower)
-                    if (PLAIN_DOWN(MODE) || ctx.n0 + wn * 64 + j * 32 < N) out[j * 32] = acc[i][j][r];
+#pragma unroll
+                    for (int ch = 0; ch < 2; ++ch)
+                        if (PLAIN_DOWN(MODE) || ctx.n0 + wn * 64 + j * 32 + ch * 16 < N) out[j * 32 + ch * 16] = acc[i][j][rh][ch][r];
             }
         }
     }
 #undef ISSUE_V
-#undef READ_FRAGS
-#undef MFMA2
+#undef READ_A
+#undef READ_B
+#undef MFMA4
 }
 
 // Persistent: one workgroup per compute unit walks its queue of work items (built by the dispatch stage).
