@@ -45,6 +45,34 @@ def profiled_traffic(cfg_name):
 
 
 
+def kstep_probe():
+    """The k-step loop of the product kernels in isolation (bench_probe.so), TFLOP/s per variant: 8 waves of 128 x 64
+    (the kernels' shape) and 4 waves of 128 x 128; without loads, then with the 32 KiB of direct loads per step whose
+    streams are shared by 32 / 8 / 4 / 2 workgroups of an XCD (1 MiB streams: the misses come out of the last-level
+    cache; 8 MiB streams: from memory, for the sharings whose streams together exceed 256 MiB)."""
+    import ctypes
+    lib = ctypes.CDLL(os.path.join(ROOT, "bench_probe.so"))   # built by __graft_entry__.build()
+    lib.bench_probe_kstep.argtypes = [ctypes.c_int] * 6 + [ctypes.POINTER(ctypes.c_float)]
+    lib.bench_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+    v = ctypes.c_float()
+    rows = []
+
+    def run(fn, *args):
+        st = fn(*args, ctypes.byref(v))
+        if st != 0:
+            raise RuntimeError(f"bench_probe: HIP error {st}")
+        return round(v.value, 1)
+
+    rows.append({"what": "MFMAs only, 8 waves, random operands", "TFLOP/s": run(lib.bench_probe_mfma, 0, 1, 200)})
+    for waves in (8, 4):
+        rows.append({"what": f"{waves} waves: fragments + barrier", "TFLOP/s": run(lib.bench_probe_kstep, 0, waves, 0, 32, 32, 40)})
+        for share, kib in ((32, 1024), (8, 1024), (4, 1024), (2, 1024), (8, 8192), (4, 8192)):
+            rows.append({"what": f"{waves} waves: + direct loads, {share} workgroups per stream of {kib} KiB "
+                                 f"({256 // share * kib // 1024} MiB in all)",
+                         "TFLOP/s": run(lib.bench_probe_kstep, 0, waves, 1, share, kib, 40)})
+    print(json.dumps({"kstep_probe": rows, "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -64,11 +92,19 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (convert_kernel fp32->fp32) three times, so that "
                          "FETCH_SIZE / WRITE_SIZE of a profiled run can be scaled by a kernel of known traffic")
+    ap.add_argument("--kstep-probe", action="store_true",
+                    help="instead of the benchmark: the rates the inner loop of the product kernels sustains by itself "
+                         "(bench_probe.so: MFMAs + fragment reads + barrier, then with the direct loads at several L2 "
+                         "miss rates), one JSON line")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus above 1 is not supported (no collectives in this path)",
               file=sys.stderr)
         sys.exit(2)
+
+    if a.kstep_probe:
+        kstep_probe()
+        return
 
     P = importlib.import_module("omega-ai_amd")
     L = importlib.import_module("omega-ai_amd._lib")
