@@ -73,6 +73,43 @@ def kstep_probe():
     print(json.dumps({"kstep_probe": rows, "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS}))
 
 
+def vendor_gemm():
+    """hipBLASLt (through torch.matmul) on y = x W^T with bf16 operands of the workload's distributions: the up product
+    (W1 | W3: 2 H outputs) and the down product of the Mixtral shape, once as ONE matrix product over all 8192 expert
+    rows (every weight tile reused by 32 row tiles) and once as 8 products of 1024 rows with 8 different weight
+    matrices (what the layer has to compute: every weight byte is used by 4 row tiles)."""
+    import torch
+    torch.manual_seed(0)
+    dev = "cuda"
+    rows = []
+
+    def one(what, M, N, K, groups, reps=20):
+        xs = [torch.randn(M, K, device=dev, dtype=torch.bfloat16) for _ in range(groups)]
+        ws = [(torch.randn(N, K, device=dev) / K ** 0.5).to(torch.bfloat16) for _ in range(groups)]
+        outs = [torch.empty(M, N, device=dev, dtype=torch.bfloat16) for _ in range(groups)]
+        for _ in range(5):
+            for g in range(groups):
+                torch.matmul(xs[g], ws[g].t(), out=outs[g])
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for g in range(groups):
+                torch.matmul(xs[g], ws[g].t(), out=outs[g])
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        tf = 2.0 * M * N * K * groups / ms / 1e9
+        rows.append({"what": what, "M": M, "N": N, "K": K, "products": groups, "ms": round(ms, 4), "TFLOP/s": round(tf, 1),
+                     "frac": round(tf / PEAK_BF16_TFLOPS, 3)})
+
+    one("up, one product over all rows", 8192, 28672, 4096, 1)
+    one("up, one product per expert", 1024, 28672, 4096, 8)
+    one("down, one product over all rows", 8192, 4096, 14336, 1)
+    one("down, one product per expert", 1024, 4096, 14336, 8)
+    print(json.dumps({"vendor_gemm": rows, "peak": PEAK_BF16_TFLOPS}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -96,6 +133,10 @@ def main():
                     help="instead of the benchmark: the rates the inner loop of the product kernels sustains by itself "
                          "(bench_probe.so: MFMAs + fragment reads + barrier, then with the direct loads at several L2 "
                          "miss rates), one JSON line")
+    ap.add_argument("--vendor-gemm", action="store_true",
+                    help="instead of the benchmark: the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) at the shapes of "
+                         "the Mixtral-shape products, as one product over all rows and as one product per expert; a "
+                         "yardstick measured on the same device, nothing of the layer runs; one JSON line")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus above 1 is not supported (no collectives in this path)",
@@ -104,6 +145,9 @@ def main():
 
     if a.kstep_probe:
         kstep_probe()
+        return
+    if a.vendor_gemm:
+        vendor_gemm()
         return
 
     P = importlib.import_module("omega-ai_amd")
