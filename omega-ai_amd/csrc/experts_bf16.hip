@@ -6,7 +6,9 @@
 //
 // Both operands are K-contiguous ("NT" product), so a lane's 8 consecutive k values are one 16-byte LDS read.
 // Workgroup = 8 waves (2 row halves x 4 column quarters, two waves per SIMD so that one computes while the
-// other waits on LDS, on the address unit or at the barrier); tile = 256 rows x 256 MFMA columns, each wave
+// other waits on LDS, on the address unit, at the barrier or through its item switch: four waves of 128 x 128, one
+// per SIMD, read a third fewer fragments and were 2-3 % faster on long full tiles, but lost twice as much per item
+// and more on ragged tiles and short items); tile = 256 rows x 256 MFMA columns, each wave
 // 4x2 MFMA blocks (the 32-row blocks of the tile alternate between the row halves, so a ragged tile splits evenly) with its 128 accumulators in AGPRs.  For the up product the 256 MFMA columns are
 // 128 columns of W1 and the same 128 columns of W3, arranged so that a wave holds h1 and h3 of the same
 // output element and applies silu(h1)*h3 in registers.
@@ -17,7 +19,7 @@
 // memory as that very image (pack.h: 1 KiB blocks of 16 rows x 32 k with the chunk index XOR-swizzled so the
 // MFMA operand reads are free of bank conflicts), so every direct load reads 1 KiB of contiguous memory.
 // The weights are packed once when they are set, xg by the gather kernel, a by the up product's epilogue.
-// Pipeline per 32-k step and wave: two phases of 8 MFMAs; the fragments of the next phase are read from LDS
+// Pipeline per 32-k step and wave: two phases of 16 MFMAs; the fragments of the next phase are read from LDS
 // while the current one computes; one barrier per step, after which the stage just read is refilled with the
 // step five ahead.  The direct loads are issued one at a time between MFMAs because the address unit is
 // shared by all waves of the CU and a burst of loads stalls the issuing wave.
