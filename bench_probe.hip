@@ -68,10 +68,10 @@ extern "C" int bench_probe_mfma(int device, int random_operands, int launches, f
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     float ms = 0.0f;
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    if (e0) hipEventDestroy(e0);
-    if (e1) hipEventDestroy(e1);
-    if (s) hipStreamDestroy(s);
-    if (scratch) hipFree(scratch);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    if (scratch) (void)hipFree(scratch);
     if (e != hipSuccess) return (int)e;
     // 8 waves per workgroup, 2 x 16 x 16 x 32 FLOP per MFMA
     const double flop = (double)iters * PROBE_ACC * 8.0 * num_cus * 16384.0;
@@ -244,11 +244,11 @@ extern "C" int bench_probe_kstep(int device, int waves, int loads, int share, in
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     float ms = 0.0f;
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    if (e0) hipEventDestroy(e0);
-    if (e1) hipEventDestroy(e1);
-    if (s) hipStreamDestroy(s);
-    if (scratch) hipFree(scratch);
-    if (src) hipFree(src);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    if (scratch) (void)hipFree(scratch);
+    if (src) (void)hipFree(src);
     if (e != hipSuccess) return (int)e;
     const double flop = (double)steps * 256.0 * 16384.0 * n_wg;  // 256 MFMAs of 2 x 16 x 16 x 32 per step and workgroup
     *tflops = (float)(flop * (launches - warm) / (ms * 1e-3) / 1e12);
