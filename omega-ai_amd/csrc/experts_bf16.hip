@@ -107,11 +107,11 @@ __device__ __forceinline__ void dma16_masked(const void *sbase, uint32_t voff, u
                  : "memory");
 }
 
-// Everything the loads of one work item need (uniform over the workgroup except the two lane offsets).
-// A: packed row group of the tile's first row; B0/B1: packed row groups of the two 128-row halves of the B tile.
+// Everything the loads of one work item need, uniform over the wave: lane l adds 16 l to every address.
+// A0/A1: k step 0 of this wave's two 16-row blocks of the A tile (packed row groups of the tile's first row and of the
+// one 128 rows on); B0/B1: the same of the two 128-row halves of the B tile.
 struct TileCtx {
-    const unsigned char *A, *B0, *B1;
-    uint32_t a_off0, a_off1;  // this lane's byte offsets of its two A blocks within a k step
+    const unsigned char *A0, *A1, *B0, *B1;
     uint64_t a_mask0, a_mask1;  // lanes that take part in the two A loads: all, or lane 0 alone for a block without valid rows
     int row0, rows, n0;
     int kt;                   // k steps of the item
@@ -151,11 +151,10 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
         c.half = 0;
         c.slab = 0;
         c.rec0 = 0;
-        c.A = uniform_ptr((const unsigned char *)Axg + (size_t)d.a_rg * rg_bytes + k0);
-        c.B0 = uniform_ptr((const unsigned char *)Wa + (size_t)d.b_rg * rg_bytes + k0);
+        c.A0 = uniform_ptr((const unsigned char *)Axg + (size_t)d.a_rg * rg_bytes + k0 + (size_t)wave * 1024u);
+        c.A1 = uniform_ptr(c.A0 + rg_bytes);
+        c.B0 = uniform_ptr((const unsigned char *)Wa + (size_t)d.b_rg * rg_bytes + k0 + (size_t)wave * 1024u);
         c.B1 = uniform_ptr(c.B0 + rg_bytes);
-        c.a_off0 = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
-        c.a_off1 = (uint32_t)KT * 8192u + c.a_off0;
         c.a_mask0 = c.a_mask1 = ~0ull;
         return c;
     }
@@ -179,14 +178,14 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
             c.rows = 0;
         }
     }
-    c.A = uniform_ptr(((!PLAIN_DOWN(MODE) && Ax != nullptr && d.xrow0 >= 0)
-                           ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
-                           : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes) + k0);
+    const unsigned char *A = ((!PLAIN_DOWN(MODE) && Ax != nullptr && d.xrow0 >= 0)
+                                  ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
+                                  : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes) + k0;
     const size_t wrg = (size_t)d.g * (N >> 7) + (d.n0 >> 7);  // row group of the weight tile
-    c.B0 = uniform_ptr((const unsigned char *)Wa + wrg * rg_bytes + k0);
+    c.B0 = uniform_ptr((const unsigned char *)Wa + wrg * rg_bytes + k0 + (size_t)wave * 1024u);
     // (a half-width item loads its 128 weight rows twice - the second copy comes out of the L2 - and drops the results
     //  of the duplicate: the products it is used for are bound by streaming the weights from memory, not by the MFMAs)
-    c.B1 = uniform_ptr(FUSED ? (const unsigned char *)Wb + wrg * rg_bytes : c.half ? c.B0 : c.B0 + rg_bytes);
+    c.B1 = uniform_ptr(FUSED ? (const unsigned char *)Wb + wrg * rg_bytes + k0 + (size_t)wave * 1024u : c.half ? c.B0 : c.B0 + rg_bytes);
     // Wave-load q (0..15) of an operand tile is the packed block q % 8 of row group q / 8; this wave issues q = wave
     // and q = wave + 8 of both operands.  A points at the row group of the whole row tile; a slice starts blk0
     // 16-row blocks into it.  A blocks that hold no valid row (ragged tile) are never used by an MFMA whose result
@@ -194,8 +193,8 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
     // they cost no extra L2 traffic while every wave still issues the same number of loads per step.
     const int blk0 = (d.row0 & (BM - 1)) >> 4;
     const int qa0 = blk0 + (16 * wave < d.rows ? wave : 0), qa1 = blk0 + (16 * (wave + 8) < d.rows ? wave + 8 : 0);
-    c.a_off0 = (uint32_t)(qa0 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa0 & 7) * 1024u + (uint32_t)lane * 16u;
-    c.a_off1 = (uint32_t)(qa1 >> 3) * (uint32_t)KT * 8192u + (uint32_t)(qa1 & 7) * 1024u + (uint32_t)lane * 16u;
+    c.A0 = uniform_ptr(A + (size_t)(qa0 >> 3) * rg_bytes + (size_t)(qa0 & 7) * 1024u);
+    c.A1 = uniform_ptr(A + (size_t)(qa1 >> 3) * rg_bytes + (size_t)(qa1 & 7) * 1024u);
     c.a_mask0 = 16 * wave < c.rows ? ~0ull : 1ull;
     c.a_mask1 = 16 * (wave + 8) < c.rows ? ~0ull : 1ull;
     return c;
@@ -205,23 +204,32 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
 // (n & 1 ? B : A, n >> 1)
 // A blocks without valid rows move 16 bytes (a_mask0 / a_mask1).
 template <bool WNT = false>
-__device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, uint32_t blk_off, int stage, int kstep, int n)
+__device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, uint32_t lane_off, int stage, int kstep, int n)
 {
     const uint32_t sb = lds_wave + stage * STAGE_BYTES;
-    const uint32_t kb = (uint32_t)kstep * 8192u;
-    if ((n & 1) == 0) dma16_masked(c.A, kb + ((n >> 1) ? c.a_off1 : c.a_off0), sb + (n >> 1) * 8192, (n >> 1) ? c.a_mask1 : c.a_mask0);
-    else if (WNT) dma16_nt((n >> 1) == 0 ? c.B0 : c.B1, kb + blk_off, sb + TILE_BYTES + (n >> 1) * 8192);
-    else dma16((n >> 1) == 0 ? c.B0 : c.B1, kb + blk_off, sb + TILE_BYTES + (n >> 1) * 8192);
+    const size_t kb = (size_t)kstep * 8192u;
+    if ((n & 1) == 0) dma16_masked(((n >> 1) ? c.A1 : c.A0) + kb, lane_off, sb + (n >> 1) * 8192, (n >> 1) ? c.a_mask1 : c.a_mask0);
+    else if (WNT) dma16_nt(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
+    else dma16(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
 }
+
+// Where the four loads a wave owes per k step read next: the pointers move on by one k step (8 KiB of the packed image)
+// with every load and are pointed at the next work item when this one's last step has been asked for.  Loads 0 and 1
+// (first row group of A and of B) run one step ahead of loads 2 and 3.
+struct LoadCursor {
+    const unsigned char *a0, *a1, *b0, *b1;
+    uint64_t m0, m1;
+};
 
 // One work item.  NBLK = number of 32-row blocks of this wave that hold valid rows (the others are never
 // computed: a ragged last row tile of an expert costs only the blocks it fills).  NBLK == 0: the wave only
 // takes part in the loads and barriers.
 // The ring of stages runs on across work items: on entry, stage `cur` holds (or is about to receive) k step 0 of this
 // item, k steps 0..NSTAGE-2 and the first half of step NSTAGE-1 are in flight, and the barrier that makes step 0
-// visible has been passed.  The last NSTAGE steps issue the first loads of the next item (dn, if it has rows)
-// instead of their own, so the matrix cores of the next item start on data that travelled during this item's
-// epilogue.
+// visible has been passed.  The last NSTAGE steps issue the first loads of the next item (dn) instead of their own,
+// so the matrix cores of the next item start on data that travelled during this item's epilogue; behind the last item
+// of a queue they fetch this item's first steps once more (lane 0 only for A), so that every step of every item
+// issues the same four loads and waits the same way.
 template <int MODE, int NBLK, bool WNT>
 __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_in, TileCtx &nx, const omega_tile_desc &dn,
                                          const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa, const bf16_t *Wb, int &cur_io,
@@ -232,7 +240,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     // the item's uniform fields and the ring position live in scalar registers for the whole item (the direct loads
     // take their base address and LDS address from scalar operands)
     TileCtx ctx = ctx_in;
-    ctx.A = uniform_ptr(ctx_in.A);
+    ctx.A0 = uniform_ptr(ctx_in.A0);
+    ctx.A1 = uniform_ptr(ctx_in.A1);
     ctx.B0 = uniform_ptr(ctx_in.B0);
     ctx.B1 = uniform_ptr(ctx_in.B1);
     ctx.row0 = __builtin_amdgcn_readfirstlane(ctx_in.row0);
@@ -247,16 +256,17 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     const int wm = wave >> 2, wn = wave & 3;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     const uint32_t lds_wave = lds0 + wave * 1024;
-    const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
+    const uint32_t lane_off = (uint32_t)lane * 16u;
     const int KT = ITEM_K(MODE) ? __builtin_amdgcn_readfirstlane(ctx_in.kt) : Kd / BK;
     const bool has_next = dn.rows > 0;
-
-// load n of virtual k step v: steps beyond this item's last belong to the next item
-#define ISSUE_V(stage, v, n)                                                              \
-    do {                                                                                  \
-        if ((v) < KT) issue_load<WNT>(ctx, lds_wave, blk_off, stage, v, n);                    \
-        else if (has_next) issue_load<WNT>(nx, lds_wave, blk_off, stage, (v) - KT, n);          \
-    } while (0)
+    LoadCursor lc;
+    lc.a0 = ctx.A0 + (size_t)NSTAGE * 8192;
+    lc.b0 = ctx.B0 + (size_t)NSTAGE * 8192;
+    lc.a1 = ctx.A1 + (size_t)(NSTAGE - 1) * 8192;
+    lc.b1 = ctx.B1 + (size_t)(NSTAGE - 1) * 8192;
+    lc.m0 = ctx.a_mask0;
+    lc.m1 = ctx.a_mask1;
+#define LOAD_B(ptr, lds) do { if (WNT) dma16_nt(ptr, lane_off, lds); else dma16(ptr, lane_off, lds); } while (0)
 
     // ---- MFMA operand addressing ----
     // Row (2i + wm)*32 + 16 rh + l16 of A, row j*128 + wn*32 + 16 ch + l16 (up: block 0 = 32 columns of W1, block 1 = the
@@ -328,55 +338,66 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     READ_B(bq, cur);
 
     // One 32-k step on stage `cur`.  The 4 direct loads a wave owes per step are issued one per pair of row blocks:
-    //   before the barrier: second half of the loads of step kt-1+NSTAGE, into the stage the previous step released
-    //   after the barrier:  first half of the loads of step kt+NSTAGE, into the stage this step releases
-    // While loads keep coming (this item's or the next one's) exactly NSTAGE-2 younger steps (12 loads) may stay in
-    // flight at the barrier; when they have stopped (last steps of a queue) everything must have landed.
-    // GEN = false: every load belongs to this item (kt < KT - NSTAGE), no run-time decisions in the loop.
-#define K_STEP(GEN, Z)                                                                                        \
+    //   before the barrier: loads 2 and 3 of step kt-1+NSTAGE, into the stage the previous step released
+    //   after the barrier:  loads 0 and 1 of step kt+NSTAGE, into the stage this step releases
+    // Every step of every item issues its four loads (see LoadCursor), so exactly NSTAGE-2 younger steps (12 loads) may
+    // stay in flight at the barrier, and every step reads the fragments of the one behind it (the last step of an item
+    // those of the next item's first, which run_tile reads again on entry).
+#define K_STEP(Z)                                                                                             \
     do {                                                                                                    \
         const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;                                                    \
         const int prv = cur == 0 ? NSTAGE - 1 : cur - 1;                                                    \
+        const uint32_t sb_prv = lds_wave + prv * STAGE_BYTES, sb_cur = lds_wave + cur * STAGE_BYTES;        \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         READ_A(af1, cur, 1);                                                                                \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
-            if ((i & 1) == 0) {                                                                             \
-                if (GEN) ISSUE_V(prv, kt - 1 + NSTAGE, 2 + (i >> 1));                                       \
-                else issue_load<WNT>(ctx, lds_wave, blk_off, prv, kt - 1 + NSTAGE, 2 + (i >> 1));                \
-            }                                                                                               \
+            if (i == 0) dma16_masked(lc.a1, lane_off, sb_prv + 8192, lc.m1);                                \
+            if (i == 2) LOAD_B(lc.b1, sb_prv + TILE_BYTES + 8192);                                          \
             MFMA4(af0, bq, i, 0, Z);                                                                         \
         }                                                                                                   \
+        lc.a1 += 8192;                                                                                      \
+        lc.b1 += 8192;                                                                                      \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         /* every wave has taken its last fragments of this stage; the next stage must have landed */        \
-        if (!GEN || has_next || kt + NSTAGE <= KT) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory"); \
-        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                                    \
+        asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");                                        \
         __syncthreads();                                                                                    \
-        if (!GEN || kt + 1 < KT) {                                                                          \
-            READ_A(af0, nxt, 0);                                                                            \
-            READ_B(bn, nxt);                                                                                \
-        }                                                                                                   \
+        READ_A(af0, nxt, 0);                                                                                \
+        READ_B(bn, nxt);                                                                                    \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
-            if ((i & 1) == 0) {                                                                             \
-                if (GEN) ISSUE_V(cur, kt + NSTAGE, i >> 1);                                                 \
-                else issue_load<WNT>(ctx, lds_wave, blk_off, cur, kt + NSTAGE, i >> 1);                          \
-            }                                                                                               \
+            if (i == 0) dma16_masked(lc.a0, lane_off, sb_cur, lc.m0);                                       \
+            if (i == 2) LOAD_B(lc.b0, sb_cur + TILE_BYTES);                                                 \
             MFMA4(af1, bq, i, 1, Z);                                                                         \
         }                                                                                                   \
+        lc.a0 += 8192;                                                                                      \
+        lc.b0 += 8192;                                                                                      \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) bq[q] = bn[q];                                        \
         cur = nxt;                                                                                          \
     } while (0)
 
     int kt = 0;
     if (ZFIRST) {
-        K_STEP(false, true);
+        K_STEP(true);
         ++kt;
     }
-    for (; kt < KT - NSTAGE; ++kt) K_STEP(false, false);
+    for (; kt < KT - NSTAGE; ++kt) K_STEP(false);
+    // from here on the loads belong to the next item; loads 2 and 3 follow one step later
     nx = make_ctx<MODE>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr);
-    for (; kt < KT; ++kt) K_STEP(true, false);
+    lc.a0 = has_next ? nx.A0 : ctx.A0;
+    lc.b0 = has_next ? nx.B0 : ctx.B0;
+    lc.m0 = has_next ? nx.a_mask0 : 1ull;
+#pragma unroll 1
+    for (int s = 0; s < NSTAGE; ++s) {
+        if (s == 1) {
+            lc.a1 = has_next ? nx.A1 : ctx.A1;
+            lc.b1 = has_next ? nx.B1 : ctx.B1;
+            lc.m1 = has_next ? nx.a_mask1 : 1ull;
+        }
+        K_STEP(false);
+    }
 #undef K_STEP
+#undef LOAD_B
     cur_io = cur;
 
     // ---- epilogue ----
@@ -490,7 +511,6 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
             }
         }
     }
-#undef ISSUE_V
 #undef READ_A
 #undef READ_B
 #undef MFMA4
@@ -516,13 +536,13 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
         // first item: k steps 0..NSTAGE-2 and the first half of step NSTAGE-1 into stages 0..NSTAGE-1
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
         const uint32_t lds_wave = lds0 + wave * 1024;
-        const uint32_t blk_off = (uint32_t)wave * 1024u + (uint32_t)lane * 16u;
+        const uint32_t lane_off = (uint32_t)lane * 16u;
         for (int st = 0; st < NSTAGE - 1; ++st) {
 #pragma unroll
-            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<WNT>(cur_ctx, lds_wave, blk_off, st, st, n);
+            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<WNT>(cur_ctx, lds_wave, lane_off, st, st, n);
         }
-        issue_load<WNT>(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 0);
-        issue_load<WNT>(cur_ctx, lds_wave, blk_off, NSTAGE - 1, NSTAGE - 1, 1);
+        issue_load<WNT>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 0);
+        issue_load<WNT>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 1);
         asm volatile("s_waitcnt vmcnt(14)" ::: "memory");  // all but steps 1.. : LOADS_PER_STEP * (NSTAGE - 2) + 2
         __syncthreads();
     }
@@ -545,6 +565,7 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
         if (dn.rows <= 0) break;
         cur_ctx = nx;
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the loads behind the last item land in LDS that nobody reads)
 }
 
 // y += the partial results of the k-sliced items of a down product, in slice order.  The sliced items are the
