@@ -376,6 +376,8 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         cur = nxt;                                                                                          \
     } while (0)
 
+    // (every item has at least NSTAGE + 1 steps: widths are multiples of 256, a k slice has 8 steps or more, an item of
+    //  the weight-gradient products 6)
     int kt = 0;
     if (ZFIRST) {
         K_STEP(true);
