@@ -81,31 +81,35 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
     return *(const uint32_t *)&r;
 }
 
-// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16*l.
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + LDS_OFF + 16*l (the sum is formed
+// in m0 by the instruction that sets it: a constant offset costs nothing).
+template <int LDS_OFF>
 __device__ __forceinline__ void dma16(const void *sbase, uint32_t voff, uint32_t lds_base)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(sbase), "v"(voff), "s"(lds_base)
-                 : "memory");
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(sbase), "v"(voff), "s"(lds_base), "n"(LDS_OFF)
+                 : "memory", "scc");
 }
 
 // Non-temporal form, for weight tiles that no other item will read again (small batches: the weights are streamed
 // once, and letting them pass the last-level cache by is worth 9 % of the stream: 5.9 -> 6.5 TB/s at 64 tokens)
+template <int LDS_OFF>
 __device__ __forceinline__ void dma16_nt(const void *sbase, uint32_t voff, uint32_t lds_base)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0 nt" ::"s"(sbase), "v"(voff), "s"(lds_base)
-                 : "memory");
+    asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0 nt" ::"s"(sbase), "v"(voff), "s"(lds_base), "n"(LDS_OFF)
+                 : "memory", "scc");
 }
 
 // The same with only the lanes of `mask` taking part: a wave whose 16-row block of the A tile holds no valid row keeps
 // its place in the load sequence (the waits count instructions) but moves 16 bytes instead of 1 KiB.
 // Only called where every lane of the wave is active (the k steps and the kernel's first loads sit in wave-uniform
 // control flow), so the mask is put back as all ones instead of being saved.
+template <int LDS_OFF>
 __device__ __forceinline__ void dma16_masked(const void *sbase, uint32_t voff, uint32_t lds_base, uint64_t mask)
 {
-    asm volatile("s_mov_b32 m0, %2\n\ts_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %1, %0\n\ts_mov_b64 exec, -1"
+    asm volatile("s_add_u32 m0, %2, %4\n\ts_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %1, %0\n\ts_mov_b64 exec, -1"
                  :
-                 : "s"(sbase), "v"(voff), "s"(lds_base), "s"(mask)
-                 : "memory");
+                 : "s"(sbase), "v"(voff), "s"(lds_base), "s"(mask), "n"(LDS_OFF)
+                 : "memory", "scc");
 }
 
 // Everything the loads of one work item need, uniform over the wave: lane l adds 16 l to every address.
@@ -209,9 +213,9 @@ __device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, 
 {
     const uint32_t sb = lds_wave + stage * STAGE_BYTES;
     const size_t kb = (size_t)kstep * 8192u;
-    if ((n & 1) == 0) dma16_masked(((n >> 1) ? c.A1 : c.A0) + kb, lane_off, sb + (n >> 1) * 8192, (n >> 1) ? c.a_mask1 : c.a_mask0);
-    else if (WNT) dma16_nt(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
-    else dma16(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
+    if ((n & 1) == 0) dma16_masked<0>(((n >> 1) ? c.A1 : c.A0) + kb, lane_off, sb + (n >> 1) * 8192, (n >> 1) ? c.a_mask1 : c.a_mask0);
+    else if (WNT) dma16_nt<0>(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
+    else dma16<0>(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
 }
 
 // Where the four loads a wave owes per k step read next: the pointers move on by one k step (8 KiB of the packed image)
@@ -267,7 +271,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     lc.b1 = ctx.B1 + (size_t)(NSTAGE - 1) * 8192;
     lc.m0 = ctx.a_mask0;
     lc.m1 = ctx.a_mask1;
-#define LOAD_B(ptr, lds) do { if (WNT) dma16_nt(ptr, lane_off, lds); else dma16(ptr, lane_off, lds); } while (0)
+#define LOAD_B(ptr, voff, lds, off) do { if (WNT) dma16_nt<off>(ptr, voff, lds); else dma16<off>(ptr, voff, lds); } while (0)
 
     // ---- MFMA operand addressing ----
     // Row (2i + wm)*32 + 16 rh + l16 of A, row j*128 + wn*32 + 16 ch + l16 (up: block 0 = 32 columns of W1, block 1 = the
@@ -344,21 +348,21 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     // Every step of every item issues its four loads (see LoadCursor), so exactly NSTAGE-2 younger steps (12 loads) may
     // stay in flight at the barrier, and every step reads the fragments of the one behind it (the last step of an item
     // those of the next item's first, which run_tile reads again on entry).
-#define K_STEP_AT(cur, Z)                                                                                     \
+// BP + IP / BC + IC: LDS address of this wave's first load into the previous / the current stage (scalar register +
+// constant); VOFF: the lane's offset from the load pointers, which then move on by ADV bytes
+#define K_STEP_BODY(cur, BP, IP, BC, IC, VOFF, ADV, Z)                                                                \
     do {                                                                                                    \
         const int nxt = (cur) + 1 == NSTAGE ? 0 : (cur) + 1;                                                \
-        const int prv = (cur) == 0 ? NSTAGE - 1 : (cur)-1;                                                  \
-        const uint32_t sb_prv = lds_wave + prv * STAGE_BYTES, sb_cur = lds_wave + (cur) * STAGE_BYTES;      \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         READ_A(af1, cur, 1);                                                                                \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
-            if (i == 0) dma16_masked(lc.a1, lane_off, sb_prv + 8192, lc.m1);                                \
-            if (i == 2) LOAD_B(lc.b1, sb_prv + TILE_BYTES + 8192);                                          \
+            if (i == 0) dma16_masked<(IP) + 8192>(lc.a1, VOFF, BP, lc.m1);                                  \
+            if (i == 2) LOAD_B(lc.b1, VOFF, BP, (IP) + TILE_BYTES + 8192);                                  \
             MFMA4(af0, bq, i, 0, Z);                                                                         \
         }                                                                                                   \
-        lc.a1 += 8192;                                                                                      \
-        lc.b1 += 8192;                                                                                      \
+        lc.a1 += (ADV);                                                                                     \
+        lc.b1 += (ADV);                                                                                     \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         /* every wave has taken its last fragments of this stage; the next stage must have landed */        \
         asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");                                        \
@@ -367,18 +371,24 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         READ_B(bn, nxt);                                                                                    \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
-            if (i == 0) dma16_masked(lc.a0, lane_off, sb_cur, lc.m0);                                       \
-            if (i == 2) LOAD_B(lc.b0, sb_cur + TILE_BYTES);                                                 \
+            if (i == 0) dma16_masked<(IC)>(lc.a0, VOFF, BC, lc.m0);                                         \
+            if (i == 2) LOAD_B(lc.b0, VOFF, BC, (IC) + TILE_BYTES);                                         \
             MFMA4(af1, bq, i, 1, Z);                                                                         \
         }                                                                                                   \
-        lc.a0 += 8192;                                                                                      \
-        lc.b0 += 8192;                                                                                      \
+        lc.a0 += (ADV);                                                                                     \
+        lc.b0 += (ADV);                                                                                     \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) bq[q] = bn[q];                                        \
     } while (0)
+// the step at a ring position known at compile time
+// (one of five in a row from position 0: the lane offsets carry the k step, the pointers move once per five)
+#define K_STEP_AT(c, Z) \
+    K_STEP_BODY(c, lds_wave, ((c) == 0 ? NSTAGE - 1 : (c)-1) * STAGE_BYTES, lds_wave, (c)*STAGE_BYTES, lane_off + (c)*8192u, 0, Z)
 // the step at the ring's position, whatever it is
 #define K_STEP(Z)                                                                                             \
     do {                                                                                                    \
-        K_STEP_AT(cur, Z);                                                                                  \
+        const uint32_t sb_prv = lds_wave + (cur == 0 ? NSTAGE - 1 : cur - 1) * STAGE_BYTES;                 \
+        const uint32_t sb_cur = lds_wave + cur * STAGE_BYTES;                                               \
+        K_STEP_BODY(cur, sb_prv, 0, sb_cur, 0, lane_off, 8192, Z);                                                       \
         cur = cur + 1 == NSTAGE ? 0 : cur + 1;                                                              \
     } while (0)
 
@@ -403,6 +413,10 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         K_STEP_AT(2, false);
         K_STEP_AT(3, false);
         K_STEP_AT(4, false);
+        lc.a0 += NSTAGE * 8192;
+        lc.b0 += NSTAGE * 8192;
+        lc.a1 += NSTAGE * 8192;
+        lc.b1 += NSTAGE * 8192;
     }
     // the remaining steps; in the last NSTAGE of them the loads belong to the next item, loads 2 and 3 one step later
     nx = make_ctx<MODE>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr);
@@ -422,6 +436,7 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     }
 #undef K_STEP
 #undef K_STEP_AT
+#undef K_STEP_BODY
 #undef LOAD_B
     cur_io = cur;
 
