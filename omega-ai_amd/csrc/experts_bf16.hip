@@ -9,7 +9,8 @@
 // other waits on LDS, on the address unit, at the barrier or through its item switch: four waves of 128 x 128, one
 // per SIMD, read a third fewer fragments and were 2-3 % faster on long full tiles, but lost twice as much per item
 // and more on ragged tiles and short items); tile = 256 rows x 256 MFMA columns, each wave
-// 4x2 MFMA blocks (the 32-row blocks of the tile alternate between the row halves, so a ragged tile splits evenly) with its 128 accumulators in AGPRs.  For the up product the 256 MFMA columns are
+// 4x2 MFMA blocks (the 32-row blocks of the tile alternate between the row halves, so a ragged tile splits evenly) with
+// 128 accumulator registers (of the 256 a wave has at two waves per SIMD).  For the up product the 256 MFMA columns are
 // 128 columns of W1 and the same 128 columns of W3, arranged so that a wave holds h1 and h3 of the same
 // output element and applies silu(h1)*h3 in registers.
 //
@@ -21,8 +22,10 @@
 // The weights are packed once when they are set, xg by the gather kernel, a by the up product's epilogue.
 // Pipeline per 32-k step and wave: two phases of 16 MFMAs; the fragments of the next phase are read from LDS
 // while the current one computes; one barrier per step, after which the stage just read is refilled with the
-// step five ahead.  The direct loads are issued one at a time between MFMAs because the address unit is
-// shared by all waves of the CU and a burst of loads stalls the issuing wave.
+// step five ahead; four direct loads per wave and step.  Every step of every item is the same code (the addresses the
+// loads read from next sit in scalar registers and are switched to the next item when its turn comes), and the bulk of
+// an item runs five steps at a time from ring position 0 with every LDS address a constant: under the power cap the
+// launch time follows the work per MFMA, instructions included (68-71 per step and wave, 32 of them MFMAs).
 //
 // Scheduling: persistent, one workgroup per compute unit.  The dispatch stage leaves every workgroup a queue of
 // work items (32-byte descriptors: an output tile, or a slice of the rows of one for the last tiles of a launch;
