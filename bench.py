@@ -202,9 +202,11 @@ def main():
     # bytes these kernels cannot avoid moving as the path is specified (not the algorithmic figures above): the gather
     # reads every token row once and writes it K times (+ once per batch for the shared experts' packed copy); the
     # combine reads the expert outputs as the fp32 rows the composition keeps them in
+    # (bf16 layers whose up product fetches the rows of x itself write no gathered copy: the dispatch stage then moves
+    #  index data only, and its byte fractions say nothing - they are left out)
+    on_load = layer.gather_on_load()
     dispatch_real = cfg.T * cfg.d * b + cfg.P * cfg.d * b + (cfg.T * cfg.d * b if cfg.Es else 0) + cfg.P * 12
     combine_real = rows * cfg.d * 4 + cfg.T * cfg.d * b + cfg.P * 8
-    gather_ms = layer.time_stage(L.STAGE_GATHER, x, cfg.T, warmup=2, iters=20)
     # block form (out = x + layer(rmsnorm(x)), the widening next to the path): whole call and its pre-norm kernel
     outb = P.DeviceBuffer(ctx, (cfg.T, cfg.d), cfg.dtype)
     block_ms = layer.time_stage(L.STAGE_FORWARD_BLOCK, x, cfg.T, out=outb, warmup=2, iters=a.steps)
@@ -289,10 +291,11 @@ def main():
             "experts_down": {"TFLOP/s": down_tflops, "frac_mfma": down_tflops / peak},
             "experts_total_frac_mfma": (up_flops + down_flops) / ((stage_ms["experts_up"] + stage_ms["experts_down"]) * 1e-3) / 1e12 / peak,
             "router": {"GB/s": router_bytes / (stage_ms["router"] * 1e-3) / 1e9, "frac_hbm": router_bytes / (stage_ms["router"] * 1e-3) / 1e9 / PEAK_HBM_GBPS},
-            "dispatch": {"GB/s": dispatch_bytes / (stage_ms["dispatch"] * 1e-3) / 1e9,
-                         "frac_hbm": dispatch_bytes / (stage_ms["dispatch"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,
-                         "frac_hbm_real_traffic": dispatch_real / (stage_ms["dispatch"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,
-                         "gather_only_ms": gather_ms, "gather_only_GB/s": 2 * cfg.P * cfg.d * b / (gather_ms * 1e-3) / 1e9,
+            "dispatch": {"rows": "fetched from x by the loads of the up product (no gathered copy)" if on_load
+                                 else "gathered copy written by the dispatch launch",
+                         "GB/s": None if on_load else dispatch_bytes / (stage_ms["dispatch"] * 1e-3) / 1e9,
+                         "frac_hbm": None if on_load else dispatch_bytes / (stage_ms["dispatch"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                         "frac_hbm_real_traffic": None if on_load else dispatch_real / (stage_ms["dispatch"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                          "index_only_ms": index_ms},
             "combine": {"GB/s": combine_bytes / (stage_ms["combine"] * 1e-3) / 1e9,
                         "frac_hbm": combine_bytes / (stage_ms["combine"] * 1e-3) / 1e9 / PEAK_HBM_GBPS,

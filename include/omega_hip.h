@@ -169,6 +169,24 @@ int omega_moe_backward_block(omega_moe *moe, const void *x_dev, const void *dout
  * omega_moe_backward reads them instead of recomputing them.  Same results either way; the forward pass writes
  * 8*H bytes more per expert row.  fp32 layers ignore the switch. */
 int omega_moe_set_training(omega_moe *moe, int on);
+/* How the rows of x reach the experts of a bf16 layer.  The reference has no dispatch (its row gathers, e.g.
+ * img_token_drop, J/engine/nn/layer/dit/kernel/TokenDropKernel.cu:147-160, always write the gathered copy).
+ *   OMEGA_GATHER_AUTO (default): by shape - see below;
+ *   OMEGA_GATHER_COPY: the dispatch stage writes every token row into its K places of an expert-contiguous buffer;
+ *   OMEGA_GATHER_ON_LOAD: no copy - the loads of the up product fetch each row of a tile from x through the
+ *     row -> token table of the dispatch stage.  Same results bit for bit.  The loads then read 64-byte pieces of
+ *     rows instead of whole lines, which costs the product 1-8 %, and K row copies per token are saved: AUTO takes
+ *     this form while H/128 <= 2 K (a row tile is read H/128 times).
+ * Training mode and fp32 layers always copy.  x must stay unchanged until the forward pass has finished either way;
+ * with ON_LOAD, omega_moe_get_workspace(moe, 0, ...) and a backward pass gather the rows when they are asked for,
+ * from the x of the last dispatch, which must still hold that batch. */
+#define OMEGA_GATHER_AUTO 0
+#define OMEGA_GATHER_COPY 1
+#define OMEGA_GATHER_ON_LOAD 2
+int omega_moe_set_gather_mode(omega_moe *moe, int mode);
+/* 1 if the last dispatch stage left the rows to the up product's loads, 0 if it wrote the gathered copy (what AUTO
+ * chose for the shape; no counterpart in the reference). */
+int omega_moe_gather_on_load(omega_moe *moe);
 /* One parameter gradient of the last omega_moe_backward, always fp32, in the layout of the weight it belongs to
  * (which / expert as for omega_moe_set_weights).  Stands in for reading layer.diffW / diffB
  * (LlamaMLPLayer.putParamterGrads, J/engine/nn/layer/llama/LlamaMLPLayer.java:285-295). */
@@ -231,9 +249,10 @@ int omega_moe_get_routing(omega_moe *moe, int T, int32_t *ids, float *w, int32_t
 /* Router intermediates, for tests: runs the router on x_dev and copies logits and probabilities
  * [T,E] to host (blocking).  Overwrites the routing state like omega_moe_router. */
 int omega_moe_get_router_probs(omega_moe *moe, const void *x_dev, int T, float *logits, float *probs);
-/* omega_moe_get_router_probs for callers that cannot allocate device memory (code under HIP graph capture around it,
- * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same result and
- * same effect on the routing state, but it calls no hipMalloc / hipFree: logits and probabilities are staged in a
+/* omega_moe_get_router_probs for callers that cannot allocate device memory (tight serving loops, harnesses that
+ * forbid hipMalloc).  It has no counterpart in the reference.  Same result and same effect on the routing state, and
+ * like it a blocking call (it waits for the stream and copies to pageable host memory, so it cannot itself be
+ * captured into a HIP graph), but it calls no hipMalloc / hipFree: logits and probabilities are staged in a
  * static device array of the library (2 x 4 MiB per device, held until the process ends) and the layer's workspace is
  * never grown.  Refused with a message: T above the workspace the layer already holds (create it with T_max >= T), and
  * T*E above 1048576.  All calls on one device share the array: calls that overlap on one device (two contexts, two

@@ -53,6 +53,8 @@ SIGNATURES = {
     "omega_jrandom_next_gaussian": (C.c_double, [C.c_void_p]),
     "omega_jrandom_normal": (None, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_float]),
     "omega_moe_set_training": (C.c_int, [C.c_void_p, C.c_int]),
+    "omega_moe_set_gather_mode": (C.c_int, [C.c_void_p, C.c_int]),
+    "omega_moe_gather_on_load": (C.c_int, [C.c_void_p]),
     "omega_moe_get_grad": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
     "omega_moe_acc_grad": (C.c_int, [C.c_void_p, C.c_float]),
     "omega_moe_update_adamw": (C.c_int, [C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int]),

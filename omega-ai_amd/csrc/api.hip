@@ -193,12 +193,13 @@ static void moe_free_backward_workspace(omega_moe *m)
 
 static void moe_free_workspace(omega_moe *m)
 {
-    void *ptrs[] = {m->ids, m->w, m->tile_counts, m->tile_base, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y,
-                    m->desc_up, m->desc_down, m->wq_up, m->wq_down, m->rms, m->hbuf};
+    void *ptrs[] = {m->ids, m->w, m->tile_counts, m->dst, m->dstp, m->src_row, m->tiles, m->xg, m->xs, m->a, m->y,
+                    m->desc_up, m->desc_down, m->wq_up, m->wq_down, m->rms, m->hbuf, m->tokp};
     for (void *p : ptrs)
         if (p) hipFree(p);
-    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->tile_base = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr; m->rms = nullptr; m->hbuf = nullptr;
-    m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr;
+    m->ids = nullptr; m->w = nullptr; m->tile_counts = nullptr; m->dst = nullptr; m->dstp = nullptr; m->src_row = nullptr; m->xs = nullptr; m->desc_up = nullptr; m->desc_down = nullptr; m->wq_up = nullptr; m->wq_down = nullptr; m->rms = nullptr; m->hbuf = nullptr;
+    m->tiles = nullptr; m->xg = nullptr; m->a = nullptr; m->y = nullptr; m->tokp = nullptr;
+    m->xg_valid = false;
     m->T_cap = 0;
     moe_free_backward_workspace(m);
     m->fwd_T = -1;
@@ -326,10 +327,11 @@ static int moe_reserve(omega_moe *m, int T)
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->rms, (size_t)T * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc(&m->hbuf, (size_t)T * c.d * m->esize));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_counts, (size_t)n_tok_tiles * c.E * 4));
-    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tile_base, (size_t)n_tok_tiles * c.E * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->dst, P * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->dstp, P * 4));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->src_row, P * 4));
+    OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tokp, m->rows_cap * 4));
+    OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->tokp, 0, m->rows_cap * 4, ctx->stream));
     OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->tiles, (size_t)m->tiles_cap * sizeof(omega_tile)));
     OMEGA_HIP_CHECK(ctx, hipMalloc(&m->xg, m->rows_cap * c.d * m->esize));
     OMEGA_HIP_CHECK(ctx, hipMalloc(&m->a, m->rows_cap * c.H * m->esize));
@@ -346,6 +348,8 @@ static int moe_reserve(omega_moe *m, int T)
         const size_t q_down = (std::max((size_t)m->tiles_cap * (c.d / 256), (size_t)m->n_wg) + OMEGA_TAIL_EXTRA) / m->n_wg + 2;
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->wq_up, q_up * m->n_wg * sizeof(omega_tile_desc)));
         OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->wq_down, q_down * m->n_wg * sizeof(omega_tile_desc)));
+        // partial results of k-sliced items of the down product: sliced entries never exceed 256, each a tile of 256 x 256
+        if (!m->y_slabs) OMEGA_HIP_CHECK(ctx, hipMalloc((void **)&m->y_slabs, (size_t)256 * 256 * 256 * 4));
         // an all-zero queue is an empty one: the product kernels return at once if no dispatch has run yet
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->wq_up, 0, q_up * m->n_wg * sizeof(omega_tile_desc), ctx->stream));
         OMEGA_HIP_CHECK(ctx, hipMemsetAsync(m->wq_down, 0, q_down * m->n_wg * sizeof(omega_tile_desc), ctx->stream));
@@ -546,6 +550,16 @@ int omega_moe_get_weights(omega_moe *m, int which, int expert, void *dst, int is
 }
 
 // ---- stages (caller holds the context lock) ----
+// Whether the up product should fetch the rows of x itself instead of reading a gathered copy: its A loads then read
+// 64-byte pieces of rows (half a line each), which costs the product 1-8 %, and the gather (K row copies per token) is
+// saved.  Every row tile is read once per column tile, H/128 times; the gather writes K rows per token: worth it while
+// H/128 <= 2 K.  Measured (forward pass): 16384 tokens, 128 experts, K = 8, H = 768: 1.63 -> 1.49 ms; 8192 tokens, 64
+// experts, K = 6, H = 1408: 1.244 -> 1.234 ms; 4096 tokens, 8 experts, K = 2, H = 14336: 2.32 -> 2.35 ms (not taken).
+static bool gather_on_load_wanted(const omega_moe *m)
+{
+    if (m->gather_mode != OMEGA_GATHER_AUTO) return m->gather_mode == OMEGA_GATHER_ON_LOAD;
+    return m->cfg.H / 128 <= 2 * m->cfg.K;
+}
 static int check_T(omega_moe *m, const void *x, int T, bool need_x)
 {
     omega_ctx *ctx = m->ctx;
@@ -596,14 +610,30 @@ static int stage_dispatch(omega_moe *m, const void *x, int T)
         // are cut into up to 4 k slices (rather than row slices, which stream the whole weight tile for a quarter of
         // the rows and are bound by that stream), if a slice keeps at least 64 k steps.
         m->down_tail_ks = (m->down_ks_max == 1 && !small && c.H >= 2 * 64 * 32) ? 4 : 1;
-        // sliced entries never exceed 256, so there are at most 256 partial results, each a tile of 256 x 256
-        if ((m->down_ks_max > 1 || m->down_tail_ks > 1) && !m->y_slabs)
-            OMEGA_HIP_CHECK(m->ctx, hipMalloc((void **)&m->y_slabs, (size_t)256 * 256 * 256 * 4));
     }
     if (m->max_m_tiles > m->tiles_cap) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "dispatch: workspace too small for this T");
-    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream));
-    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));
+    // bf16 layers outside training: the up product fetches the rows of x through the row -> token table itself, so the
+    // gathered copy xg (and the packed copy xs for shared experts) is neither written nor read; it is made on demand
+    // for what still wants it (a backward pass, omega_moe_get_workspace).  A lane's offset into x is 32 bits wide.
+    m->gather_on_load = m->cfg.dtype == OMEGA_DTYPE_BF16 && !m->training && gather_on_load_wanted(m) &&
+                        (double)T * m->cfg.d * 2.0 < 4.0e9;
+    m->xg_valid = false;
+    m->last_x = x;
+    // (bf16 layers: the index launch copies the rows as well; fp32 layers gather in a launch of its own)
+    const bool bf = m->cfg.dtype == OMEGA_DTYPE_BF16;
+    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_index(m, T, bm, m->ctx->stream, bf && !m->gather_on_load ? x : nullptr));
+    if (!bf) OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));
+    m->xg_valid = !m->gather_on_load;
     m->dispatched_T = T;
+    return OMEGA_OK;
+}
+// the gathered rows xg / xs of the batch the dispatch stage last ran for, if the forward pass went without them
+static int ensure_gathered(omega_moe *m, const void *x, int T)
+{
+    if (m->xg_valid) return OMEGA_OK;
+    if (!x) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "the gathered rows need the layer input of the last dispatch");
+    OMEGA_HIP_CHECK(m->ctx, launch_dispatch_gather(m, x, T, m->ctx->stream));
+    m->xg_valid = true;
     return OMEGA_OK;
 }
 // x: the rows the shared experts read in fp32 layers (bf16 layers read the packed copy the gather left in xs)
@@ -611,13 +641,18 @@ static int stage_experts(omega_moe *m, const void *x, int T, int which)
 {
     if (m->dispatched_T != T || m->bm != moe_tile_m(m, T))
         OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "experts: dispatch has not run for this T");
+    if (which == 0 && m->gather_on_load && !x) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "experts: x is NULL");
+    if (which == 1 && !m->a_valid) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "experts_down: the up product has not run since `a` was overwritten");
     if (m->cfg.dtype == OMEGA_DTYPE_BF16) OMEGA_HIP_CHECK(m->ctx, launch_experts_bf16(m, x, T, which, m->ctx->stream));
     else OMEGA_HIP_CHECK(m->ctx, launch_experts_f32(m, x, T, which, m->ctx->stream));
+    if (which == 0) m->a_valid = true;
+    else m->y_valid = true;
     return OMEGA_OK;
 }
 static int stage_combine(omega_moe *m, int T, void *out, const void *resid)
 {
     if (m->dispatched_T != T) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "combine: dispatch has not run for this T");
+    if (!m->y_valid) OMEGA_FAIL(m->ctx, OMEGA_ERR_INVALID_ARG, "combine: the down product has not run since `y` was overwritten");
     OMEGA_HIP_CHECK(m->ctx, launch_combine(m, T, out, resid, m->ctx->stream));
     return OMEGA_OK;
 }
@@ -692,10 +727,23 @@ static int forward_impl(omega_moe *m, const void *x, int T, void *out, int block
 int omega_moe_set_training(omega_moe *m, int on)
 {
     MOE_ENTER(m);
+    if (m->training != (on != 0)) m->dispatched_T = -1;  // the dispatch stage prepares different things for the two modes
     m->training = on != 0;
     m->rec_valid = false;
     return OMEGA_OK;
 }
+
+int omega_moe_set_gather_mode(omega_moe *m, int mode)
+{
+    MOE_ENTER(m);
+    if (mode != OMEGA_GATHER_AUTO && mode != OMEGA_GATHER_COPY && mode != OMEGA_GATHER_ON_LOAD)
+        OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "set_gather_mode: unknown mode");
+    if (m->gather_mode != mode) m->dispatched_T = -1;  // the dispatch stage prepares different things for the two forms
+    m->gather_mode = mode;
+    return OMEGA_OK;
+}
+
+int omega_moe_gather_on_load(omega_moe *m) { return m != nullptr && m->gather_on_load ? 1 : 0; }
 
 int omega_moe_forward(omega_moe *m, const void *x, int T, void *out)
 {
@@ -724,6 +772,7 @@ static int backward_impl(omega_moe *m, const void *x, const void *dout, int T, v
     // and meets the gradient of the residual branch
     const void *xin = block ? m->hbuf : x;
     void *dxl = block ? m->bw_dhx : dx;
+    if (bf) RUN(ensure_gathered(m, xin, T));
     OMEGA_HIP_CHECK(ctx, bf ? launch_backward_bf16(m, xin, dout, T, dxl, ctx->stream) : launch_backward_f32(m, xin, dout, T, dxl, ctx->stream));
     if (bf) {  // the pass wrote the states of the weight-gradient blocks into the other copy
         m->bw_zero_phase ^= 1;
@@ -754,6 +803,7 @@ int omega_moe_time_backward(omega_moe *m, const void *x, const void *dout, int T
     if (!dout || !dx || !ms_avg || iters <= 0 || warmup < 0) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "time_backward: bad argument");
     RUN(moe_reserve_backward(m, T));
     const bool bf = m->cfg.dtype == OMEGA_DTYPE_BF16;
+    if (bf) RUN(ensure_gathered(m, x, T));
     for (int i = 0; i < warmup + iters; ++i) {
         if (i == warmup) OMEGA_HIP_CHECK(ctx, hipEventRecord(m->ev0, ctx->stream));
         OMEGA_HIP_CHECK(ctx, bf ? launch_backward_bf16(m, x, dout, T, dx, ctx->stream) : launch_backward_f32(m, x, dout, T, dx, ctx->stream));
@@ -974,7 +1024,7 @@ int omega_moe_experts_up(omega_moe *m, const void *x, int T)
 {
     MOE_ENTER(m);
     stage_invalidates(m);
-    RUN(check_T(m, x, T, m->cfg.Es > 0));
+    RUN(check_T(m, x, T, m->cfg.Es > 0 || m->gather_on_load));
     if (T == 0) return OMEGA_OK;
     if (T > m->T_cap) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "experts: router has not run for this T");
     return stage_experts(m, x, T, 0);
@@ -1090,6 +1140,10 @@ int omega_moe_get_workspace(omega_moe *m, int which, int T, void *host_dst)
     const int cols = which == 1 ? c.H : which == 3 ? 2 * c.H : c.d;
     const size_t es = which == 2 ? 4 : m->esize;
     const bool packed = c.dtype == OMEGA_DTYPE_BF16 && which != 2;
+    if (which == 0 && c.dtype == OMEGA_DTYPE_BF16) {
+        if (m->dispatched_T != T) OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "get_workspace: dispatch has not run for this T");
+        RUN(ensure_gathered(m, m->last_x, T));
+    }
     const void *src = which == 0 ? m->xg : which == 1 ? m->a : which == 3 ? m->bw_dh16 : (const void *)m->y;
     const size_t bytes = m->rows_cap * cols * es;
     std::vector<int32_t> meta(G + 2), off(c.E + 1);
@@ -1125,6 +1179,12 @@ int omega_moe_fill_workspace(omega_moe *m, int which, int byte_value)
         OMEGA_FAIL(ctx, OMEGA_ERR_INVALID_ARG, "fill_workspace: selector must be 1 (a) or 2 (y) and the workspace must exist");
     void *p = which == 1 ? m->a : (void *)m->y;
     const size_t bytes = which == 1 ? m->rows_cap * m->cfg.H * m->esize : m->rows_cap * m->cfg.d * 4;
+    // what the last forward left in the buffer is gone: a backward pass needs a new forward, and the stages that read
+    // the buffer (down product, combine) a new run of the stage that writes it.  (The routing and the dispatch tables
+    // are untouched: omega_moe_experts_up / _down may follow.)
+    stage_invalidates(m);
+    if (which == 1) m->a_valid = false;
+    m->y_valid = false;
     OMEGA_HIP_CHECK(ctx, hipMemsetAsync(p, byte_value, bytes, ctx->stream));
     return OMEGA_OK;
 }

@@ -784,9 +784,10 @@ hipError_t launch_backward_bf16(const omega_moe *m, const void *x, const void *d
     STEP(launch_product_bf16(m, MODE_DA, m->bw_dy16, m->bw_dys16, m->W2T, nullptr, m->bw_dh16, m->bw_h1, m->bw_h3, m->wq_da,
                              c.H, c.d, s));
     // (the forward's down table: where it holds k slices, their partial results go through y_slabs like the forward's)
-    STEP(launch_product_bf16(m, MODE_DOWN, m->bw_dh16, nullptr, m->W13T, nullptr, m->bw_dxg, m->y_slabs, nullptr, m->wq_down, c.d,
-                             2 * c.H, s));
-    if (m->y_slabs != nullptr) STEP(launch_down_slab_reduce(m, m->bw_dxg, s));
+    const bool sliced = m->down_ks_max > 1 || m->down_tail_ks > 1;
+    STEP(launch_product_bf16(m, MODE_DOWN, m->bw_dh16, nullptr, m->W13T, nullptr, m->bw_dxg, sliced ? (void *)m->y_slabs : nullptr,
+                             nullptr, m->wq_down, c.d, 2 * c.H, s));
+    if (sliced) STEP(launch_down_slab_reduce(m, m->bw_dxg, s));
     // weight gradients: the experts' rows become the K axis of transposed images
     STEP(launch_transpose_groups(m, m->bw_dy16, m->bw_dys16, c.d, m->bw_dyT, T, s));
     STEP(launch_transpose_groups(m, m->a, nullptr, c.H, m->bw_aT, T, s));

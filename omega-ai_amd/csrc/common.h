@@ -68,12 +68,18 @@ struct omega_moe {
     int32_t *ids = nullptr;          // [T,K]
     float *w = nullptr;              // [T,K]
     int32_t *tile_counts = nullptr;  // [n_tok_tiles,E] histogram per token tile (router)
-    int32_t *tile_base = nullptr;    // [n_tok_tiles,E] exclusive prefix of tile_counts over the tiles (scan)
     int32_t *counts = nullptr;       // [E]
     int32_t *offsets = nullptr;      // [E+1]
     int32_t *dst = nullptr;          // [T*K] logical row of each pair
     int32_t *dstp = nullptr;         // [T*K] physical row of each pair
     int32_t *src_row = nullptr;      // [T*K]
+    int32_t *tokp = nullptr;         // [rows_cap] token of every physical row of a routed expert (padding rows: stale or 0)
+    // bf16 layers: the up product of this batch fetches the rows of x through tokp itself and no gathered copy exists
+    // (xg / xs hold an earlier batch) until something that needs one asks for it
+    bool gather_on_load = false;
+    int gather_mode = OMEGA_GATHER_AUTO;  // omega_moe_set_gather_mode
+    bool xg_valid = false;
+    const void *last_x = nullptr;    // input of the last dispatch (the caller's buffer, or hbuf in the block form)
     omega_tile *tiles = nullptr;     // [max_m_tiles]
     int32_t *tile_meta = nullptr;    // [0] = number of row tiles; [1+g] = first row tile of group g (G+1 entries);
                                      // [G+2], [G+3] = entries of desc_up, desc_down; [G+4..G+6] = entries of the
@@ -141,6 +147,7 @@ struct omega_moe {
     // the buffers were reallocated).  A stage is refused unless the stage before it ran for the same T, because the
     // index buffers are what the next stage's addresses are formed from.
     int routed_T = -1, dispatched_T = -1;
+    bool a_valid = true, y_valid = true;  // false once omega_moe_fill_workspace has overwritten the buffer
     bool fwd_block = false;          // ... and whether it was the block form
     void *bw_dhx = nullptr;          // [T,d] layer dtype: input gradient of the layer inside the block form
     bool training = false;           // forward keeps h1 / h3 (bf16 layers: as block records in bw_h1 / bw_h3)
@@ -183,7 +190,7 @@ hipError_t launch_rmsnorm(const omega_moe *m, const void *x, int T, void *h, hip
 hipError_t launch_rmsnorm_backward(const omega_moe *m, const void *x, const void *dh, const void *resid, int T, void *dx,
                                    hipStream_t s);
 hipError_t launch_router(const omega_moe *m, const void *x, int T, float *logits_out, float *probs_out, hipStream_t s);
-hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s);
+hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s, const void *x_rows = nullptr);
 hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipStream_t s);
 hipError_t launch_experts_f32(const omega_moe *m, const void *x, int T, int which, hipStream_t s);
 hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s);

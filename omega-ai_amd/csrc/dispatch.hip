@@ -3,59 +3,24 @@
 // Pair p = t*K+j goes to logical row dst[p] = offsets[id_p] + #{q<p : id_q == id_p} of the expert-contiguous
 // order (a stable counting sort of the pair list by expert id); src_row[dst[p]] = t.  In the buffers the
 // experts' segments start on row-tile boundaries (physical row dstp[p] = first_tile[id_p]*bm + rank).
-// The router left one histogram row per token tile (16 or 32 tokens, router_tok_tile) in tile_counts[tile][e].  Two
-// launches - three when the histogram is large:
-//   scan    (histograms above 16384 cells only) one workgroup per 8 experts: exclusive prefix over the tiles of each
-//           expert (tile_base) and the per-expert totals -> counts[e]
-//   rank    one workgroup per token tile: the prefix of its tile and the totals (summed from the histogram rows in the
-//           same pass unless a scan launch left them); offsets = exclusive scan of counts, first_tile = exclusive scan
-//           of ceil(counts/bm); rank of each pair among the earlier pairs of its tile with the same expert (ballots
-//           within 64-pair chunks, per-chunk counts across them); dst/dstp/src_row; workgroup g (mod grid) writes the
-//           row tiles and the work items of group g, workgroup 0 publishes counts, offsets and the totals
-//   gather  one wave per token: the row of x is read once with 16-byte accesses and written to its K
-//           destination rows (gather semantics as img_token_drop,
-//           J/engine/nn/layer/dit/kernel/TokenDropKernel.cu:147-160); fp32 layers keep rows contiguous,
-//           bf16 layers write the packed tile image the product kernels load (pack.h)
-// No global atomics anywhere, so counts, offsets and the permutation are deterministic.
+// The router left one histogram row per token tile (16 or 32 tokens, router_tok_tile) in tile_counts[tile][e].  One launch (fp32 layers: two):
+//   rank    one workgroup per token tile: the prefix of its tile and the experts' totals, summed from the histogram
+//           rows in the same pass (a single-pass scan: no workgroup waits for another); offsets = exclusive scan of the
+//           totals, first_tile = exclusive scan of ceil(totals/bm); rank of each pair among the earlier pairs of its
+//           tile with the same expert (ballots within 64-pair chunks, per-chunk counts across them); dst / dstp /
+//           src_row / tokp; the row-tile list and the work-item tables; workgroup 0 publishes counts, offsets and the
+//           totals.  bf16 layers: the workgroup then copies the rows of its own tile into the packed image of the
+//           gathered rows (copy_tile_rows) - unless the up product fetches them itself (tokp) -, and the launch's
+//           first workgroups build the product kernels' per-workgroup queues from the same totals (schedule_queues)
+//   gather  (fp32 layers, and bf16 rows asked for after the fact) one wave per token: the row of x is read once with
+//           16-byte accesses and written to its K destination rows (gather semantics as img_token_drop,
+//           J/engine/nn/layer/dit/kernel/TokenDropKernel.cu:147-160)
+// No floating-point or order-dependent atomics anywhere: counts, offsets and the permutation are deterministic.
 #include "common.h"
 #include "pack.h"
 
 #define TOK_TILE_MAX ROUTER_TOK_TILE_MAX
-#define SCAN_EC 8     // experts per scan workgroup
-#define SCAN_SEG 32   // tile segments per expert
 
-__global__ __launch_bounds__(256) void dispatch_scan_kernel(const int32_t *__restrict__ tile_counts,
-                                                            int32_t *__restrict__ tile_base, int n_tiles, int E,
-                                                            int32_t *__restrict__ counts)
-{
-    __shared__ int segsum[SCAN_SEG][SCAN_EC];
-    const int el = threadIdx.x % SCAN_EC, seg = threadIdx.x / SCAN_EC;
-    const int e = blockIdx.x * SCAN_EC + el;
-    const int per = ceil_div(n_tiles, SCAN_SEG);
-    const int b = min(seg * per, n_tiles), en = min(b + per, n_tiles);
-    int sum = 0;
-    if (e < E)
-        for (int t = b; t < en; ++t) sum += tile_counts[(size_t)t * E + e];
-    segsum[seg][el] = sum;
-    __syncthreads();
-    int base = 0, total = 0;
-    for (int s2 = 0; s2 < SCAN_SEG; ++s2) {
-        const int v = segsum[s2][el];
-        if (s2 < seg) base += v;
-        total += v;
-    }
-    if (e < E) {
-        if (seg == 0) counts[e] = total;
-        for (int t = b; t < en; ++t) {
-            const int c = tile_counts[(size_t)t * E + e];
-            tile_base[(size_t)t * E + e] = base;
-            base += c;
-        }
-    }
-}
-
-// The work items of group g in one product's table (see the comment in dispatch_rank_kernel): NT column tiles of
-// ncols columns, Mg row tiles starting at row tile mt0; the launch has total_mt row tiles in all.  All 256 threads.
 // K slices of a table (small batches of the down product, see write_group_items): Nt output tiles that would leave
 // at least half of the 256 compute units idle are each cut into KS <= ks_max slices of the k range, at least 8 k steps
 // long; 1 = no slicing.
@@ -82,118 +47,395 @@ __device__ __forceinline__ int table_tail_k_slices(int Nt, int tail_ks, int KT)
 // this is cut into row blocks of about equal size, each of which walks all column tiles.
 #define OMEGA_ROW_BLOCK_MAX 8
 
+// a / b for 0 <= a < 2^22, 0 < b < 2^22 through the float reciprocal (a quarter of the instructions of the integer
+// division the compiler emits); exact: the estimate is off by at most one, and is corrected
+__device__ __forceinline__ int small_div(int a, int b)
+{
+    int q = (int)((float)a * __builtin_amdgcn_rcpf((float)b));
+    const int r = a - q * b;
+    q += r >= b ? 1 : 0;
+    q -= r < 0 ? 1 : 0;
+    return q;
+}
+
+// What a product's table is made for: NT column tiles of ncols columns; k slices as table_k_slices / table_tail_k_slices
+struct table_params {
+    int NT, ncols, ks_max, KT, tail_ks;
+};
+
+// How the tiles of a launch with total_mt row tiles map to table entries: the first Nt - r tiles are one entry each;
+// when the last r = Nt mod 256 tiles would occupy at most half of the compute units, each of them is `per` adjacent
+// entries - k slices (down product, long k) or S = 256/r (2..4) slices of its 32-row blocks -, so that the slices of a
+// tile run side by side on one XCD and share operand tiles in its L2; a small batch has every tile in KS k slices.
+struct table_shape {
+    int Nt, r, KS, TKS, S;
+    __device__ __forceinline__ table_shape(const table_params &tp, int total_mt)
+    {
+        Nt = total_mt * tp.NT;
+        r = Nt % 256;
+        KS = table_k_slices(Nt, tp.ks_max, tp.KT);
+        TKS = KS > 1 ? 1 : table_tail_k_slices(Nt, tp.tail_ks, tp.KT);
+        S = (r == 0 || r > 128 || KS > 1 || TKS > 1) ? 1 : min(4, 256 / r);
+    }
+    __device__ __forceinline__ int per(int at) const { return KS > 1 ? KS : at < Nt - r ? 1 : TKS > 1 ? TKS : S; }
+    __device__ __forceinline__ int first(int at) const { return KS > 1 ? at * KS : at < Nt - r ? at : Nt - r + (at - (Nt - r)) * per(at); }
+    __device__ __forceinline__ int entries() const { return KS > 1 ? Nt * KS : Nt - r + r * (TKS > 1 ? TKS : S); }
+    // tile and slice of entry `ent`
+    __device__ __forceinline__ void locate(int ent, int &at, int &sub) const
+    {
+        at = ent;
+        sub = 0;
+        if (KS > 1) {
+            at = small_div(ent, KS);
+            sub = ent - at * KS;
+        } else if (ent >= Nt - r) {
+            const int p = TKS > 1 ? TKS : S, ti = small_div(ent - (Nt - r), p);
+            at = Nt - r + ti;
+            sub = ent - (Nt - r) - ti * p;
+        }
+    }
+};
+
+// Slice `sub` of tile `at` of a table, a tile of group g (rows rows in Mg row tiles from row tile mt0 on).
+// Order within a group: row blocks of at most OMEGA_ROW_BLOCK_MAX row tiles; inside a row block column tile after
+// column tile, the row tiles of the block fastest.  (Walking the column tiles twice, first with the taller row tiles
+// and then with the others, makes most rounds of 32 entries cost the same, so that the queue builder has nothing to
+// deal: dispatch 50 -> 39 us at the Mixtral shape, but its up product 1.529 -> 1.544 ms - each weight tile is then
+// fetched twice.)
+// The group's rows are dealt evenly, in blocks of 32, to its Mg row tiles (instead of full tiles and a ragged last
+// one): the same number of tiles and of MFMA blocks, but tiles of nearly one cost.  (Equal tiles in units of 16 rows -
+// every tile the same number of MFMA blocks, the last one of each half empty - cut the L2 miss traffic of the up
+// product by a fifth when every expert has 1040 rows, and still lost 4 % of time to the extra blocks.)
+__device__ __forceinline__ omega_tile_desc group_item(const table_params &tp, const table_shape &ts, int at, int sub, int g,
+                                                      int rows, int Mg, int mt0, int bm, bool shared)
+{
+    const int NT = tp.NT, l = at - mt0 * NT;
+    const int nblk = (rows + 31) >> 5;
+    const int qblk = small_div(nblk, Mg), nhi = nblk - qblk * Mg;  // the first nhi row tiles hold qblk + 1 blocks, the others qblk
+    const int NB = (Mg + OMEGA_ROW_BLOCK_MAX - 1) / OMEGA_ROW_BLOCK_MAX;
+    int f = 0, RB = Mg;
+    if (NB > 1) {
+        // row block b holds row tiles [b*Mg/NB, (b+1)*Mg/NB); the entries before it number (first tile) * NT
+        int b = min(NB - 1, small_div(small_div(l, NT) * NB, Mg));
+        while (small_div(b * Mg, NB) * NT > l) --b;
+        while (b + 1 < NB && small_div((b + 1) * Mg, NB) * NT <= l) ++b;
+        f = small_div(b * Mg, NB);
+        RB = small_div((b + 1) * Mg, NB) - f;
+    }
+    const int li = l - f * NT;
+    const int n = small_div(li, RB), mt = f + li - n * RB;
+    const int tfirst = 32 * (mt * qblk + min(mt, nhi));
+    const int trows = min(32 * ((mt + 1) * qblk + min(mt + 1, nhi)), rows) - tfirst;
+    const int ent = ts.first(at) + sub;
+    omega_tile_desc dsc;
+    dsc.g = g;
+    dsc.n0 = n * tp.ncols;
+    dsc.a_rg = 0;
+    dsc.b_rg = tp.ncols == 128 ? 1 : 0;  // read by the plain 256-column products only: a half-width item
+    // (items without k slices: kt0 = first 32 x 32 block record of the item - 8 records per row-tile slot - for the
+    //  products that keep or read h1 / h3 block records)
+    dsc.kt0 = (mt0 + mt) * 8;
+    dsc.row0 = mt0 * bm + tfirst;
+    dsc.rows = trows;
+    dsc.xrow0 = shared ? tfirst : -1;
+    if (ts.KS > 1 || (at >= ts.Nt - ts.r && ts.TKS > 1)) {
+        // slice `sub` of a_rg slices of the k range (kt0 = slice, xrow0 = number of the sliced entry = of its partial
+        // result)
+        dsc.a_rg = ts.KS > 1 ? ts.KS : ts.TKS;
+        dsc.kt0 = sub;
+        dsc.xrow0 = ts.KS > 1 ? ent : ent - (ts.Nt - ts.r);
+    } else if (at >= ts.Nt - ts.r && ts.S > 1) {
+        const int tb = (trows + 31) >> 5;  // the tile's 32-row blocks, dealt evenly to the S slices
+        const int sfirst = 32 * small_div(sub * tb, ts.S);
+        dsc.row0 += sfirst;
+        dsc.rows = max(0, min(32 * small_div((sub + 1) * tb, ts.S), trows) - sfirst);  // 0: nothing to do
+        dsc.xrow0 = shared ? tfirst + sfirst : -1;
+        dsc.kt0 += sfirst >> 5;
+    }
+    return dsc;
+}
+
+// The work item at place `ent` of a table, from the groups' row counts alone (mt_s[g] = first row tile of group g,
+// mt_s[G] = all row tiles; off_s[e] = first logical row of expert e; a shared expert holds T rows): whoever needs an
+// entry - the table writers, the queue builders - forms it without waiting for anybody else.
+__device__ __forceinline__ omega_tile_desc item_desc(int ent, const table_params &tp, const table_shape &ts, const int *mt_s,
+                                                     const int *off_s, int E, int G, int T, int bm)
+{
+    int at, sub;
+    ts.locate(ent, at, sub);
+    // the group of tile `at`: the last g with first_tile[g]*NT <= at (groups without rows have no tiles and are passed over)
+    int lo = 0, hi = G;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (mt_s[mid] * tp.NT <= at) lo = mid;
+        else hi = mid;
+    }
+    const int g = lo;
+    return group_item(tp, ts, at, sub, g, g < E ? off_s[g + 1] - off_s[g] : T, mt_s[g + 1] - mt_s[g], mt_s[g], bm, g >= E);
+}
+
+// The table entries of group g, written by the 256 threads of a workgroup.
 __device__ __forceinline__ void write_group_items(omega_tile_desc *__restrict__ desc, int NT, int ncols, int g, int rows,
                                                   int Mg, int mt0, int total_mt, int bm, bool shared, int ks_max = 1,
                                                   int KT = 0, int tail_ks = 1)
 {
     if (desc == nullptr) return;
-    const int Nt = total_mt * NT, r = Nt % 256;
-    const int KS = table_k_slices(Nt, ks_max, KT);
-    const int TKS = KS > 1 ? 1 : table_tail_k_slices(Nt, tail_ks, KT);
-    const int S = (r == 0 || r > 128 || KS > 1 || TKS > 1) ? 1 : min(4, 256 / r);
-    // the group's rows are dealt evenly, in blocks of 32, to its Mg row tiles (instead of full tiles and a ragged last
-    // one): the same number of tiles and of MFMA blocks, but tiles of nearly one cost.  (Equal tiles in units of 16 rows -
-    // every tile the same number of MFMA blocks, the last one of each half empty - cut the L2 miss traffic of the up
-    // product by a fifth when every expert has 1040 rows, and still lost 4 % of time to the extra blocks.)
-    const int nblk = (rows + 31) >> 5;
-    const int qblk = nblk / Mg, nhi = nblk % Mg;  // the first nhi row tiles hold qblk + 1 blocks, the others qblk
-    // order within the group: row blocks of RB row tiles; inside a row block column tile after column tile, the row
-    // tiles of the block fastest.  (Walking the column tiles twice, first with the taller row tiles and then with the
-    // others, makes most rounds of 32 entries cost the same, so that the queue builder has nothing to deal: dispatch
-    // 50 -> 39 us at the Mixtral shape, but its up product 1.529 -> 1.544 ms - each weight tile is then fetched twice.)
-    const int NB = (Mg + OMEGA_ROW_BLOCK_MAX - 1) / OMEGA_ROW_BLOCK_MAX;
+    const table_params tp = {NT, ncols, ks_max, KT, tail_ks};
+    const table_shape ts(tp, total_mt);
     for (int l = threadIdx.x; l < Mg * NT; l += 256) {
-        // row block b holds row tiles [b*Mg/NB, (b+1)*Mg/NB); the entries before it number (first tile) * NT
-        int b = min(NB - 1, (l / NT) * NB / Mg);
-        while ((b * Mg) / NB * NT > l) --b;
-        while (b + 1 < NB && ((b + 1) * Mg) / NB * NT <= l) ++b;
-        const int f = (b * Mg) / NB, RB = ((b + 1) * Mg) / NB - f;
-        const int li = l - f * NT;
-        const int mt = f + li % RB, n = li / RB;
-        const int at = mt0 * NT + l;
-        const int tfirst = 32 * (mt * qblk + min(mt, nhi));
-        const int trows = min(32 * ((mt + 1) * qblk + min(mt + 1, nhi)), rows) - tfirst;
-        omega_tile_desc dsc;
-        dsc.g = g;
-        dsc.n0 = n * ncols;
-        dsc.a_rg = 0;
-        dsc.b_rg = ncols == 128 ? 1 : 0;  // read by the plain 256-column products only: a half-width item
-        // (items without k slices: kt0 = first 32 x 32 block record of the item - 8 records per row-tile slot - for the
-        //  products that keep or read h1 / h3 block records)
-        dsc.kt0 = (mt0 + mt) * 8;
-        if (KS > 1) {
-            // slice ks of KS (a_rg = KS, kt0 = ks, xrow0 = number of the sliced entry = of its partial result) runs over
-            // its part of the k range; adjacent entries, so the slices of a tile run on one XCD and share its rows
-            dsc.row0 = mt0 * bm + tfirst;
-            dsc.rows = trows;
-            dsc.a_rg = KS;
-            for (int ks = 0; ks < KS; ++ks) {
-                dsc.kt0 = ks;
-                dsc.xrow0 = at * KS + ks;
-                desc[at * KS + ks] = dsc;
-            }
-        } else if (at < Nt - r) {
-            dsc.row0 = mt0 * bm + tfirst;
-            dsc.rows = trows;
-            dsc.xrow0 = shared ? tfirst : -1;
-            desc[at] = dsc;
-        } else if (TKS > 1) {
-            // one of the last r tiles of a large launch, as TKS k slices (fields as above)
-            const int ti = at - (Nt - r);
-            dsc.row0 = mt0 * bm + tfirst;
-            dsc.rows = trows;
-            dsc.a_rg = TKS;
-            for (int ks = 0; ks < TKS; ++ks) {
-                dsc.kt0 = ks;
-                dsc.xrow0 = ti * TKS + ks;
-                desc[Nt - r + ti * TKS + ks] = dsc;
-            }
-        } else {
-            const int tb = (trows + 31) >> 5;  // the tile's 32-row blocks, dealt evenly to the S slices
-            const int rec0 = dsc.kt0;
-            for (int sl = 0; sl < S; ++sl) {
-                const int sfirst = 32 * ((sl * tb) / S);
-                dsc.row0 = mt0 * bm + tfirst + sfirst;
-                dsc.rows = max(0, min(32 * (((sl + 1) * tb) / S), trows) - sfirst);  // 0: nothing to do
-                dsc.xrow0 = shared ? tfirst + sfirst : -1;
-                dsc.kt0 = rec0 + (sfirst >> 5);
-                desc[Nt - r + (at - (Nt - r)) * S + sl] = dsc;
-            }
-        }
+        const int at = mt0 * NT + l, per = ts.per(at), first = ts.first(at);
+        for (int q = 0; q < per; ++q) desc[first + q] = group_item(tp, ts, at, q, g, rows, Mg, mt0, bm, shared);
     }
 }
 
 // entries of a table whose launch has total_mt row tiles and NT column tiles (with the last tiles sliced)
 __device__ __forceinline__ int table_entries(int total_mt, int NT, int ks_max = 1, int KT = 0, int tail_ks = 1)
 {
-    const int Nt = total_mt * NT, r = Nt % 256;
-    const int KS = table_k_slices(Nt, ks_max, KT);
-    if (KS > 1) return Nt * KS;
-    const int TKS = table_tail_k_slices(Nt, tail_ks, KT);
-    if (TKS > 1) return Nt - r + r * TKS;
-    const int S = (r == 0 || r > 128) ? 1 : min(4, 256 / r);
-    return Nt - r + r * S;
+    const table_params tp = {NT, 0, ks_max, KT, tail_ks};
+    return table_shape(tp, total_mt).entries();
+}
+
+// Per-workgroup queues of the persistent product kernels.  A product launch has n_wg workgroups, one per compute
+// unit; workgroup w runs on XCD w % 8.  The table is consumed in rounds of n_wg consecutive entries, XCD x taking a
+// contiguous eighth of each round (of what is left, in the last one), so the tiles in flight on one XCD are
+// neighbours in the table and share operand tiles in its L2.  Within a round the entries of an XCD are dealt to its
+// workgroups cheapest entry to the workgroup with the most work so far (ragged row tiles cost less than full ones),
+// which keeps the queues' total work level without any run-time arbitration.
+// One workgroup of 256 threads per (product, XCD).  Per chunk of SCHED_RC rounds: all threads fetch the costs and rank
+// the entries of every round by cost; wave 0 deals the rounds one after the other (lane j < n_wg/8 stands for
+// workgroup j*8 + x; what depends on the round before is only the order of the workgroups by work, 32 keys ranked by
+// the 64 lanes against 16 keys each out of LDS); all threads write the descriptors to their queue slots.
+#define SCHED_RC 128  // rounds per chunk
+#define SCHED_WGS 16  // 2 products x 8 XCDs
+#define SCHED_SCRATCH (5 * SCHED_RC * 32 + 256)  // bytes of LDS schedule_queues works in
+
+__device__ __forceinline__ int work_item_cost(int rows)
+{
+    if (rows <= 0) return 0;
+    const int nb = (rows + 31) >> 5;  // 32-row MFMA blocks of the item (the two waves of a SIMD share them)
+    return 2 + (14 * nb) / 8;         // sixteenths of a full tile; the loads and the fixed part do not shrink
+}
+
+// where the entries of a table come from: the table in memory (the backward pass's products) ...
+struct table_source {
+    const omega_tile_desc *desc;
+    int kcost;  // 0: an item costs by its rows; 1: by its k steps (weight-gradient items, all 256 rows high)
+    __device__ __forceinline__ int cost(int L) const
+    {
+        return kcost ? min(255, 2 + desc[L].xrow0 / 8) : work_item_cost(desc[L].rows);
+    }
+    __device__ __forceinline__ omega_tile_desc get(int L) const { return desc[L]; }
+};
+// ... or the groups' row counts (the forward pass: the queue builders run beside the table writers, not behind them)
+struct analytic_source {
+    table_params tp;
+    table_shape ts;
+    const int *mt_s, *off_s;
+    int E, G, T, bm;
+    __device__ __forceinline__ omega_tile_desc get(int L) const { return item_desc(L, tp, ts, mt_s, off_s, E, G, T, bm); }
+    __device__ __forceinline__ int cost(int L) const { return work_item_cost(get(L).rows); }
+};
+
+// (Dealing the rounds of a table in 2 or 4 independent chains, one workgroup each, shortens the one step that depends
+// on the round before - the order of the workgroups by work - and was measured: the queue builders finish 5-9 us
+// earlier, and the up product of 4096 tokens x 8 experts loses 2 %, 30 us, to the coarser levelling.)
+template <class Source>
+__device__ __forceinline__ void schedule_queues(const Source &src, omega_tile_desc *__restrict__ wq, int total, int n_wg, int x,
+                                                unsigned char *scratch)
+{
+    unsigned char *cost_s = scratch;                                            // [round][place]
+    unsigned short *sorted_s = (unsigned short *)(scratch + SCHED_RC * 32);     // [round][p] = cost << 8 | place of the p-th cheapest entry
+    unsigned short *place_s = (unsigned short *)(scratch + 3 * SCHED_RC * 32);  // [round][workgroup j] = 0x8000 | (queue slot - len0) << 5 | source place
+    int *len0_s = (int *)(scratch + 5 * SCHED_RC * 32);
+    int *keys_s = len0_s + 32;
+    const int tid = threadIdx.x, lane = tid & 63, nthr = blockDim.x;
+    const int wpx = n_wg >> 3;
+    const int rounds = (total + n_wg - 1) / n_wg;
+    // entry of (round r, place i of this XCD), or -1
+    auto entry = [&](int r, int i) {
+        const int base = r * n_wg, left = min(n_wg, total - base);
+        const int per = (left + 7) >> 3;
+        const int L = base + x * per + i;
+        return (i < per && L < base + left) ? L : -1;
+    };
+    // wave 0, lanes j and j + 32 alike: total cost and length of the queue of workgroup j*8 + x
+    int work = 0, len = 0;
+    for (int r0 = 0; r0 < rounds; r0 += SCHED_RC) {
+        const int nr = min(SCHED_RC, rounds - r0);
+        for (int idx = tid; idx < nr * 32; idx += nthr) {
+            const int L = entry(r0 + (idx >> 5), idx & 31);
+            cost_s[idx] = (unsigned char)(L >= 0 ? src.cost(L) : 0);
+        }
+        if (tid < 32) len0_s[tid] = len;
+        __syncthreads();
+        // every round's entries in the order of rising cost (ties to the lower place; places that stand for no workgroup
+        // stay where they are): keys are unique, so an entry's rank is a count of smaller keys
+        for (int idx = tid; idx < nr * 32; idx += nthr) {
+            const int i = idx & 31;
+            const uint4 *cs = (const uint4 *)(cost_s + (idx & ~31));
+            const uint4 lo = cs[0], hi = cs[1];
+            const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            const int c = cost_s[idx], key = (c << 5) | i;
+            int rk = 0;
+#pragma unroll
+            for (int o = 0; o < 32; ++o) {
+                const int ko = (int)(((w[o >> 2] >> ((o & 3) * 8)) & 255) << 5) | o;
+                rk += (o < wpx && ko < key) ? 1 : 0;
+            }
+            sorted_s[(idx & ~31) + (i < wpx ? rk : i)] = (unsigned short)((c << 8) | i);
+        }
+        __syncthreads();
+        if (tid < 64) {
+            const int i = lane & 31, h = lane >> 5;
+            int c_next = cost_s[i];
+            for (int r = 0; r < nr; ++r) {
+                const int c = c_next;
+                c_next = r + 1 < nr ? cost_s[(r + 1) * 32 + i] : 0;
+                int ce, srcp;
+                // a round whose entries all cost the same (the common case: tiles of one expert after the even split)
+                // needs no dealing - it adds the same work to every queue: each workgroup takes the entry of its place
+                const int c0 = __builtin_amdgcn_readfirstlane(c);
+                if (__ballot(i < wpx && c != c0) == 0) {
+                    ce = c;
+                    srcp = i;
+                } else {
+                    // place of the workgroup by falling work (ties to the lower workgroup): lanes i and i + 32 count the
+                    // larger keys among 16 keys each; the workgroup at place p takes the p-th cheapest entry
+                    const int key = i < wpx ? (work << 6) | (63 - i) : -1;
+                    if (lane < 32) keys_s[lane] = key;
+                    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // one wave: its LDS accesses complete in order
+                    const int4 *kp = (const int4 *)(keys_s + 16 * h);
+                    const int4 k0 = kp[0], k1 = kp[1], k2 = kp[2], k3 = kp[3];
+                    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                    const int cnt = (k0.x > key) + (k0.y > key) + (k0.z > key) + (k0.w > key) + (k1.x > key) + (k1.y > key) +
+                                    (k1.z > key) + (k1.w > key) + (k2.x > key) + (k2.y > key) + (k2.z > key) + (k2.w > key) +
+                                    (k3.x > key) + (k3.y > key) + (k3.z > key) + (k3.w > key);
+                    const int rank_w = i < wpx ? cnt + __shfl_xor(cnt, 32, 64) : i;
+                    const int mine = sorted_s[r * 32 + rank_w];
+                    ce = mine >> 8;
+                    srcp = mine & 31;
+                }
+                unsigned short pl = 0;
+                if (i < wpx && ce > 0) {
+                    pl = (unsigned short)(0x8000 | ((len - len0_s[i]) << 5) | srcp);
+                    work += ce;
+                    ++len;
+                }
+                if (lane < 32) place_s[r * 32 + lane] = pl;
+            }
+        }
+        __syncthreads();
+        for (int idx = tid; idx < nr * 32; idx += nthr) {
+            const unsigned short pl = place_s[idx];
+            if (pl) {
+                const omega_tile_desc d = src.get(entry(r0 + (idx >> 5), pl & 31));
+                wq[(size_t)(len0_s[idx & 31] + ((pl >> 5) & 0x3ff)) * n_wg + (idx & 31) * 8 + x] = d;
+            }
+        }
+        __syncthreads();
+    }
+    if (tid < wpx) {  // a queue ends with an entry without rows
+        omega_tile_desc z = {};
+        wq[(size_t)len * n_wg + tid * 8 + x] = z;
+    }
+}
+
+// up to three tables per launch: table p is scheduled by workgroups 8p .. 8p+7
+struct sched_args {
+    const omega_tile_desc *desc[3];
+    omega_tile_desc *wq[3];
+    int total_slot[3];  // index in tile_meta of the table's number of entries
+    int kcost[3];       // see table_source
+    const int32_t *tile_meta;
+    int n_wg;
+};
+
+// The rows of one token tile into the packed image of the gathered rows (and of the shared experts' copy), by the
+// workgroup that has just ranked the tile's pairs (gather semantics as img_token_drop,
+// J/engine/nn/layer/dit/kernel/TokenDropKernel.cu:147-160).  In the packed image rows 2i and 2i+1 share every 128-byte
+// line (64 bytes of a k step each).  The tile's pairs, sorted by destination row (pairs of one expert are
+// consecutive rows), are therefore copied in units of such a row pair where the tile holds both rows: 8 lanes write one
+// whole line (4 lanes per row), an instruction covers 8 k steps of the two rows; a row whose neighbour belongs to
+// another tile goes by itself, 16 k steps per instruction.  (A wave per token writing 64-byte pieces wrote 1.4 times
+// the bytes of the rows.)  The source rows are read in the same pattern, 512 or 1024 contiguous bytes of a row per
+// instruction; a token's row is read K times, all but the first out of the L2.
+template <bool NT>
+__device__ __forceinline__ void copy_tile_rows(const unsigned char *__restrict__ x, int d, int t0, int ntok, int npairs,
+                                               const int *sort_prow, const unsigned char *sort_tok,
+                                               unsigned char *__restrict__ xg, unsigned char *__restrict__ xs)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    const int KT = d >> 5;
+    const size_t row_bytes = (size_t)d * 2;
+    const int n_units = npairs + (xs != nullptr ? (ntok + 1) >> 1 : 0);
+    for (int u = wave; u < n_units; u += n_waves) {
+        // unit: destination row pa (token ta), and row pa + 1 (token tb) with it if it belongs to the tile as well
+        int pa, ta, tb = -1;
+        unsigned char *base = xg;
+        if (u < npairs) {
+            pa = sort_prow[u];
+            if (u > 0 && (pa & 1) && sort_prow[u - 1] == pa - 1) continue;  // the second row of the unit before
+            ta = sort_tok[u];
+            if (!(pa & 1) && u + 1 < npairs && sort_prow[u + 1] == pa + 1) tb = sort_tok[u + 1];
+        } else {
+            ta = 2 * (u - npairs);
+            pa = t0 + ta;  // row t of the shared experts' copy is token t; t0 is even
+            if (ta + 1 < ntok) tb = ta + 1;
+            base = xs;
+        }
+        const bool two = tb >= 0;
+        // lane -> (row of the unit, k step within the instruction, chunk)
+        const int sel = two ? (lane >> 2) & 1 : 0, kk = two ? lane >> 3 : lane >> 2, kpi = two ? 8 : 16, c = lane & 3;
+        const int prow = pa + sel;
+        const unsigned char *src = x + (size_t)(t0 + (sel ? tb : ta)) * row_bytes + c * 16;
+        for (int kb0 = 0; kb0 < KT; kb0 += kpi * 4) {
+            uint4 v[4];  // 4 KiB in flight per wave, 16 waves (the kernel keeps to 64 registers: two workgroups per compute unit)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int kb = kb0 + q * kpi + kk;
+                v[q] = kb < KT ? *(const uint4 *)(src + (size_t)kb * 64) : uint4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int kb = kb0 + q * kpi + kk;
+                if (kb < KT) {
+                    unsigned char *o = base + pk_chunk_off(prow, kb, c, KT);
+                    if (NT) {
+                        typedef unsigned v4u __attribute__((ext_vector_type(4)));
+                        const v4u t4 = {v[q].x, v[q].y, v[q].z, v[q].w};
+                        __builtin_nontemporal_store(t4, (v4u *)o);
+                    } else {
+                        *(uint4 *)o = v[q];
+                    }
+                }
+            }
+        }
+    }
 }
 
 // MAXE: experts are limited to 256 per layer by the router kernels.
 #define MAXE 256
 #define RANK_CHUNKS (TOK_TILE_MAX * 64 / 64)  // 64-pair chunks of the largest token tile (K <= 64)
-// FUSED: the workgroup forms the prefix of its token tile over the tiles before it, and the per-expert totals, from
-// the router's histogram rows itself (a single pass: no scan launch in front; used while the histogram is small enough
-// for every workgroup to read all of it); else tile_base / counts come from dispatch_scan_kernel.
-template <bool FUSED>
-__global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__restrict__ ids,
+// One workgroup per token tile, behind n_sched workgroups that build the product kernels' queues (see the head of the file).
+// 256 threads, or 1024 when the workgroups copy rows (x / xg given): the index work is done by the first 256; the
+// kernel keeps to 64 registers so that two such workgroups share a compute unit and the queue builders run beside the
+// tiles' workgroups, not behind them.
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void dispatch_rank_kernel(const int32_t *__restrict__ ids,
                                                             const int32_t *__restrict__ tile_counts,
-                                                            const int32_t *__restrict__ tile_base,
                                                             int32_t *__restrict__ counts, int n_tiles, int T, int tok_tile,
                                                             int K, int E, int Es, int bm, int32_t *__restrict__ offsets,
                                                             int32_t *__restrict__ dst, int32_t *__restrict__ dstp,
-                                                            int32_t *__restrict__ src_row,
+                                                            int32_t *__restrict__ src_row, int32_t *__restrict__ tokp,
                                                             omega_tile *__restrict__ tiles,
                                                             int32_t *__restrict__ tile_meta,
                                                             omega_tile_desc *__restrict__ desc_up, int nt_up, int ncols_up,
                                                             omega_tile_desc *__restrict__ desc_down, int nt_down,
-                                                            int ncols_down, int ks_max_down, int kt_down, int tail_ks_down)
+                                                            int ncols_down, int ks_max_down, int kt_down, int tail_ks_down,
+                                                            omega_tile_desc *__restrict__ wq_up,
+                                                            omega_tile_desc *__restrict__ wq_down, int n_wg,
+                                                            const unsigned char *__restrict__ x, int d,
+                                                            unsigned char *__restrict__ xg, unsigned char *__restrict__ xs,
+                                                            int nt_stores, int n_sched)
 {
     __shared__ int off_s[MAXE + 1];        // logical first row of each expert
     __shared__ int mt_s[MAXE + 64 + 1];    // first row tile of each group (routed, then shared)
@@ -201,56 +443,105 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     __shared__ int base_s[MAXE];           // pairs of each expert in the token tiles before this one
     __shared__ int tot_s[MAXE];            // pairs of each expert in the whole batch
     __shared__ int part_s[2][256];
-    __shared__ int ccount[RANK_CHUNKS][MAXE];  // pairs of each expert in each 64-pair chunk of this tile
-    const int tid = threadIdx.x, tile = blockIdx.x, lane = tid & 63, wave = tid >> 6;
+    // pairs of each expert in each 64-pair chunk of this tile; the queue builders, which rank nothing, work in it
+    __shared__ __attribute__((aligned(16))) int ccount[RANK_CHUNKS][MAXE];
+    static_assert(sizeof(int) * RANK_CHUNKS * MAXE >= SCHED_SCRATCH, "the queue builders' scratch fits the chunk counts");
+    // the tile's pairs in the order of their destination rows (row copies by this workgroup): row and token within the tile
+    __shared__ __attribute__((aligned(16))) int sort_prow[TOK_TILE_MAX * 64];
+    __shared__ unsigned char sort_tok[TOK_TILE_MAX * 64];
+    // (256 threads, or 1024 when the workgroup copies rows as well: the index work is done by the first 256)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthr = blockDim.x;
+    // the first n_sched workgroups build the product kernels' queues (bf16 layers): they need the experts' totals and
+    // the scans of them like everybody else, and nothing that another workgroup of this launch writes
+    const bool sched = (int)blockIdx.x < n_sched;
+    const int tile = sched ? n_tiles : (int)blockIdx.x - n_sched;
     const int t0 = tile * tok_tile;
-    const int npairs = min(tok_tile, T - t0) * K;
+    const int npairs = sched ? 0 : min(tok_tile, T - t0) * K;
     const int nchunks = (npairs + 63) >> 6;
 
-    for (int i = tid; i < npairs; i += 256) id_s[i] = ids[(size_t)t0 * K + i];
-    for (int i = tid; i < nchunks * E; i += 256) ccount[i / E][i % E] = 0;
-    if (FUSED) {
-        // thread (segment s of the tiles, expert e): pairs of e in its tiles, and in those of them before this tile
+    // (row copies: the tile's rows are asked for now, one load per 128-byte line, so that they travel while the index
+    //  work below keeps the memory idle; the copies then find them in the L2 or the last-level cache)
+    int prefetched = 0;
+    if (xg != nullptr && !sched) {
+        const size_t tile_bytes = (size_t)min(tok_tile, T - t0) * d * 2;
+        const unsigned char *xt = x + (size_t)t0 * d * 2;
+        for (size_t o = (size_t)tid * 128; o < tile_bytes; o += (size_t)nthr * 128) prefetched ^= *(const int *)(xt + o);
+    }
+    for (int i = tid; i < npairs; i += nthr) id_s[i] = ids[(size_t)t0 * K + i];
+    for (int i = tid; i < nchunks * E; i += nthr) ccount[i / E][i % E] = 0;
+    {
+        // thread (segment s of the token tiles, expert e): pairs of e in its tiles, and in those of them before this tile.
+        // Every workgroup sums the whole histogram itself, so nobody waits for a scan launch or for another workgroup
+        // (a second level of sums written by the router's last-arriving workgroups was tried: the device-scope fences
+        // it needs between workgroups on different XCDs cost the router 30-45 us at 8192-16384 tokens).
+        // Rows whose length is a multiple of four experts are read 16 bytes at a time (a quarter of the loads; the
+        // partial sums then take four times the room and borrow the row-copy lists, which are filled much later).
+        const bool vec = (E & 3) == 0;
+        const int EU = vec ? E >> 2 : E;  // units of a row: groups of four experts, or experts
         int ES = 1;
-        while (ES < E) ES <<= 1;
-        const int segs = 256 / ES, sg = tid / ES, e = tid % ES;
+        while (ES < EU) ES <<= 1;
+        const int segs = min(256 / ES, 16), sg = tid / ES, eu = tid % ES;  // (at most 16 partial sums per expert to add up)
         const int per = (n_tiles + segs - 1) / segs;
         const int b = min(sg * per, n_tiles), en = min(b + per, n_tiles);
-        int before = 0, all = 0;
-        if (e < E) {
+        int4 before = {0, 0, 0, 0}, all = {0, 0, 0, 0};
+        if (eu < EU && sg < segs) {
             int t = b;
-            for (; t + 4 <= en; t += 4) {  // four independent loads in flight
-                int c[4];
+            if (vec) {
+                const int4 *rows = (const int4 *)tile_counts;
+                for (; t + 8 <= en; t += 8) {  // eight independent loads in flight
+                    int4 c[8];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) c[u] = tile_counts[(size_t)(t + u) * E + e];
+                    for (int u = 0; u < 8; ++u) c[u] = rows[(size_t)(t + u) * EU + eu];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    all += c[u];
-                    before += t + u < tile ? c[u] : 0;
+                    for (int u = 0; u < 8; ++u) {
+                        all.x += c[u].x; all.y += c[u].y; all.z += c[u].z; all.w += c[u].w;
+                        if (t + u < tile) { before.x += c[u].x; before.y += c[u].y; before.z += c[u].z; before.w += c[u].w; }
+                    }
+                }
+                for (; t < en; ++t) {
+                    const int4 c = rows[(size_t)t * EU + eu];
+                    all.x += c.x; all.y += c.y; all.z += c.z; all.w += c.w;
+                    if (t < tile) { before.x += c.x; before.y += c.y; before.z += c.z; before.w += c.w; }
+                }
+            } else {
+                for (; t + 16 <= en; t += 16) {  // sixteen independent loads in flight
+                    int c[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) c[u] = tile_counts[(size_t)(t + u) * E + eu];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        all.x += c[u];
+                        before.x += t + u < tile ? c[u] : 0;
+                    }
+                }
+                for (; t < en; ++t) {
+                    const int c = tile_counts[(size_t)t * E + eu];
+                    all.x += c;
+                    before.x += t < tile ? c : 0;
                 }
             }
-            for (; t < en; ++t) {
-                const int c = tile_counts[(size_t)t * E + e];
-                all += c;
-                before += t < tile ? c : 0;
+        }
+        int *pb = vec ? sort_prow : &part_s[0][0], *pa = vec ? sort_prow + 1024 : &part_s[1][0];  // [segment][expert]
+        if (sg < segs && eu < EU) {
+            if (vec) {
+                *(int4 *)(pb + sg * E + 4 * eu) = before;
+                *(int4 *)(pa + sg * E + 4 * eu) = all;
+            } else {
+                pb[sg * E + eu] = before.x;
+                pa[sg * E + eu] = all.x;
             }
         }
-        part_s[0][tid] = before;
-        part_s[1][tid] = all;
         __syncthreads();
         if (tid < E) {
             int bsum = 0, asum = 0;
             for (int q = 0; q < segs; ++q) {
-                bsum += part_s[0][q * ES + tid];
-                asum += part_s[1][q * ES + tid];
+                bsum += pb[q * E + tid];
+                asum += pa[q * E + tid];
             }
             base_s[tid] = bsum;
             tot_s[tid] = asum;
             if (tile == 0) counts[tid] = asum;
         }
-    } else if (tid < E) {
-        base_s[tid] = tile_base[(size_t)tile * E + tid];
-        tot_s[tid] = counts[tid];
     }
     __syncthreads();
 
@@ -286,16 +577,27 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
         }
     }
 
+    const int G = E + Es;
+    if (sched) {
+        __syncthreads();  // the scans above
+        const int job = blockIdx.x, pass = job >> 3;
+        const table_params tp = pass == 0 ? table_params{nt_up, ncols_up, 1, 0, 1}
+                                          : table_params{nt_down, ncols_down, ks_max_down, kt_down, tail_ks_down};
+        const table_shape ts(tp, mt_s[G]);
+        const analytic_source src = {tp, ts, mt_s, off_s, E, G, T, bm};
+        schedule_queues(src, pass == 0 ? wq_up : wq_down, ts.entries(), n_wg, job & 7, (unsigned char *)&ccount[0][0]);
+        return;
+    }
+
     // Stable rank of every pair among the pairs of its expert.  Within a 64-pair chunk (one wave): the lanes with one
     // expert find each other by ballot, a lane's rank is the number of them below it; across chunks: per-chunk counts
     // in LDS.  Each wave takes every fourth chunk.
-    int my_rank[RANK_CHUNKS / 4], my_e[RANK_CHUNKS / 4];
+    int my_re[RANK_CHUNKS / 4];  // rank within the chunk | expert << 8, or -1
 #pragma unroll
     for (int cq = 0; cq < RANK_CHUNKS / 4; ++cq) {
         const int ch = wave + 4 * cq;
-        my_rank[cq] = 0;
-        my_e[cq] = -1;
-        if (ch >= nchunks) continue;  // uniform over the wave
+        my_re[cq] = -1;
+        if (ch >= nchunks || wave >= 4) continue;  // uniform over the wave
         const int i = ch * 64 + lane;
         const bool valid = i < npairs;
         const int e = valid ? id_s[i] : -1;
@@ -309,36 +611,66 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
         }
         if (valid) {
             const unsigned long long below = mine & ((1ull << lane) - 1ull);
-            my_rank[cq] = __popcll(below);
-            my_e[cq] = e;
+            my_re[cq] = __popcll(below) | (e << 8);
             if (below == 0) ccount[ch][e] = __popcll(mine);  // the lowest lane of each expert of the chunk
         }
     }
     __syncthreads();
+    // (row copies by this workgroup: where the pairs of each expert start in the tile's pair list sorted by destination row)
+    int *run_off = &part_s[0][0];
+    if (xg != nullptr && tid < 64) {
+        int c[4], run = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = tid * 4 + i;
+            c[i] = 0;
+            if (e < E)
+                for (int ch = 0; ch < nchunks; ++ch) c[i] += ccount[ch][e];
+            run += c[i];
+        }
+        int incl = run;
+#pragma unroll
+        for (int m = 1; m < 64; m <<= 1) {
+            const int o = __shfl_up(incl, m, 64);
+            if (tid >= m) incl += o;
+        }
+        int ex = incl - run;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (tid * 4 + i < E) run_off[tid * 4 + i] = ex;
+            ex += c[i];
+        }
+    }
+    if (xg != nullptr) __syncthreads();
 #pragma unroll
     for (int cq = 0; cq < RANK_CHUNKS / 4; ++cq) {
-        const int ch = wave + 4 * cq, e = my_e[cq];
-        if (ch >= nchunks || e < 0) continue;
+        const int ch = wave + 4 * cq, e = my_re[cq] >> 8;
+        if (ch >= nchunks || e < 0 || wave >= 4) continue;
         const int i = ch * 64 + lane;
-        int rank = base_s[e] + my_rank[cq];
-        for (int c2 = 0; c2 < ch; ++c2) rank += ccount[c2][e];
+        int lrank = my_re[cq] & 255;  // rank among the tile's pairs of the expert
+        for (int c2 = 0; c2 < ch; ++c2) lrank += ccount[c2][e];
+        const int rank = base_s[e] + lrank;
         const int r = off_s[e] + rank;
         dst[(size_t)t0 * K + i] = r;
         dstp[(size_t)t0 * K + i] = mt_s[e] * bm + rank;
         src_row[r] = t0 + i / K;
+        if (tokp != nullptr) tokp[mt_s[e] * bm + rank] = t0 + i / K;
+        if (xg != nullptr) {
+            sort_prow[run_off[e] + lrank] = mt_s[e] * bm + rank;
+            sort_tok[run_off[e] + lrank] = (unsigned char)(i / K);
+        }
     }
 
-    const int G = E + Es;
     if (tile == 0) {
-        for (int e = tid; e <= E; e += 256) offsets[e] = off_s[e];
+        for (int e = tid; e <= E; e += nthr) offsets[e] = off_s[e];
         if (tid == 0) tile_meta[0] = mt_s[G];
-        for (int g = tid; g <= G; g += 256) tile_meta[1 + g] = mt_s[g];
+        for (int g = tid; g <= G; g += nthr) tile_meta[1 + g] = mt_s[g];
     }
     // row-tile list: group g is written by workgroup g (mod grid), like the work-item tables below
     for (int g = tile; g < G; g += gridDim.x) {
         const int rows = g < E ? off_s[g + 1] - off_s[g] : T;
         const int nm = mt_s[g + 1] - mt_s[g];
-        for (int mt = tid; mt < nm; mt += 256) {
+        for (int mt = tid; mt < nm; mt += nthr) {
             omega_tile tl;
             tl.g = g;
             tl.row0 = (mt_s[g] + mt) * bm;
@@ -349,181 +681,39 @@ __global__ __launch_bounds__(256) void dispatch_rank_kernel(const int32_t *__res
     }
 
     // ---- work-item tables of the two grouped products (bf16 layers) ----
-    // Tile number first_tile[g]*NT + n*Mg + m = (expert g, column tile n, row tile m): row tiles fastest, so that
-    // tiles that run at the same time share weight tiles.  A group with more than OMEGA_ROW_BLOCK_MAX row tiles is cut
-    // into row blocks of at most that many row tiles, each walking all column tiles (row tiles of the block fastest):
-    // the 32 consecutive entries an XCD works on at a time then form a block of about 8 row tiles x 4 column tiles that
-    // fetches each of its operand tiles once, where one column tile x 32 row tiles would fetch the rows again for every
-    // column tile (down product: 8192 tokens, 64 experts + 2 shared, 0.390 -> 0.368 ms; 16384 tokens, 128 skewed
-    // experts, 0.502 -> 0.486 ms).
-    // The rows of a group are dealt evenly (in blocks of 32) to
-    // its row tiles, instead of full tiles and a ragged last one: the same number of tiles and of MFMA blocks, but
-    // tiles of one cost, so that the workgroups of an XCD, which share operand tiles through its L2, stay in step.
-    // The compute units take 256 tiles at a time; when the
-    // last r = Nt mod 256 tiles would occupy at most half of them, each of those tiles is cut into S = 256/r (2..4)
-    // slices of its 32-row blocks (adjacent entries, so that the slices of a tile run side by side on one XCD and share
-    // the weight tile in its L2).  Group g is written by workgroup g (mod grid).
+    // (item_desc describes their order.)  Every workgroup writes a strided share of the entries; the product kernels
+    // read the per-workgroup queues that the queue builders of this launch form from the same figures, the tables
+    // serve what comes later (adding up the partial results of k slices).
     if (desc_up != nullptr || desc_down != nullptr) {
+        const table_params tpu = {nt_up, ncols_up, 1, 0, 1}, tpd = {nt_down, ncols_down, ks_max_down, kt_down, tail_ks_down};
+        const table_shape tsu(tpu, mt_s[G]), tsd(tpd, mt_s[G]);
         if (tile == 0 && tid == 0) {
-            tile_meta[G + 2] = table_entries(mt_s[G], nt_up);
-            tile_meta[G + 3] = table_entries(mt_s[G], nt_down, ks_max_down, kt_down, tail_ks_down);
-            const int Nt = mt_s[G] * nt_down, KS = table_k_slices(Nt, ks_max_down, kt_down);
-            const int TKS = KS > 1 ? 1 : table_tail_k_slices(Nt, tail_ks_down, kt_down);
-            tile_meta[G + 7] = KS;
+            tile_meta[G + 2] = tsu.entries();
+            tile_meta[G + 3] = tsd.entries();
+            tile_meta[G + 7] = tsd.KS;
             // the k-sliced entries of the down table (their partial results are added up behind the product)
-            tile_meta[G + 8] = KS > 1 ? 0 : Nt - Nt % 256;
-            tile_meta[G + 9] = KS > 1 ? Nt * KS : TKS > 1 ? (Nt % 256) * TKS : 0;
+            tile_meta[G + 8] = tsd.KS > 1 ? 0 : tsd.Nt - tsd.r;
+            tile_meta[G + 9] = tsd.KS > 1 ? tsd.Nt * tsd.KS : tsd.TKS > 1 ? tsd.r * tsd.TKS : 0;
         }
-        for (int g = tile; g < G; g += gridDim.x) {
-            const int rows = g < E ? off_s[g + 1] - off_s[g] : T;
-            const int Mg = mt_s[g + 1] - mt_s[g];
-            write_group_items(desc_up, nt_up, ncols_up, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E);
-            write_group_items(desc_down, nt_down, ncols_down, g, rows, Mg, mt_s[g], mt_s[G], bm, g >= E, ks_max_down, kt_down, tail_ks_down);
-        }
+        if (desc_up != nullptr)
+            for (int ent = tile * nthr + tid; ent < tsu.entries(); ent += n_tiles * nthr)
+                desc_up[ent] = item_desc(ent, tpu, tsu, mt_s, off_s, E, G, T, bm);
+        if (desc_down != nullptr)
+            for (int ent = tile * nthr + tid; ent < tsd.entries(); ent += n_tiles * nthr)
+                desc_down[ent] = item_desc(ent, tpd, tsd, mt_s, off_s, E, G, T, bm);
     }
-}
 
-// Per-workgroup queues of the persistent product kernels.  A product launch has n_wg workgroups, one per compute
-// unit; workgroup w runs on XCD w % 8.  The table is consumed in rounds of n_wg consecutive entries, XCD x taking a
-// contiguous eighth of each round (of what is left, in the last one), so the tiles in flight on one XCD are
-// neighbours in the table and share operand tiles in its L2.  Within a round the entries of an XCD are dealt to its
-// workgroups cheapest entry to the workgroup with the most work so far (ragged row tiles cost less than full ones),
-// which keeps the queues' total work level without any run-time arbitration.
-// One workgroup of 256 threads per (product, XCD); it runs as one of the first workgroups of the gather launch, which
-// needs nothing from it, so its time is hidden.  Three steps per chunk of SCHED_RC rounds: all threads fetch the
-// costs; wave 0 deals the rounds one after the other (lane j < n_wg/8 stands for workgroup j*8 + x); all threads
-// copy the descriptors to their queue slots.
-#define SCHED_RC 256  // rounds per chunk (LDS: 32 bytes of cost + 64 bytes of placement per round)
-#define SCHED_WGS 16  // 2 products x 8 XCDs
-
-__device__ __forceinline__ int work_item_cost(int rows)
-{
-    if (rows <= 0) return 0;
-    const int nb = (rows + 31) >> 5;  // 32-row MFMA blocks of the item (the two waves of a SIMD share them)
-    return 2 + (14 * nb) / 8;         // sixteenths of a full tile; the loads and the fixed part do not shrink
-}
-
-// up to three tables per launch: table p is scheduled by workgroups 8p .. 8p+7
-struct sched_args {
-    const omega_tile_desc *desc[3];
-    omega_tile_desc *wq[3];
-    int total_slot[3];  // index in tile_meta of the table's number of entries
-    int kcost[3];       // 0: an item costs by its rows; 1: by its k steps (weight-gradient items, all 256 rows high)
-    const int32_t *tile_meta;
-    int n_wg;
-};
-
-__device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
-{
-    __shared__ unsigned char cost_s[SCHED_RC * 32];
-    __shared__ unsigned short place_s[SCHED_RC * 32];  // [round][workgroup j] = 0x8000 | (queue slot - len0) << 5 | source lane
-    __shared__ int len0_s[32];
-    const int pass = which >> 3, x = which & 7, tid = threadIdx.x, lane = tid & 63;
-    const omega_tile_desc *desc = pass == 0 ? a.desc[0] : pass == 1 ? a.desc[1] : a.desc[2];
-    omega_tile_desc *wq = pass == 0 ? a.wq[0] : pass == 1 ? a.wq[1] : a.wq[2];
-    const int kcost = pass == 0 ? a.kcost[0] : pass == 1 ? a.kcost[1] : a.kcost[2];
-    const int n_wg = a.n_wg, wpx = n_wg >> 3;
-    const int total = a.tile_meta[pass == 0 ? a.total_slot[0] : pass == 1 ? a.total_slot[1] : a.total_slot[2]];
-    const int rounds = (total + n_wg - 1) / n_wg;
-    // entry of (round r, place i of this XCD), or -1
-    auto entry = [&](int r, int i) {
-        const int base = r * n_wg, left = min(n_wg, total - base);
-        const int per = (left + 7) >> 3;
-        const int L = base + x * per + i;
-        return (i < per && L < base + left) ? L : -1;
-    };
-    int work = 0, len = 0;  // wave 0, lane j: total cost and length of the queue of workgroup j*8 + x
-    for (int r0 = 0; r0 < rounds; r0 += SCHED_RC) {
-        const int nr = min(SCHED_RC, rounds - r0);
-        for (int i0 = 0; i0 < nr * 32; i0 += 4 * 256) {  // four independent loads in flight per thread
-            int rows[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int idx = i0 + u * 256 + tid;
-                const int L = idx < nr * 32 ? entry(r0 + (idx >> 5), idx & 31) : -1;
-                rows[u] = L >= 0 ? (kcost ? -desc[L].xrow0 : desc[L].rows) : 0;
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int idx = i0 + u * 256 + tid;
-                if (idx < nr * 32) cost_s[idx] = (unsigned char)(rows[u] < 0 ? min(255, 2 + (-rows[u]) / 8) : work_item_cost(rows[u]));
-            }
-        }
-        if (tid < 32) len0_s[tid] = len;
-        __syncthreads();
-        if (tid < 64) {
-            int c_next = lane < 32 ? cost_s[lane] : 0;
-            for (int r = 0; r < nr; ++r) {
-                const int c = c_next;
-                c_next = (lane < 32 && r + 1 < nr) ? cost_s[(r + 1) * 32 + lane] : 0;
-                int ce, src;
-                // a round whose entries all cost the same (the common case: tiles of one expert after the even split)
-                // needs no dealing - it adds the same work to every queue: each workgroup takes the entry of its place
-                const unsigned long long act = __ballot(lane < wpx);
-                const int c0 = __builtin_amdgcn_readfirstlane(c);
-                if (__ballot(lane < wpx && c == c0) == act) {
-                    ce = c;
-                    src = lane;
-                } else {
-                    // place of the lane's entry by rising cost and of its workgroup by falling work; lanes that stand
-                    // for no workgroup keep their own place
-                    // keys are unique (ties go to the lower lane), so a place is a count of larger keys; lane o's key is
-                    // broadcast through a scalar register
-                    const int key = lane < wpx ? (work << 6) | (63 - lane) : -1;
-                    int rank_w = 0;
-#pragma unroll
-                    for (int o = 0; o < 32; ++o) rank_w += __builtin_amdgcn_readlane(key, o) > key ? 1 : 0;
-                    const int ckey = lane < wpx ? (c << 6) | lane : 0x7fffffff;
-                    int rank_c = 0;
-#pragma unroll
-                    for (int o = 0; o < 32; ++o) rank_c += __builtin_amdgcn_readlane(ckey, o) < ckey ? 1 : 0;
-                    if (lane >= wpx) { rank_c = lane; rank_w = lane; }
-                    // lane p receives the entry whose cost has place p, then every workgroup fetches the entry of its place
-                    const int sorted = __builtin_amdgcn_ds_permute(rank_c << 2, (c << 8) | lane);
-                    const int mine = __builtin_amdgcn_ds_bpermute(rank_w << 2, sorted);
-                    ce = mine >> 8;
-                    src = mine & 31;
-                }
-                if (lane < 32) {
-                    unsigned short pl = 0;
-                    if (lane < wpx && ce > 0) {
-                        pl = (unsigned short)(0x8000 | ((len - len0_s[lane]) << 5) | src);
-                        work += ce;
-                        ++len;
-                    }
-                    place_s[r * 32 + lane] = pl;
-                }
-            }
-        }
-        __syncthreads();
-        for (int i0 = 0; i0 < nr * 32; i0 += 2 * 256) {  // two independent copies in flight per thread
-            const int idx0 = i0 + tid, idx1 = i0 + 256 + tid;
-            const unsigned short pl0 = idx0 < nr * 32 ? place_s[idx0] : 0, pl1 = idx1 < nr * 32 ? place_s[idx1] : 0;
-            const uint4 *sp0 = (const uint4 *)(desc + (pl0 ? entry(r0 + (idx0 >> 5), pl0 & 31) : 0));
-            const uint4 *sp1 = (const uint4 *)(desc + (pl1 ? entry(r0 + (idx1 >> 5), pl1 & 31) : 0));
-            const uint4 lo0 = sp0[0], hi0 = sp0[1], lo1 = sp1[0], hi1 = sp1[1];
-            if (pl0) {
-                uint4 *dp = (uint4 *)(wq + (size_t)(len0_s[idx0 & 31] + ((pl0 >> 5) & 0x3ff)) * n_wg + (idx0 & 31) * 8 + x);
-                dp[0] = lo0;
-                dp[1] = hi0;
-            }
-            if (pl1) {
-                uint4 *dp = (uint4 *)(wq + (size_t)(len0_s[idx1 & 31] + ((pl1 >> 5) & 0x3ff)) * n_wg + (idx1 & 31) * 8 + x);
-                dp[0] = lo1;
-                dp[1] = hi1;
-            }
-        }
-        __syncthreads();
-    }
-    if (tid < wpx) {
-        omega_tile_desc z = {};
-        wq[(size_t)len * n_wg + tid * 8 + x] = z;
+    // ---- row copies (bf16 layers whose up product reads a gathered copy) ----
+    if (xg != nullptr) {
+        asm volatile("; the prefetched words are dropped here" ::"v"(prefetched));
+        __syncthreads();  // sort_prow / sort_tok
+        if (nt_stores) copy_tile_rows<true>(x, d, t0, min(tok_tile, T - t0), npairs, sort_prow, sort_tok, xg, xs);
+        else copy_tile_rows<false>(x, d, t0, min(tok_tile, T - t0), npairs, sort_prow, sort_tok, xg, xs);
     }
 }
 
 // One wave per token; 16-byte chunks; up to 8 chunks in flight per lane.  PACKED: destination rows are in the
 // packed tile image (chunk index = 4*kstep + c); when xs != nullptr, the token is also copied to row t of xs.
-// The first n_sched workgroups build the product kernels' queues instead (see schedule_queues).
 // NT: the rows are written with non-temporal stores, from half the last-level cache (256 MiB) of gathered rows on.
 // 16384 tokens x 8 slots x 2048 (512 MiB): launch 0.204 -> 0.158 ms and the products that follow gain 2 %;
 // 8192 x 6 x 2048 (192 MiB): launch 0.090 -> 0.073 ms, forward pass 1.332 -> 1.321 ms; 4096 x 2 x 4096 (64 MiB): launch
@@ -531,15 +721,10 @@ __device__ __forceinline__ void schedule_queues(const sched_args &a, int which)
 template <bool PACKED, bool NT>
 __global__ __launch_bounds__(256) void dispatch_gather_kernel(const uint4 *__restrict__ x, const int32_t *__restrict__ dstp,
                                                               int T, int K, int chunks_per_row,
-                                                              unsigned char *__restrict__ xg, unsigned char *__restrict__ xs,
-                                                              int n_sched, sched_args sa)
+                                                              unsigned char *__restrict__ xg, unsigned char *__restrict__ xs)
 {
-    if (PACKED && (int)blockIdx.x < n_sched) {
-        schedule_queues(sa, blockIdx.x);
-        return;
-    }
     const int lane = threadIdx.x & 63;
-    const int t = ((int)blockIdx.x - n_sched) * 4 + (threadIdx.x >> 6);
+    const int t = (int)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= T) return;
     const uint4 *src = x + (size_t)t * chunks_per_row;
     const int KT = chunks_per_row >> 2;
@@ -584,30 +769,21 @@ __global__ __launch_bounds__(256) void dispatch_gather_bytes_kernel(const unsign
     }
 }
 
-// Largest histogram (token tiles x experts) for which every rank workgroup sums all of it itself instead of reading
-// the prefix a scan launch left: 64 KiB per workgroup out of the L2.
-#define RANK_FUSED_MAX_CELLS 16384
-
-hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s)
+// x != nullptr (bf16 layers): the workgroups also copy the rows of their token tiles into xg (and xs)
+hipError_t launch_dispatch_index(const omega_moe *m, int T, int bm, hipStream_t s, const void *x)
 {
     const omega_moe_config &c = m->cfg;
+    const bool rows = x != nullptr && c.dtype == OMEGA_DTYPE_BF16;
+    // from half the last-level cache of gathered rows on, the rows are written around it
+    const int nt_stores = (size_t)T * c.K * c.d * 2 > OMEGA_LLC_BYTES / 2 ? 1 : 0;
     const int tok_tile = router_tok_tile(c.E);
     const int n_tiles = ceil_div(T, tok_tile);
-    const bool fused = (size_t)n_tiles * c.E <= RANK_FUSED_MAX_CELLS;
-    if (!fused) {
-        hipLaunchKernelGGL(dispatch_scan_kernel, dim3(ceil_div(c.E, SCAN_EC)), dim3(256), 0, s, m->tile_counts,
-                           m->tile_base, n_tiles, c.E, m->counts);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-#define RANK_LAUNCH(F)                                                                                                      \
-    hipLaunchKernelGGL(dispatch_rank_kernel<F>, dim3(n_tiles), dim3(256), 0, s, m->ids, m->tile_counts, m->tile_base, m->counts, \
-                       n_tiles, T, tok_tile, c.K, c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tiles,          \
-                       m->tile_meta, m->desc_up, c.H / 128, 128, m->desc_down, c.d / m->down_cols, m->down_cols,             \
-                       m->down_ks_max, c.H / 32, m->down_tail_ks)
-    if (fused) RANK_LAUNCH(true);
-    else RANK_LAUNCH(false);
-#undef RANK_LAUNCH
+    const int n_sched = m->desc_up != nullptr ? SCHED_WGS : 0;  // bf16 layers
+    hipLaunchKernelGGL(dispatch_rank_kernel, dim3(n_tiles + n_sched), dim3(rows ? 1024 : 256), 0, s, m->ids, m->tile_counts, m->counts,
+                       n_tiles, T, tok_tile, c.K, c.E, c.Es, bm, m->offsets, m->dst, m->dstp, m->src_row, m->tokp, m->tiles,
+                       m->tile_meta, m->desc_up, c.H / 128, 128, m->desc_down, c.d / m->down_cols, m->down_cols,
+                       m->down_ks_max, c.H / 32, m->down_tail_ks, m->wq_up, m->wq_down, m->n_wg, (const unsigned char *)x, c.d,
+                       (unsigned char *)(rows ? m->xg : nullptr), (unsigned char *)(rows ? m->xs : nullptr), nt_stores, n_sched);
     return hipGetLastError();
 }
 
@@ -616,19 +792,15 @@ hipError_t launch_dispatch_gather(const omega_moe *m, const void *x, int T, hipS
     const omega_moe_config &c = m->cfg;
     const size_t row_bytes = (size_t)c.d * m->esize;
     if (c.dtype == OMEGA_DTYPE_BF16) {  // d % 256 == 0 is guaranteed at creation: rows are whole 64-byte k steps
-        const int G = c.E + c.Es;
-        sched_args sa = {{m->desc_up, m->desc_down, nullptr}, {m->wq_up, m->wq_down, nullptr}, {G + 2, G + 3, 0}, {0, 0, 0},
-                         m->tile_meta, m->n_wg};
         if ((size_t)T * c.K * row_bytes > OMEGA_LLC_BYTES / 2)
-            hipLaunchKernelGGL((dispatch_gather_kernel<true, true>), dim3(ceil_div(T, 4) + SCHED_WGS), dim3(256), 0, s, (const uint4 *)x,
-                               m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs, SCHED_WGS, sa);
+            hipLaunchKernelGGL((dispatch_gather_kernel<true, true>), dim3(ceil_div(T, 4)), dim3(256), 0, s, (const uint4 *)x,
+                               m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs);
         else
-            hipLaunchKernelGGL((dispatch_gather_kernel<true, false>), dim3(ceil_div(T, 4) + SCHED_WGS), dim3(256), 0, s, (const uint4 *)x,
-                               m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs, SCHED_WGS, sa);
+            hipLaunchKernelGGL((dispatch_gather_kernel<true, false>), dim3(ceil_div(T, 4)), dim3(256), 0, s, (const uint4 *)x,
+                               m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)m->xs);
     } else if (row_bytes % 16 == 0 && ((uintptr_t)x % 16) == 0) {
         hipLaunchKernelGGL((dispatch_gather_kernel<false, false>), dim3(ceil_div(T, 4)), dim3(256), 0, s, (const uint4 *)x,
-                           m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)nullptr, 0,
-                           sched_args{});
+                           m->dstp, T, c.K, (int)(row_bytes / 16), (unsigned char *)m->xg, (unsigned char *)nullptr);
     } else {
         hipLaunchKernelGGL(dispatch_gather_bytes_kernel, dim3(T), dim3(256), 0, s, (const unsigned char *)x, m->dstp, T,
                            c.K, row_bytes, (unsigned char *)m->xg);
@@ -739,7 +911,15 @@ __global__ __launch_bounds__(256) void bw_tables_kernel(int32_t *__restrict__ ti
     }
 }
 
-__global__ __launch_bounds__(256) void bw_sched_kernel(sched_args sa) { schedule_queues(sa, blockIdx.x); }
+__global__ __launch_bounds__(256) void bw_sched_kernel(sched_args sa)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char scratch[SCHED_SCRATCH];
+    const int pass = blockIdx.x >> 3, x = blockIdx.x & 7;
+    const table_source src = {pass == 0 ? sa.desc[0] : pass == 1 ? sa.desc[1] : sa.desc[2],
+                              pass == 0 ? sa.kcost[0] : pass == 1 ? sa.kcost[1] : sa.kcost[2]};
+    const int total = sa.tile_meta[pass == 0 ? sa.total_slot[0] : pass == 1 ? sa.total_slot[1] : sa.total_slot[2]];
+    schedule_queues(src, pass == 0 ? sa.wq[0] : pass == 1 ? sa.wq[1] : sa.wq[2], total, sa.n_wg, x, scratch);
+}
 
 hipError_t launch_backward_tables(const omega_moe *m, int T, hipStream_t s)
 {

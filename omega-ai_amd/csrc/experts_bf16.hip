@@ -103,17 +103,18 @@ __device__ __forceinline__ void dma16_nt(const void *sbase, uint32_t voff, uint3
 }
 
 // The same with only the lanes of `mask` taking part: a wave whose 16-row block of the A tile holds no valid row keeps
-// its place in the load sequence (the waits count instructions) but moves 16 bytes instead of 1 KiB.
-// Only called where every lane of the wave is active (the k steps and the kernel's first loads sit in wave-uniform
-// control flow), so the mask is put back as all ones instead of being saved.
+// its place in the load sequence (the waits count instructions) but moves 16 bytes instead of 1 KiB.  `active` = the
+// lanes that are active at the call (read once per work item, read_active_lanes) and are active again afterwards;
+// `mask` must be a subset of them.
 template <int LDS_OFF>
-__device__ __forceinline__ void dma16_masked(const void *sbase, uint32_t voff, uint32_t lds_base, uint64_t mask)
+__device__ __forceinline__ void dma16_masked(const void *sbase, uint32_t voff, uint32_t lds_base, uint64_t mask, uint64_t active)
 {
-    asm volatile("s_add_u32 m0, %2, %4\n\ts_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %1, %0\n\ts_mov_b64 exec, -1"
+    asm volatile("s_add_u32 m0, %2, %5\n\ts_mov_b64 exec, %3\n\tglobal_load_lds_dwordx4 %1, %0\n\ts_mov_b64 exec, %4"
                  :
-                 : "s"(sbase), "v"(voff), "s"(lds_base), "s"(mask), "n"(LDS_OFF)
+                 : "s"(sbase), "v"(voff), "s"(lds_base), "s"(mask), "s"(active), "n"(LDS_OFF)
                  : "memory", "scc");
 }
+__device__ __forceinline__ uint64_t read_active_lanes() { return __builtin_amdgcn_read_exec(); }
 
 // Everything the loads of one work item need, uniform over the wave: lane l adds 16 l to every address.
 // A0/A1: k step 0 of this wave's two 16-row blocks of the A tile (packed row groups of the tile's first row and of the
@@ -126,6 +127,8 @@ struct TileCtx {
     int half;                 // plain 256-column products: the item covers the first 128 columns only
     int slab;                 // down products: 0 = the item writes the output, > 0 = partial result `slab` of those behind Aux1
     int rec0;                 // products that write or read h1 / h3 block records: record of the item's first 32-row block
+    uint32_t va0, va1;        // per lane: what the lane adds to A0 / A1 (16 * lane, or the place of its source row when the
+                              // rows are gathered by the loads themselves, see GATHER)
 };
 
 __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char *p)
@@ -141,13 +144,38 @@ __device__ __forceinline__ uint64_t uniform_u64(uint64_t v)
     return ((uint64_t)hi << 32) | lo;
 }
 
+// The token a lane's two A loads of an item fetch when the loads gather the rows themselves (GATHER): lane l of the
+// load of 16-row block q brings 16 bytes of tile row 16 q + l / 4.  Rows past the item's last read token 0 (any valid
+// row: they are never used), the rows of a shared expert are the tokens themselves.
+struct GatherTok {
+    int t0, t1;
+};
+__device__ __forceinline__ GatherTok gather_tokens(const omega_tile_desc &d, const int32_t *__restrict__ tokp, int wave, int lane)
+{
+    const int r0 = 16 * wave + (lane >> 2), r1 = r0 + 128;
+    GatherTok g;
+    if (d.xrow0 >= 0) {
+        g.t0 = r0 < d.rows ? d.xrow0 + r0 : 0;
+        g.t1 = r1 < d.rows ? d.xrow0 + r1 : 0;
+    } else {
+        g.t0 = r0 < d.rows ? tokp[d.row0 + r0] : 0;
+        g.t1 = r1 < d.rows ? tokp[d.row0 + r1] : 0;
+    }
+    return g;
+}
+
 // slices: the launch has room for partial results (Aux1), so items that are k slices run as such
-template <int MODE>
+// GATHER (up products of the forward pass): A is the layer input itself, row-major [T, Kd]; every lane of an A load
+// reads its 16 bytes from the row of the token that sits in its tile row (gt), in the chunk order of the packed image,
+// so the tile lands in LDS exactly as a packed xg would have delivered it and no gathered copy is ever written.
+template <int MODE, bool GATHER = false>
 __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa,
-                                            const bf16_t *Wb, int N, int Kd, int wave, int lane, bool slices)
+                                            const bf16_t *Wb, int N, int Kd, int wave, int lane, bool slices,
+                                            GatherTok gt = GatherTok{0, 0})
 {
     constexpr bool FUSED = FUSED_TILE(MODE);
     TileCtx c;
+    c.va0 = c.va1 = (uint32_t)lane * 16u;
     const int KT = Kd / BK;
     const size_t rg_bytes = (size_t)KT * 8192;  // a packed row group (128 rows) occupies KT * 8 KiB
     c.row0 = d.row0;
@@ -199,24 +227,37 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
     // 16-row blocks into it.  A blocks that hold no valid row (ragged tile) are never used by an MFMA whose result
     // is kept: their loads are pointed at the first block, which another wave loads in the same step anyway, so
     // they cost no extra L2 traffic while every wave still issues the same number of loads per step.
+    c.a_mask0 = 16 * wave < c.rows ? ~0ull : 1ull;
+    c.a_mask1 = 16 * (wave + 8) < c.rows ? ~0ull : 1ull;
+    if (GATHER) {
+        // chunk order of the packed image: the 16 bytes at place p of tile row r hold chunk p ^ swz(physical row)
+        const int pr = d.row0 + 16 * wave + (lane >> 2);  // (the row 128 further on has the same swizzle)
+        const uint32_t ch = (uint32_t)(((lane & 3) ^ swz(pr)) << 4);
+        c.A0 = c.A1 = uniform_ptr((const unsigned char *)Axg);
+        c.va0 = (uint32_t)gt.t0 * (uint32_t)(Kd * 2) + ch;
+        c.va1 = (uint32_t)gt.t1 * (uint32_t)(Kd * 2) + ch;
+        return c;
+    }
     const int blk0 = (d.row0 & (BM - 1)) >> 4;
     const int qa0 = blk0 + (16 * wave < d.rows ? wave : 0), qa1 = blk0 + (16 * (wave + 8) < d.rows ? wave + 8 : 0);
     c.A0 = uniform_ptr(A + (size_t)(qa0 >> 3) * rg_bytes + (size_t)(qa0 & 7) * 1024u);
     c.A1 = uniform_ptr(A + (size_t)(qa1 >> 3) * rg_bytes + (size_t)(qa1 & 7) * 1024u);
-    c.a_mask0 = 16 * wave < c.rows ? ~0ull : 1ull;
-    c.a_mask1 = 16 * (wave + 8) < c.rows ? ~0ull : 1ull;
     return c;
 }
 
 // direct load n (0..3) of k step `kstep` of a work item into ring stage `stage`: n -> (operand, row group) =
 // (n & 1 ? B : A, n >> 1)
 // A blocks without valid rows move 16 bytes (a_mask0 / a_mask1).
-template <bool WNT = false>
-__device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, uint32_t lane_off, int stage, int kstep, int n)
+// (A_STEP: bytes from one k step of A to the next: 8 KiB of the packed image, or 64 bytes of a row when the loads gather)
+template <bool WNT = false, int A_STEP = 8192>
+__device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, uint32_t lane_off, int stage, int kstep, int n,
+                                           uint64_t active)
 {
     const uint32_t sb = lds_wave + stage * STAGE_BYTES;
     const size_t kb = (size_t)kstep * 8192u;
-    if ((n & 1) == 0) dma16_masked<0>(((n >> 1) ? c.A1 : c.A0) + kb, lane_off, sb + (n >> 1) * 8192, (n >> 1) ? c.a_mask1 : c.a_mask0);
+    if ((n & 1) == 0)
+        dma16_masked<0>(((n >> 1) ? c.A1 : c.A0) + (size_t)kstep * A_STEP, (n >> 1) ? c.va1 : c.va0, sb + (n >> 1) * 8192,
+                        ((n >> 1) ? c.a_mask1 : c.a_mask0) & active, active);
     else if (WNT) dma16_nt<0>(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
     else dma16<0>(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
 }
@@ -238,12 +279,14 @@ struct LoadCursor {
 // so the matrix cores of the next item start on data that travelled during this item's epilogue; behind the last item
 // of a queue they fetch this item's first steps once more (lane 0 only for A), so that every step of every item
 // issues the same four loads and waits the same way.
-template <int MODE, int NBLK, bool WNT>
+template <int MODE, int NBLK, bool WNT, bool GATHER>
 __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_in, TileCtx &nx, const omega_tile_desc &dn,
                                          const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa, const bf16_t *Wb, int &cur_io,
-                                         void *Cout, void *Aux1, void *Aux2, int N, int Kd, int wave, int lane)
+                                         void *Cout, void *Aux1, void *Aux2, int N, int Kd, int wave, int lane,
+                                         const int32_t *__restrict__ tokp)
 {
     constexpr bool FUSED = FUSED_TILE(MODE), SWAP = SWAPPED(MODE);
+    constexpr int A_STEP = GATHER ? BK * 2 : 8192;  // bytes from one k step of A to the next
     constexpr int NB = NBLK > 0 ? NBLK : 1;
     // the item's uniform fields and the ring position live in scalar registers for the whole item (the direct loads
     // take their base address and LDS address from scalar operands)
@@ -268,12 +311,25 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     const int KT = ITEM_K(MODE) ? __builtin_amdgcn_readfirstlane(ctx_in.kt) : Kd / BK;
     const bool has_next = dn.rows > 0;
     LoadCursor lc;
-    lc.a0 = ctx.A0 + (size_t)NSTAGE * 8192;
+    lc.a0 = ctx.A0 + (size_t)NSTAGE * A_STEP;
     lc.b0 = ctx.B0 + (size_t)NSTAGE * 8192;
-    lc.a1 = ctx.A1 + (size_t)(NSTAGE - 1) * 8192;
+    lc.a1 = ctx.A1 + (size_t)(NSTAGE - 1) * A_STEP;
     lc.b1 = ctx.B1 + (size_t)(NSTAGE - 1) * 8192;
-    lc.m0 = ctx.a_mask0;
-    lc.m1 = ctx.a_mask1;
+    // (the masked A loads switch lanes off and on again: the lanes active here, and the masks as subsets of them)
+    const uint64_t active = uniform_u64(read_active_lanes());
+    lc.m0 = ctx.a_mask0 & active;
+    lc.m1 = ctx.a_mask1 & active;
+    // what a lane adds to the A pointers: 16 * lane, or (GATHER) the place of the token of its tile row in the input
+    uint32_t va0 = GATHER ? ctx_in.va0 : lane_off, va1 = GATHER ? ctx_in.va1 : lane_off;
+    // GATHER: the tokens of the next item's rows are fetched now and used when the loads turn to that item; every k
+    // step in between waits until at most 12 younger loads are in flight, so they have long arrived by then (the
+    // compiler does not see these loads and must not be left to wait for them: its wait would drain the load ring)
+    int nt0 = 0, nt1 = 0;
+    if (GATHER && dn.rows > 0 && dn.xrow0 < 0) {
+        const int r0 = 16 * wave + (lane >> 2), r1 = r0 + 128;
+        const uint32_t o0 = (uint32_t)(dn.row0 + (r0 < dn.rows ? r0 : 0)) * 4u, o1 = (uint32_t)(dn.row0 + (r1 < dn.rows ? r1 : 0)) * 4u;
+        asm volatile("global_load_dword %0, %2, %4\n\tglobal_load_dword %1, %3, %4" : "=&v"(nt0), "=&v"(nt1) : "v"(o0), "v"(o1), "s"(tokp) : "memory");
+    }
 #define LOAD_B(ptr, voff, lds, off) do { if (WNT) dma16_nt<off>(ptr, voff, lds); else dma16<off>(ptr, voff, lds); } while (0)
 
     // ---- MFMA operand addressing ----
@@ -353,18 +409,18 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     // those of the next item's first, which run_tile reads again on entry).
 // BP + IP / BC + IC: LDS address of this wave's first load into the previous / the current stage (scalar register +
 // constant); VOFF: the lane's offset from the load pointers, which then move on by ADV bytes
-#define K_STEP_BODY(cur, BP, IP, BC, IC, VOFF, ADV, Z)                                                                \
+#define K_STEP_BODY(cur, BP, IP, BC, IC, VOFF, ADV, VA0, VA1, ADVA, Z)                                                \
     do {                                                                                                    \
         const int nxt = (cur) + 1 == NSTAGE ? 0 : (cur) + 1;                                                \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         READ_A(af1, cur, 1);                                                                                \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
-            if (i == 0) dma16_masked<(IP) + 8192>(lc.a1, VOFF, BP, lc.m1);                                  \
+            if (i == 0) dma16_masked<(IP) + 8192>(lc.a1, VA1, BP, lc.m1, active);                                   \
             if (i == 2) LOAD_B(lc.b1, VOFF, BP, (IP) + TILE_BYTES + 8192);                                  \
             MFMA4(af0, bq, i, 0, Z);                                                                         \
         }                                                                                                   \
-        lc.a1 += (ADV);                                                                                     \
+        lc.a1 += (ADVA);                                                                                    \
         lc.b1 += (ADV);                                                                                     \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         /* every wave has taken its last fragments of this stage; the next stage must have landed */        \
@@ -374,24 +430,25 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         READ_B(bn, nxt);                                                                                    \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
-            if (i == 0) dma16_masked<(IC)>(lc.a0, VOFF, BC, lc.m0);                                         \
+            if (i == 0) dma16_masked<(IC)>(lc.a0, VA0, BC, lc.m0, active);                                      \
             if (i == 2) LOAD_B(lc.b0, VOFF, BC, (IC) + TILE_BYTES);                                         \
             MFMA4(af1, bq, i, 1, Z);                                                                         \
         }                                                                                                   \
-        lc.a0 += (ADV);                                                                                     \
+        lc.a0 += (ADVA);                                                                                    \
         lc.b0 += (ADV);                                                                                     \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) bq[q] = bn[q];                                        \
     } while (0)
 // the step at a ring position known at compile time
 // (one of five in a row from position 0: the lane offsets carry the k step, the pointers move once per five)
-#define K_STEP_AT(c, Z) \
-    K_STEP_BODY(c, lds_wave, ((c) == 0 ? NSTAGE - 1 : (c)-1) * STAGE_BYTES, lds_wave, (c)*STAGE_BYTES, lane_off + (c)*8192u, 0, Z)
+#define K_STEP_AT(c, Z)                                                                                                 \
+    K_STEP_BODY(c, lds_wave, ((c) == 0 ? NSTAGE - 1 : (c)-1) * STAGE_BYTES, lds_wave, (c)*STAGE_BYTES, lane_off + (c)*8192u, 0, \
+                va0 + (c) * (uint32_t)A_STEP, va1 + (c) * (uint32_t)A_STEP, 0, Z)
 // the step at the ring's position, whatever it is
 #define K_STEP(Z)                                                                                             \
     do {                                                                                                    \
         const uint32_t sb_prv = lds_wave + (cur == 0 ? NSTAGE - 1 : cur - 1) * STAGE_BYTES;                 \
         const uint32_t sb_cur = lds_wave + cur * STAGE_BYTES;                                               \
-        K_STEP_BODY(cur, sb_prv, 0, sb_cur, 0, lane_off, 8192, Z);                                                       \
+        K_STEP_BODY(cur, sb_prv, 0, sb_cur, 0, lane_off, 8192, va0, va1, A_STEP, Z);                                      \
         cur = cur + 1 == NSTAGE ? 0 : cur + 1;                                                              \
     } while (0)
 
@@ -416,24 +473,40 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         K_STEP_AT(2, false);
         K_STEP_AT(3, false);
         K_STEP_AT(4, false);
-        lc.a0 += NSTAGE * 8192;
+        lc.a0 += NSTAGE * A_STEP;
         lc.b0 += NSTAGE * 8192;
-        lc.a1 += NSTAGE * 8192;
+        lc.a1 += NSTAGE * A_STEP;
         lc.b1 += NSTAGE * 8192;
     }
     // the remaining steps; in the last NSTAGE of them the loads belong to the next item, loads 2 and 3 one step later
-    nx = make_ctx<MODE>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr);
+    GatherTok gnext = {0, 0};
+    if (GATHER) {
+        // (four k steps issue more than 12 loads behind the token loads; a shorter run waits for everything once)
+        if (KT - NSTAGE - left < 4) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("; the token loads issued at the item's start have landed" : "+v"(nt0), "+v"(nt1)::"memory");
+        const int r0 = 16 * wave + (lane >> 2), r1 = r0 + 128;
+        if (dn.xrow0 >= 0) {
+            gnext.t0 = r0 < dn.rows ? dn.xrow0 + r0 : 0;
+            gnext.t1 = r1 < dn.rows ? dn.xrow0 + r1 : 0;
+        } else {
+            gnext.t0 = r0 < dn.rows ? nt0 : 0;
+            gnext.t1 = r1 < dn.rows ? nt1 : 0;
+        }
+    }
+    nx = make_ctx<MODE, GATHER>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr, gnext);
 #pragma unroll 1
     for (int s = -left; s < NSTAGE; ++s) {
         if (s == 0) {
             lc.a0 = has_next ? nx.A0 : ctx.A0;
             lc.b0 = has_next ? nx.B0 : ctx.B0;
-            lc.m0 = has_next ? nx.a_mask0 : 1ull;
+            lc.m0 = (has_next ? nx.a_mask0 : 1ull) & active;
+            if (GATHER && has_next) va0 = nx.va0;
         }
         if (s == 1) {
             lc.a1 = has_next ? nx.A1 : ctx.A1;
             lc.b1 = has_next ? nx.B1 : ctx.B1;
-            lc.m1 = has_next ? nx.a_mask1 : 1ull;
+            lc.m1 = (has_next ? nx.a_mask1 : 1ull) & active;
+            if (GATHER && has_next) va1 = nx.va1;
         }
         K_STEP(false);
     }
@@ -561,12 +634,16 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 
 // Persistent: one workgroup per compute unit walks its queue of work items (built by the dispatch stage).
 // WNT: weight tiles are loaded around the last-level cache (see dma16_nt)
-template <int MODE, bool WNT = false>
+// GATHER: the A loads fetch the rows of the layer input themselves (Axg = Ax = the input, row-major; tokp = token of
+// every physical row); see make_ctx
+template <int MODE, bool WNT = false, bool GATHER = false>
 __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
                                                                    const bf16_t *__restrict__ Wa, const bf16_t *__restrict__ Wb,
                                                                    void *__restrict__ Cout, void *Aux1, void *Aux2,
-                                                                   const omega_tile_desc *__restrict__ wq, int N, int Kd)
+                                                                   const omega_tile_desc *__restrict__ wq, int N, int Kd,
+                                                                   const int32_t *__restrict__ tokp = nullptr)
 {
+    constexpr int A_STEP = GATHER ? BK * 2 : 8192;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -574,18 +651,20 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
 
     omega_tile_desc d = wq[wg];
     if (d.rows <= 0) return;
-    TileCtx cur_ctx = make_ctx<MODE>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr);
+    TileCtx cur_ctx = make_ctx<MODE, GATHER>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr,
+                                             GATHER ? gather_tokens(d, tokp, wave, lane) : GatherTok{0, 0});
     {
         // first item: k steps 0..NSTAGE-2 and the first half of step NSTAGE-1 into stages 0..NSTAGE-1
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
         const uint32_t lds_wave = lds0 + wave * 1024;
         const uint32_t lane_off = (uint32_t)lane * 16u;
+        const uint64_t active = read_active_lanes();
         for (int st = 0; st < NSTAGE - 1; ++st) {
 #pragma unroll
-            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<WNT>(cur_ctx, lds_wave, lane_off, st, st, n);
+            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<WNT, A_STEP>(cur_ctx, lds_wave, lane_off, st, st, n, active);
         }
-        issue_load<WNT>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 0);
-        issue_load<WNT>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 1);
+        issue_load<WNT, A_STEP>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 0, active);
+        issue_load<WNT, A_STEP>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 1, active);
         asm volatile("s_waitcnt vmcnt(14)" ::: "memory");  // all but steps 1.. : LOADS_PER_STEP * (NSTAGE - 2) + 2
         __syncthreads();
     }
@@ -596,7 +675,7 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
         // 32-row blocks alternate between the two row halves of the workgroup: block b belongs to waves with wm = b % 2
         const int nblk = max(0, min(4, (((cur_ctx.rows + 31) >> 5) + 1 - (wave >> 2)) >> 1));
 #define RUN_TILE(NBLK) \
-    run_tile<MODE, NBLK, WNT>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, Aux1, Aux2, N, Kd, wave, lane)
+    run_tile<MODE, NBLK, WNT, GATHER>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, Aux1, Aux2, N, Kd, wave, lane, tokp)
         switch (nblk) {
             case 4: RUN_TILE(4); break;
             case 3: RUN_TILE(3); break;
@@ -668,7 +747,8 @@ hipError_t experts_bf16_init(void)
     const void *fns[] = {(const void *)experts_bf16_kernel<MODE_UP>, (const void *)experts_bf16_kernel<MODE_DOWN>,
                          (const void *)experts_bf16_kernel<MODE_UPRAW>, (const void *)experts_bf16_kernel<MODE_DA>,
                          (const void *)experts_bf16_kernel<MODE_WGRAD>, (const void *)experts_bf16_kernel<MODE_UPREC>,
-                         (const void *)experts_bf16_kernel<MODE_UP, true>, (const void *)experts_bf16_kernel<MODE_DOWN, true>};
+                         (const void *)experts_bf16_kernel<MODE_UP, true>, (const void *)experts_bf16_kernel<MODE_DOWN, true>,
+                         (const void *)experts_bf16_kernel<MODE_UP, false, true>, (const void *)experts_bf16_kernel<MODE_UP, true, true>};
     for (const void *f : fns) {
         hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
         if (e != hipSuccess) return e;
@@ -679,7 +759,6 @@ hipError_t experts_bf16_init(void)
 hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int which, hipStream_t s)
 {
     const omega_moe_config &c = m->cfg;
-    (void)x;
     // the ring must be shorter than an item: K >= (NSTAGE + 1) * BK (guaranteed at creation: d, H >= 256)
     if ((which == 0 ? c.d : c.H) < (NSTAGE + 1) * BK) return hipErrorInvalidValue;
     // A batch with at most 64 rows per routed expert on average streams every weight tile once (one row tile per
@@ -692,6 +771,16 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
         hipLaunchKernelGGL(experts_bf16_kernel<MODE_UPREC>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s,
                            (const bf16_t *)m->xg, (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a,
                            (void *)m->bw_h1, (void *)m->bw_h3, m->wq_up, c.H, c.d);
+    } else if (which == 0 && m->gather_on_load) {
+        // the loads of the product fetch the rows of x themselves: no gathered copy (and no packed copy for the shared experts)
+        if (wnt)
+            hipLaunchKernelGGL((experts_bf16_kernel<MODE_UP, true, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)x,
+                               (const bf16_t *)x, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
+                               (void *)nullptr, m->wq_up, c.H, c.d, m->tokp);
+        else
+            hipLaunchKernelGGL((experts_bf16_kernel<MODE_UP, false, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)x,
+                               (const bf16_t *)x, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
+                               (void *)nullptr, m->wq_up, c.H, c.d, m->tokp);
     } else if (which == 0) {
         if (wnt)
             hipLaunchKernelGGL((experts_bf16_kernel<MODE_UP, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,

@@ -263,6 +263,9 @@ public:
     Tensor *getDiff() { return diff_.get(); }
     // forward keeps h1 / h3 for back(), as the reference's layers keep their outputs
     void setTraining(bool on) { check(ctx_.get(), omega_moe_set_training(moe_, on ? 1 : 0)); }
+    /// OMEGA_GATHER_AUTO / _COPY / _ON_LOAD: how the rows of x reach the experts of a bf16 layer
+    void setGatherMode(int mode) { check(ctx_.get(), omega_moe_set_gather_mode(moe_, mode)); }
+    bool gatherOnLoad() const { return omega_moe_gather_on_load(moe_) != 0; }
     // update() of a layer without an updater: w -= learnRate * diffW (FullyLayer.update, FullyLayer.java:569-590)
     float learnRate = 0.0f;
     bool freeze = false;  // Layer.freeze: a frozen layer's update() does nothing (FullyLayer.java:571)

@@ -51,6 +51,8 @@ public final class OmegaHip {
     private static final MethodHandle BACKWARD = h("omega_moe_backward", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, ADDRESS));
     private static final MethodHandle BACKWARD_BLOCK = h("omega_moe_backward_block", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, ADDRESS));
     private static final MethodHandle SET_TRAINING = h("omega_moe_set_training", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT));
+    private static final MethodHandle SET_GATHER_MODE = h("omega_moe_set_gather_mode", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT));
+    private static final MethodHandle GATHER_ON_LOAD = h("omega_moe_gather_on_load", FunctionDescriptor.of(JAVA_INT, ADDRESS));
     private static final MethodHandle GET_GRAD = h("omega_moe_get_grad", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, JAVA_INT));
     private static final MethodHandle ACC_GRAD = h("omega_moe_acc_grad", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_FLOAT));
     private static final MethodHandle UPDATE = h("omega_moe_update", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_FLOAT));
@@ -261,6 +263,24 @@ public final class OmegaHip {
     public static void setTraining(MemorySegment ctx, MemorySegment moe, boolean on) {
         try {
             check(ctx, (int) SET_TRAINING.invokeExact(moe, on ? 1 : 0));
+        } catch (Throwable t) {
+            throw wrap(t);
+        }
+    }
+
+    /** Whether the last dispatch left the rows of x to the up product's loads (omega_moe_gather_on_load). */
+    public static boolean gatherOnLoad(MemorySegment moe) {
+        try {
+            return (int) GATHER_ON_LOAD.invokeExact(moe) != 0;
+        } catch (Throwable t) {
+            throw wrap(t);
+        }
+    }
+
+    /** 0 by shape, 1 gathered copy, 2 rows fetched by the up product's loads (omega_moe_set_gather_mode). */
+    public static void setGatherMode(MemorySegment ctx, MemorySegment moe, int mode) {
+        try {
+            check(ctx, (int) SET_GATHER_MODE.invokeExact(moe, mode));
         } catch (Throwable t) {
             throw wrap(t);
         }

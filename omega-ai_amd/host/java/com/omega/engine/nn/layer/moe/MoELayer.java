@@ -332,6 +332,11 @@ public class MoELayer extends Layer {
         OmegaHip.setTraining(ctx, moe, on);
     }
 
+    /** How the rows of x reach the experts of a bf16 layer: 0 by shape, 1 gathered copy, 2 fetched by the up product's loads. */
+    public void setGatherMode(int mode) {
+        OmegaHip.setGatherMode(ctx, moe, mode);
+    }
+
     /** One parameter gradient (fp32, layout of its weight): W_GATE, W_GATE_BIAS, W_NORM, W_W1 / W_W3 / W_W2 of expert g. */
     public float[] grad(int which, int g) {
         int n = which == OmegaHip.W_GATE ? nExperts * embedDim

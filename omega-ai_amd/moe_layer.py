@@ -236,6 +236,15 @@ class MoELayer:
         """Forward keeps h1 / h3 for back(), as the reference's layers keep their outputs."""
         self.ctx.check(self.lib.omega_moe_set_training(self.handle, int(bool(on))))
 
+    def set_gather_mode(self, mode):
+        """How the rows of x reach the experts of a bf16 layer: 0 by shape, 1 gathered copy, 2 fetched by the up
+        product's loads (omega_moe_set_gather_mode)."""
+        self.ctx.check(self.lib.omega_moe_set_gather_mode(self.handle, int(mode)))
+
+    def gather_on_load(self):
+        """True if the last dispatch left the rows of x to the up product's loads (no gathered copy)."""
+        return bool(self.lib.omega_moe_gather_on_load(self.handle))
+
     def initBack(self):
         """(Re)allocates the input gradient when the batch size changes (FullyLayer.initBack,
         J/engine/nn/layer/FullyLayer.java:130-144); the parameter gradients live in the native handle."""

@@ -189,6 +189,22 @@ def test_stage_calls_out_of_order_are_refused():
     # a forward leaves the stages usable for its T only
     assert lib.omega_moe_combine(h, cfg.T, out.ptr) == L.OK
     refused(lib.omega_moe_combine(h, cfg.T - 1, out.ptr))
+    # overwriting a workspace buffer takes the stages that read it out until the stage that writes it has run again,
+    # and a backward pass needs a new forward
+    dout = P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], "bf16")
+    dx = P.DeviceBuffer(G.ctx(), (cfg.T, cfg.d), "bf16")
+    layer.fill_workspace("y", 0xFF)
+    refused(lib.omega_moe_combine(h, cfg.T, out.ptr))
+    assert lib.omega_moe_backward(h, x.ptr, dout.ptr, cfg.T, dx.ptr) == L.ERR_INVALID_ARG
+    assert lib.omega_moe_experts_down(h, cfg.T) == L.OK
+    assert lib.omega_moe_combine(h, cfg.T, out.ptr) == L.OK
+    assert np.array_equal(out.to_numpy(), staged)
+    layer.fill_workspace("a", 0xFF)
+    refused(lib.omega_moe_experts_down(h, cfg.T))
+    refused(lib.omega_moe_combine(h, cfg.T, out.ptr))
+    assert lib.omega_moe_experts(h, x.ptr, cfg.T) == L.OK
+    assert lib.omega_moe_combine(h, cfg.T, out.ptr) == L.OK
+    assert np.array_equal(out.to_numpy(), staged)
     layer.close()
 
 

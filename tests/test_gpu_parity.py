@@ -135,6 +135,48 @@ def test_bf16_scaled_configs(G, name, kw):
     layer.close()
 
 
+@pytest.mark.parametrize("name,kw", [
+    ("c2_mixtral", dict(T=1000, d=256, H=384)),        # ragged row tiles, rows that share a line with another tile's
+    ("c2_mixtral", dict(T=37, d=512, H=512)),          # a small batch (k slices of the down product)
+    ("c4_finegrained", dict(T=515, d=256, H=384)),     # shared experts (their rows are the tokens themselves), odd T
+    ("c5_skewed", dict(T=1024, d=256, H=256)),         # empty experts, K = 8
+])
+def test_bf16_gather_modes_agree(G, name, kw):
+    """The rows of x reach the experts either as a gathered copy written by the dispatch stage or through the loads of
+    the up product (omega_moe_set_gather_mode): the same bits either way, against the oracle, and the gathered rows
+    asked for afterwards are x[src_row] in both.  A second forward with fewer tokens in each mode (the row -> token
+    table then holds stale entries behind the valid rows)."""
+    cfg = scaled(C.CONFIGS[name], **kw)
+    inp = make_inputs(cfg, 31337)
+    ref = G.oracle_forward(cfg, inp)
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    T2 = max(1, cfg.T // 3)
+    cfg2 = scaled(cfg, T=T2)
+    inp2 = {**inp, "x": inp["x"][:T2]}
+    ref2 = G.oracle_forward(cfg2, inp2)
+    x2 = G.P.DeviceBuffer.from_numpy(G.ctx(), inp2["x"], cfg.dtype)
+    outs = {}
+    for mode in (1, 2):
+        layer = G.build_layer(cfg, inp)
+        layer.set_gather_mode(mode)
+        out = layer.forward(x).to_numpy()
+        G.assert_routing_bit_exact(layer.routing(), ref)
+        assert N.rel_l2(out, ref["out"]) <= BF16_TOL
+        assert np.array_equal(layer.workspace("xg", cfg.T), inp["x"][ref["src_row"]])
+        out2 = layer.forward(x2).to_numpy()
+        G.assert_routing_bit_exact(layer.routing(), ref2)
+        assert N.rel_l2(out2, ref2["out"]) <= BF16_TOL
+        assert np.array_equal(layer.workspace("xg", T2), inp2["x"][ref2["src_row"]])
+        assert np.array_equal(layer.forward(x).to_numpy(), out)
+        outs[mode] = (out, out2)
+        layer.close()
+    assert np.array_equal(outs[1][0], outs[2][0]) and np.array_equal(outs[1][1], outs[2][1])
+    layer = G.build_layer(cfg, inp)
+    with pytest.raises(RuntimeError):
+        layer.set_gather_mode(3)
+    layer.close()
+
+
 @pytest.mark.parametrize("T,d,H,E,K,Es", [
     (1, 512, 1024, 8, 2, 0),      # two experts with one row each: 32 k steps in 4 slices (no slice under 8 steps)
     (3, 256, 2048, 8, 2, 0),      # 8 slices of 8 steps

@@ -13,6 +13,15 @@ pytestmark = pytest.mark.gpu
 L = importlib.import_module("omega-ai_amd._lib")
 
 
+def free_device_bytes():
+    """hipMemGetInfo through the runtime the library itself is linked against."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
 @pytest.mark.parametrize("dtype,E,K,d", [("bf16", 8, 2, 512), ("f32", 12, 3, 96), ("bf16", 128, 8, 256)])
 def test_noalloc_router_probs_matches_the_allocating_entry_point(dtype, E, K, d):
     from tests import gpu_util as G
@@ -24,7 +33,10 @@ def test_noalloc_router_probs_matches_the_allocating_entry_point(dtype, E, K, d)
     for T in (cfg.T, 257):                                   # two calls in a row, the second with a smaller input
         lg0, p0 = layer.router_probs(x, T)                   # the existing entry point (stages in hipMalloc'ed memory)
         r0 = layer.routing(T)
+        G.ctx().sync()
+        free0 = free_device_bytes()
         lg1, p1 = layer.router_probs_noalloc(x, T)
+        assert free_device_bytes() == free0, "the entry point allocated (or freed) device memory"
         r1 = layer.routing(T)
         assert np.array_equal(lg0.view(np.uint32), lg1.view(np.uint32)), T
         assert np.array_equal(p0.view(np.uint32), p1.view(np.uint32)), T
