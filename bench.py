@@ -45,71 +45,6 @@ def profiled_traffic(cfg_name):
 
 
 
-def kstep_probe():
-    """The k-step loop of the product kernels in isolation (bench_probe.so), TFLOP/s per variant: 8 waves of 128 x 64
-    (the kernels' shape) and 4 waves of 128 x 128; without loads, then with the 32 KiB of direct loads per step whose
-    streams are shared by 32 / 8 / 4 / 2 workgroups of an XCD (1 MiB streams: the misses come out of the last-level
-    cache; 8 MiB streams: from memory, for the sharings whose streams together exceed 256 MiB)."""
-    import ctypes
-    lib = ctypes.CDLL(os.path.join(ROOT, "bench_probe.so"))   # built by __graft_entry__.build()
-    lib.bench_probe_kstep.argtypes = [ctypes.c_int] * 6 + [ctypes.POINTER(ctypes.c_float)]
-    lib.bench_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
-    v = ctypes.c_float()
-    rows = []
-
-    def run(fn, *args):
-        st = fn(*args, ctypes.byref(v))
-        if st != 0:
-            raise RuntimeError(f"bench_probe: HIP error {st}")
-        return round(v.value, 1)
-
-    rows.append({"what": "MFMAs only, 8 waves, random operands", "TFLOP/s": run(lib.bench_probe_mfma, 0, 1, 200)})
-    for waves in (8, 4):
-        rows.append({"what": f"{waves} waves: fragments + barrier", "TFLOP/s": run(lib.bench_probe_kstep, 0, waves, 0, 32, 32, 40)})
-        for share, kib in ((32, 1024), (8, 1024), (4, 1024), (2, 1024), (8, 8192), (4, 8192)):
-            rows.append({"what": f"{waves} waves: + direct loads, {share} workgroups per stream of {kib} KiB "
-                                 f"({256 // share * kib // 1024} MiB in all)",
-                         "TFLOP/s": run(lib.bench_probe_kstep, 0, waves, 1, share, kib, 40)})
-    print(json.dumps({"kstep_probe": rows, "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS}))
-
-
-def vendor_gemm():
-    """hipBLASLt (through torch.matmul) on y = x W^T with bf16 operands of the workload's distributions: the up product
-    (W1 | W3: 2 H outputs) and the down product of the Mixtral shape, once as ONE matrix product over all 8192 expert
-    rows (every weight tile reused by 32 row tiles) and once as 8 products of 1024 rows with 8 different weight
-    matrices (what the layer has to compute: every weight byte is used by 4 row tiles)."""
-    import torch
-    torch.manual_seed(0)
-    dev = "cuda"
-    rows = []
-
-    def one(what, M, N, K, groups, reps=20):
-        xs = [torch.randn(M, K, device=dev, dtype=torch.bfloat16) for _ in range(groups)]
-        ws = [(torch.randn(N, K, device=dev) / K ** 0.5).to(torch.bfloat16) for _ in range(groups)]
-        outs = [torch.empty(M, N, device=dev, dtype=torch.bfloat16) for _ in range(groups)]
-        for _ in range(5):
-            for g in range(groups):
-                torch.matmul(xs[g], ws[g].t(), out=outs[g])
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            for g in range(groups):
-                torch.matmul(xs[g], ws[g].t(), out=outs[g])
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / reps
-        tf = 2.0 * M * N * K * groups / ms / 1e9
-        rows.append({"what": what, "M": M, "N": N, "K": K, "products": groups, "ms": round(ms, 4), "TFLOP/s": round(tf, 1),
-                     "frac": round(tf / PEAK_BF16_TFLOPS, 3)})
-
-    one("up, one product over all rows", 8192, 28672, 4096, 1)
-    one("up, one product per expert", 1024, 28672, 4096, 8)
-    one("down, one product over all rows", 8192, 4096, 14336, 1)
-    one("down, one product per expert", 1024, 4096, 14336, 8)
-    print(json.dumps({"vendor_gemm": rows, "peak": PEAK_BF16_TFLOPS}))
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -129,26 +64,11 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 256 MiB device copy (convert_kernel fp32->fp32) three times, so that "
                          "FETCH_SIZE / WRITE_SIZE of a profiled run can be scaled by a kernel of known traffic")
-    ap.add_argument("--kstep-probe", action="store_true",
-                    help="instead of the benchmark: the rates the inner loop of the product kernels sustains by itself "
-                         "(bench_probe.so: MFMAs + fragment reads + barrier, then with the direct loads at several L2 "
-                         "miss rates), one JSON line")
-    ap.add_argument("--vendor-gemm", action="store_true",
-                    help="instead of the benchmark: the vendor's bf16 GEMM (torch.matmul -> hipBLASLt) at the shapes of "
-                         "the Mixtral-shape products, as one product over all rows and as one product per expert; a "
-                         "yardstick measured on the same device, nothing of the layer runs; one JSON line")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus above 1 is not supported (no collectives in this path)",
               file=sys.stderr)
         sys.exit(2)
-
-    if a.kstep_probe:
-        kstep_probe()
-        return
-    if a.vendor_gemm:
-        vendor_gemm()
-        return
 
     P = importlib.import_module("omega-ai_amd")
     L = importlib.import_module("omega-ai_amd._lib")

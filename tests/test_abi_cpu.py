@@ -71,18 +71,13 @@ def test_missing_library_fails_loudly(tmp_path, monkeypatch):
 
 
 def test_bench_probe_library_exports_and_refuses_bad_arguments():
-    """bench_probe.so (bench.py's measurement aids, not part of the layer library): both entry points are exported and
-    the k-step probe turns down arguments that would take its loads outside its buffer, before any device call."""
+    """bench_probe.so (bench.py's matrix-core ceiling probe, not part of the layer library): the entry point is exported
+    and turns down a launch count it cannot time, before any device call."""
     path = os.path.join(ROOT, "bench_probe.so")
     if not os.path.exists(path):
         pytest.skip("bench_probe.so not built (python -c 'import __graft_entry__ as g; g.build()')")
     p = C.CDLL(path)
-    p.bench_probe_kstep.argtypes = [C.c_int] * 6 + [C.POINTER(C.c_float)]
     p.bench_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]
     v = C.c_float()
     assert p.bench_probe_mfma(0, 1, 2, C.byref(v)) != 0                       # too few launches
-    for waves, loads, share, kib, launches in ((3, 1, 4, 1024, 40), (8, 1, 3, 1024, 40), (8, 1, 64, 1024, 40),
-                                               (8, 1, 4, 1000, 40), (8, 1, 4, 16, 40), (8, 1, 1, 16384, 40),
-                                               (8, 1, 4, 1024, 2)):
-        assert p.bench_probe_kstep(0, waves, loads, share, kib, launches, C.byref(v)) != 0, (waves, share, kib, launches)
-    assert p.bench_probe_kstep(0, 8, 1, 4, 1024, 40, None) != 0
+    assert p.bench_probe_mfma(0, 1, 200, None) != 0
