@@ -127,8 +127,6 @@ struct TileCtx {
     int half;                 // plain 256-column products: the item covers the first 128 columns only
     int slab;                 // down products: 0 = the item writes the output, > 0 = partial result `slab` of those behind Aux1
     int rec0;                 // products that write or read h1 / h3 block records: record of the item's first 32-row block
-    uint32_t va0, va1;        // per lane: what the lane adds to A0 / A1 (16 * lane, or the place of its source row when the
-                              // rows are gathered by the loads themselves, see GATHER)
 };
 
 __device__ __forceinline__ const unsigned char *uniform_ptr(const unsigned char *p)
@@ -144,38 +142,13 @@ __device__ __forceinline__ uint64_t uniform_u64(uint64_t v)
     return ((uint64_t)hi << 32) | lo;
 }
 
-// The token a lane's two A loads of an item fetch when the loads gather the rows themselves (GATHER): lane l of the
-// load of 16-row block q brings 16 bytes of tile row 16 q + l / 4.  Rows past the item's last read token 0 (any valid
-// row: they are never used), the rows of a shared expert are the tokens themselves.
-struct GatherTok {
-    int t0, t1;
-};
-__device__ __forceinline__ GatherTok gather_tokens(const omega_tile_desc &d, const int32_t *__restrict__ tokp, int wave, int lane)
-{
-    const int r0 = 16 * wave + (lane >> 2), r1 = r0 + 128;
-    GatherTok g;
-    if (d.xrow0 >= 0) {
-        g.t0 = r0 < d.rows ? d.xrow0 + r0 : 0;
-        g.t1 = r1 < d.rows ? d.xrow0 + r1 : 0;
-    } else {
-        g.t0 = r0 < d.rows ? tokp[d.row0 + r0] : 0;
-        g.t1 = r1 < d.rows ? tokp[d.row0 + r1] : 0;
-    }
-    return g;
-}
-
 // slices: the launch has room for partial results (Aux1), so items that are k slices run as such
-// GATHER (up products of the forward pass): A is the layer input itself, row-major [T, Kd]; every lane of an A load
-// reads its 16 bytes from the row of the token that sits in its tile row (gt), in the chunk order of the packed image,
-// so the tile lands in LDS exactly as a packed xg would have delivered it and no gathered copy is ever written.
-template <int MODE, bool GATHER = false>
+template <int MODE>
 __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa,
-                                            const bf16_t *Wb, int N, int Kd, int wave, int lane, bool slices,
-                                            GatherTok gt = GatherTok{0, 0})
+                                            const bf16_t *Wb, int N, int Kd, int wave, int lane, bool slices)
 {
     constexpr bool FUSED = FUSED_TILE(MODE);
     TileCtx c;
-    c.va0 = c.va1 = (uint32_t)lane * 16u;
     const int KT = Kd / BK;
     const size_t rg_bytes = (size_t)KT * 8192;  // a packed row group (128 rows) occupies KT * 8 KiB
     c.row0 = d.row0;
@@ -229,15 +202,6 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
     // they cost no extra L2 traffic while every wave still issues the same number of loads per step.
     c.a_mask0 = 16 * wave < c.rows ? ~0ull : 1ull;
     c.a_mask1 = 16 * (wave + 8) < c.rows ? ~0ull : 1ull;
-    if (GATHER) {
-        // chunk order of the packed image: the 16 bytes at place p of tile row r hold chunk p ^ swz(physical row)
-        const int pr = d.row0 + 16 * wave + (lane >> 2);  // (the row 128 further on has the same swizzle)
-        const uint32_t ch = (uint32_t)(((lane & 3) ^ swz(pr)) << 4);
-        c.A0 = c.A1 = uniform_ptr((const unsigned char *)Axg);
-        c.va0 = (uint32_t)gt.t0 * (uint32_t)(Kd * 2) + ch;
-        c.va1 = (uint32_t)gt.t1 * (uint32_t)(Kd * 2) + ch;
-        return c;
-    }
     const int blk0 = (d.row0 & (BM - 1)) >> 4;
     const int qa0 = blk0 + (16 * wave < d.rows ? wave : 0), qa1 = blk0 + (16 * (wave + 8) < d.rows ? wave + 8 : 0);
     c.A0 = uniform_ptr(A + (size_t)(qa0 >> 3) * rg_bytes + (size_t)(qa0 & 7) * 1024u);
@@ -248,16 +212,14 @@ __device__ __forceinline__ TileCtx make_ctx(const omega_tile_desc &d, const bf16
 // direct load n (0..3) of k step `kstep` of a work item into ring stage `stage`: n -> (operand, row group) =
 // (n & 1 ? B : A, n >> 1)
 // A blocks without valid rows move 16 bytes (a_mask0 / a_mask1).
-// (A_STEP: bytes from one k step of A to the next: 8 KiB of the packed image, or 64 bytes of a row when the loads gather)
-template <bool WNT = false, int A_STEP = 8192>
+template <bool WNT = false>
 __device__ __forceinline__ void issue_load(const TileCtx &c, uint32_t lds_wave, uint32_t lane_off, int stage, int kstep, int n,
                                            uint64_t active)
 {
     const uint32_t sb = lds_wave + stage * STAGE_BYTES;
     const size_t kb = (size_t)kstep * 8192u;
     if ((n & 1) == 0)
-        dma16_masked<0>(((n >> 1) ? c.A1 : c.A0) + (size_t)kstep * A_STEP, (n >> 1) ? c.va1 : c.va0, sb + (n >> 1) * 8192,
-                        ((n >> 1) ? c.a_mask1 : c.a_mask0) & active, active);
+        dma16_masked<0>(((n >> 1) ? c.A1 : c.A0) + kb, lane_off, sb + (n >> 1) * 8192, ((n >> 1) ? c.a_mask1 : c.a_mask0) & active, active);
     else if (WNT) dma16_nt<0>(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
     else dma16<0>(((n >> 1) == 0 ? c.B0 : c.B1) + kb, lane_off, sb + TILE_BYTES + (n >> 1) * 8192);
 }
@@ -279,14 +241,12 @@ struct LoadCursor {
 // so the matrix cores of the next item start on data that travelled during this item's epilogue; behind the last item
 // of a queue they fetch this item's first steps once more (lane 0 only for A), so that every step of every item
 // issues the same four loads and waits the same way.
-template <int MODE, int NBLK, bool WNT, bool GATHER>
+template <int MODE, int NBLK, bool WNT>
 __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_in, TileCtx &nx, const omega_tile_desc &dn,
                                          const bf16_t *Axg, const bf16_t *Ax, const bf16_t *Wa, const bf16_t *Wb, int &cur_io,
-                                         void *Cout, void *Aux1, void *Aux2, int N, int Kd, int wave, int lane,
-                                         const int32_t *__restrict__ tokp)
+                                         void *Cout, void *Aux1, void *Aux2, int N, int Kd, int wave, int lane)
 {
     constexpr bool FUSED = FUSED_TILE(MODE), SWAP = SWAPPED(MODE);
-    constexpr int A_STEP = GATHER ? BK * 2 : 8192;  // bytes from one k step of A to the next
     constexpr int NB = NBLK > 0 ? NBLK : 1;
     // the item's uniform fields and the ring position live in scalar registers for the whole item (the direct loads
     // take their base address and LDS address from scalar operands)
@@ -311,25 +271,14 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     const int KT = ITEM_K(MODE) ? __builtin_amdgcn_readfirstlane(ctx_in.kt) : Kd / BK;
     const bool has_next = dn.rows > 0;
     LoadCursor lc;
-    lc.a0 = ctx.A0 + (size_t)NSTAGE * A_STEP;
+    lc.a0 = ctx.A0 + (size_t)NSTAGE * 8192;
     lc.b0 = ctx.B0 + (size_t)NSTAGE * 8192;
-    lc.a1 = ctx.A1 + (size_t)(NSTAGE - 1) * A_STEP;
+    lc.a1 = ctx.A1 + (size_t)(NSTAGE - 1) * 8192;
     lc.b1 = ctx.B1 + (size_t)(NSTAGE - 1) * 8192;
     // (the masked A loads switch lanes off and on again: the lanes active here, and the masks as subsets of them)
     const uint64_t active = uniform_u64(read_active_lanes());
     lc.m0 = ctx.a_mask0 & active;
     lc.m1 = ctx.a_mask1 & active;
-    // what a lane adds to the A pointers: 16 * lane, or (GATHER) the place of the token of its tile row in the input
-    uint32_t va0 = GATHER ? ctx_in.va0 : lane_off, va1 = GATHER ? ctx_in.va1 : lane_off;
-    // GATHER: the tokens of the next item's rows are fetched now and used when the loads turn to that item; every k
-    // step in between waits until at most 12 younger loads are in flight, so they have long arrived by then (the
-    // compiler does not see these loads and must not be left to wait for them: its wait would drain the load ring)
-    int nt0 = 0, nt1 = 0;
-    if (GATHER && dn.rows > 0 && dn.xrow0 < 0) {
-        const int r0 = 16 * wave + (lane >> 2), r1 = r0 + 128;
-        const uint32_t o0 = (uint32_t)(dn.row0 + (r0 < dn.rows ? r0 : 0)) * 4u, o1 = (uint32_t)(dn.row0 + (r1 < dn.rows ? r1 : 0)) * 4u;
-        asm volatile("global_load_dword %0, %2, %4\n\tglobal_load_dword %1, %3, %4" : "=&v"(nt0), "=&v"(nt1) : "v"(o0), "v"(o1), "s"(tokp) : "memory");
-    }
 #define LOAD_B(ptr, voff, lds, off) do { if (WNT) dma16_nt<off>(ptr, voff, lds); else dma16<off>(ptr, voff, lds); } while (0)
 
     // ---- MFMA operand addressing ----
@@ -409,18 +358,18 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
     // those of the next item's first, which run_tile reads again on entry).
 // BP + IP / BC + IC: LDS address of this wave's first load into the previous / the current stage (scalar register +
 // constant); VOFF: the lane's offset from the load pointers, which then move on by ADV bytes
-#define K_STEP_BODY(cur, BP, IP, BC, IC, VOFF, ADV, VA0, VA1, ADVA, Z)                                                \
+#define K_STEP_BODY(cur, BP, IP, BC, IC, VOFF, ADV, Z)                                                                \
     do {                                                                                                    \
         const int nxt = (cur) + 1 == NSTAGE ? 0 : (cur) + 1;                                                \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         READ_A(af1, cur, 1);                                                                                \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
-            if (i == 0) dma16_masked<(IP) + 8192>(lc.a1, VA1, BP, lc.m1, active);                                   \
+            if (i == 0) dma16_masked<(IP) + 8192>(lc.a1, VOFF, BP, lc.m1, active);                                  \
             if (i == 2) LOAD_B(lc.b1, VOFF, BP, (IP) + TILE_BYTES + 8192);                                  \
             MFMA4(af0, bq, i, 0, Z);                                                                         \
         }                                                                                                   \
-        lc.a1 += (ADVA);                                                                                    \
+        lc.a1 += (ADV);                                                                                     \
         lc.b1 += (ADV);                                                                                     \
         __builtin_amdgcn_sched_barrier(0);                                                                  \
         /* every wave has taken its last fragments of this stage; the next stage must have landed */        \
@@ -430,25 +379,24 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         READ_B(bn, nxt);                                                                                    \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                       \
         {                                                                                                   \
-            if (i == 0) dma16_masked<(IC)>(lc.a0, VA0, BC, lc.m0, active);                                      \
+            if (i == 0) dma16_masked<(IC)>(lc.a0, VOFF, BC, lc.m0, active);                                     \
             if (i == 2) LOAD_B(lc.b0, VOFF, BC, (IC) + TILE_BYTES);                                         \
             MFMA4(af1, bq, i, 1, Z);                                                                         \
         }                                                                                                   \
-        lc.a0 += (ADVA);                                                                                    \
+        lc.a0 += (ADV);                                                                                     \
         lc.b0 += (ADV);                                                                                     \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) bq[q] = bn[q];                                        \
     } while (0)
 // the step at a ring position known at compile time
 // (one of five in a row from position 0: the lane offsets carry the k step, the pointers move once per five)
-#define K_STEP_AT(c, Z)                                                                                                 \
-    K_STEP_BODY(c, lds_wave, ((c) == 0 ? NSTAGE - 1 : (c)-1) * STAGE_BYTES, lds_wave, (c)*STAGE_BYTES, lane_off + (c)*8192u, 0, \
-                va0 + (c) * (uint32_t)A_STEP, va1 + (c) * (uint32_t)A_STEP, 0, Z)
+#define K_STEP_AT(c, Z) \
+    K_STEP_BODY(c, lds_wave, ((c) == 0 ? NSTAGE - 1 : (c)-1) * STAGE_BYTES, lds_wave, (c)*STAGE_BYTES, lane_off + (c)*8192u, 0, Z)
 // the step at the ring's position, whatever it is
 #define K_STEP(Z)                                                                                             \
     do {                                                                                                    \
         const uint32_t sb_prv = lds_wave + (cur == 0 ? NSTAGE - 1 : cur - 1) * STAGE_BYTES;                 \
         const uint32_t sb_cur = lds_wave + cur * STAGE_BYTES;                                               \
-        K_STEP_BODY(cur, sb_prv, 0, sb_cur, 0, lane_off, 8192, va0, va1, A_STEP, Z);                                      \
+        K_STEP_BODY(cur, sb_prv, 0, sb_cur, 0, lane_off, 8192, Z);                                                       \
         cur = cur + 1 == NSTAGE ? 0 : cur + 1;                                                              \
     } while (0)
 
@@ -473,40 +421,24 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
         K_STEP_AT(2, false);
         K_STEP_AT(3, false);
         K_STEP_AT(4, false);
-        lc.a0 += NSTAGE * A_STEP;
+        lc.a0 += NSTAGE * 8192;
         lc.b0 += NSTAGE * 8192;
-        lc.a1 += NSTAGE * A_STEP;
+        lc.a1 += NSTAGE * 8192;
         lc.b1 += NSTAGE * 8192;
     }
     // the remaining steps; in the last NSTAGE of them the loads belong to the next item, loads 2 and 3 one step later
-    GatherTok gnext = {0, 0};
-    if (GATHER) {
-        // (four k steps issue more than 12 loads behind the token loads; a shorter run waits for everything once)
-        if (KT - NSTAGE - left < 4) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        asm volatile("; the token loads issued at the item's start have landed" : "+v"(nt0), "+v"(nt1)::"memory");
-        const int r0 = 16 * wave + (lane >> 2), r1 = r0 + 128;
-        if (dn.xrow0 >= 0) {
-            gnext.t0 = r0 < dn.rows ? dn.xrow0 + r0 : 0;
-            gnext.t1 = r1 < dn.rows ? dn.xrow0 + r1 : 0;
-        } else {
-            gnext.t0 = r0 < dn.rows ? nt0 : 0;
-            gnext.t1 = r1 < dn.rows ? nt1 : 0;
-        }
-    }
-    nx = make_ctx<MODE, GATHER>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr, gnext);
+    nx = make_ctx<MODE>(dn, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr);
 #pragma unroll 1
     for (int s = -left; s < NSTAGE; ++s) {
         if (s == 0) {
             lc.a0 = has_next ? nx.A0 : ctx.A0;
             lc.b0 = has_next ? nx.B0 : ctx.B0;
             lc.m0 = (has_next ? nx.a_mask0 : 1ull) & active;
-            if (GATHER && has_next) va0 = nx.va0;
         }
         if (s == 1) {
             lc.a1 = has_next ? nx.A1 : ctx.A1;
             lc.b1 = has_next ? nx.B1 : ctx.B1;
             lc.m1 = (has_next ? nx.a_mask1 : 1ull) & active;
-            if (GATHER && has_next) va1 = nx.va1;
         }
         K_STEP(false);
     }
@@ -634,16 +566,12 @@ __device__ __forceinline__ void run_tile(unsigned char *smem, const TileCtx ctx_
 
 // Persistent: one workgroup per compute unit walks its queue of work items (built by the dispatch stage).
 // WNT: weight tiles are loaded around the last-level cache (see dma16_nt)
-// GATHER: the A loads fetch the rows of the layer input themselves (Axg = Ax = the input, row-major; tokp = token of
-// every physical row); see make_ctx
-template <int MODE, bool WNT = false, bool GATHER = false>
+template <int MODE, bool WNT = false>
 __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
                                                                    const bf16_t *__restrict__ Wa, const bf16_t *__restrict__ Wb,
                                                                    void *__restrict__ Cout, void *Aux1, void *Aux2,
-                                                                   const omega_tile_desc *__restrict__ wq, int N, int Kd,
-                                                                   const int32_t *__restrict__ tokp = nullptr)
+                                                                   const omega_tile_desc *__restrict__ wq, int N, int Kd)
 {
-    constexpr int A_STEP = GATHER ? BK * 2 : 8192;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -651,8 +579,7 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
 
     omega_tile_desc d = wq[wg];
     if (d.rows <= 0) return;
-    TileCtx cur_ctx = make_ctx<MODE, GATHER>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr,
-                                             GATHER ? gather_tokens(d, tokp, wave, lane) : GatherTok{0, 0});
+    TileCtx cur_ctx = make_ctx<MODE>(d, Axg, Ax, Wa, Wb, N, Kd, wave, lane, PLAIN_DOWN(MODE) && Aux1 != nullptr);
     {
         // first item: k steps 0..NSTAGE-2 and the first half of step NSTAGE-1 into stages 0..NSTAGE-1
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -661,10 +588,10 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
         const uint64_t active = read_active_lanes();
         for (int st = 0; st < NSTAGE - 1; ++st) {
 #pragma unroll
-            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<WNT, A_STEP>(cur_ctx, lds_wave, lane_off, st, st, n, active);
+            for (int n = 0; n < LOADS_PER_STEP; ++n) issue_load<WNT>(cur_ctx, lds_wave, lane_off, st, st, n, active);
         }
-        issue_load<WNT, A_STEP>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 0, active);
-        issue_load<WNT, A_STEP>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 1, active);
+        issue_load<WNT>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 0, active);
+        issue_load<WNT>(cur_ctx, lds_wave, lane_off, NSTAGE - 1, NSTAGE - 1, 1, active);
         asm volatile("s_waitcnt vmcnt(14)" ::: "memory");  // all but steps 1.. : LOADS_PER_STEP * (NSTAGE - 2) + 2
         __syncthreads();
     }
@@ -675,7 +602,7 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
         // 32-row blocks alternate between the two row halves of the workgroup: block b belongs to waves with wm = b % 2
         const int nblk = max(0, min(4, (((cur_ctx.rows + 31) >> 5) + 1 - (wave >> 2)) >> 1));
 #define RUN_TILE(NBLK) \
-    run_tile<MODE, NBLK, WNT, GATHER>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, Aux1, Aux2, N, Kd, wave, lane, tokp)
+    run_tile<MODE, NBLK, WNT>(smem, cur_ctx, nx, dn, Axg, Ax, Wa, Wb, stage, Cout, Aux1, Aux2, N, Kd, wave, lane)
         switch (nblk) {
             case 4: RUN_TILE(4); break;
             case 3: RUN_TILE(3); break;
@@ -686,6 +613,344 @@ __global__ __launch_bounds__(NWAVES * 64) void experts_bf16_kernel(const bf16_t 
 #undef RUN_TILE
         if (dn.rows <= 0) break;
         cur_ctx = nx;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the loads behind the last item land in LDS that nobody reads)
+}
+
+// =====================================================================================================================
+// Up product with one wave per SIMD (forward pass outside training): four waves of 128 rows x 128 MFMA columns, the 256
+// accumulators of a wave in the AGPRs.  Same 256 x 256 tile, LDS ring, packed operands, work items and queues as the
+// kernel above; what changes is the fragment traffic - a wave reads 8 A and 8 B fragments per 64 MFMAs (16 KiB) where
+// two waves of 128 x 64 read 24 KiB - and that one barrier per k step joins four waves instead of eight.
+// 16-row units of the tile alternate between the two row halves of the workgroup (unit u belongs to the waves with
+// wm = u % 2), so a ragged tile leaves both halves the same work; units without valid rows issue no MFMAs.
+// Every k step is the same code: the MFMAs run on one set of fragments while the other set is read for the next step
+// and the wave's 8 direct loads of the step five ahead go out; when the loads reach the end of an item they turn to
+// the next one of the queue.  Items start on rows that are multiples of 32 (item_desc), so a wave's fragment addresses
+// never change and the fragments read during an item's last step are the next item's first.
+// =====================================================================================================================
+#define U4_WAVES 4
+#define U4_LOADS 8  // direct loads per wave and k step
+
+struct Up4Item {                // uniform over the wave unless said otherwise
+    const unsigned char *A;    // k step 0 of the tile's rows (packed image), or x (GATHER)
+    const unsigned char *B0, *B1;  // k step 0 of the 128 rows of W1 / of W3
+    uint32_t va[4];             // per lane: what the lane adds to A for the wave's A loads (16-row blocks wave + 4 n)
+    int row0, rows, n0;
+};
+
+// GATHER: token of tile row 16 * (wave + 4 n) + lane / 4, or 0 behind the item's rows
+struct Up4Tok {
+    int t[4];
+};
+
+template <bool GATHER>
+__device__ __forceinline__ Up4Item up4_item(const omega_tile_desc &d, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *W1,
+                                            const bf16_t *W3, int N, int Kd, int wave, int lane, const Up4Tok &tk)
+{
+    Up4Item c;
+    const int KT = Kd / BK;
+    const size_t rg_bytes = (size_t)KT * 8192;
+    c.row0 = d.row0;
+    c.rows = d.rows;
+    c.n0 = d.n0;
+    const size_t wrg = (size_t)d.g * (N >> 7) + (d.n0 >> 7);
+    c.B0 = uniform_ptr((const unsigned char *)W1 + wrg * rg_bytes);
+    c.B1 = uniform_ptr((const unsigned char *)W3 + wrg * rg_bytes);
+    if (GATHER) {
+        c.A = uniform_ptr((const unsigned char *)Axg);
+        const int pr = d.row0 + 16 * wave + (lane >> 2);  // (rows 64 n further on have the same swizzle)
+        const uint32_t ch = (uint32_t)(((lane & 3) ^ swz(pr)) << 4);
+#pragma unroll
+        for (int n = 0; n < 4; ++n) c.va[n] = (uint32_t)tk.t[n] * (uint32_t)(Kd * 2) + ch;
+        return c;
+    }
+    c.A = uniform_ptr((Ax != nullptr && d.xrow0 >= 0) ? (const unsigned char *)Ax + (size_t)(d.xrow0 / BM * 2) * rg_bytes
+                                                      : (const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes);
+    const int blk0 = (d.row0 & (BM - 1)) >> 4;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+        // a block without valid rows is never used by an MFMA whose result is kept: all its lanes read the same 16 bytes of
+        // the item's first block (one request instead of sixteen lines), and every step still issues the same loads
+        const int q = wave + 4 * n;
+        const bool valid = 16 * q < d.rows;
+        const int qa = blk0 + (valid ? q : 0);
+        c.va[n] = (uint32_t)(qa >> 3) * (uint32_t)rg_bytes + (uint32_t)(qa & 7) * 1024u + (valid ? (uint32_t)lane * 16u : 0u);
+    }
+    return c;
+}
+
+__device__ __forceinline__ Up4Tok up4_tokens(const omega_tile_desc &d, const int32_t *__restrict__ tokp, int wave, int lane)
+{
+    Up4Tok k;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+        const int r = 16 * (wave + 4 * n) + (lane >> 2);
+        k.t[n] = r < d.rows ? (d.xrow0 >= 0 ? d.xrow0 + r : tokp[d.row0 + r]) : 0;
+    }
+    return k;
+}
+
+// What the waves of the kernel carry from one item to the next: the ring position, the fragments read during the
+// step before, and where the loads have got to.
+struct Up4State {
+    int cur;
+    bf16x8_t fa0[8], fb0[8], fa1[8], fb1[8];
+    const unsigned char *lA, *lB0, *lB1;
+    uint32_t va[4];
+};
+
+// One work item for a wave with NU units of valid rows (units beyond them issue no MFMAs; the accumulators live for
+// one item, so every NU is its own straight-line code with NU * 32 accumulator registers).
+template <int NU, bool WNT, bool GATHER>
+__device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, const Up4Item &it, Up4Item &nxt_it,
+                                             const omega_tile_desc &dn, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *W1,
+                                             const bf16_t *W3, void *Cout, int N, int Kd, int wave, int lane,
+                                             const int32_t *__restrict__ tokp)
+{
+    constexpr int A_STEP = GATHER ? BK * 2 : 8192;
+    constexpr int NA = NU > 0 ? NU : 1;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int KT = Kd / BK;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    const uint32_t lds_wave = lds0 + wave * 1024;
+    const uint32_t vb0 = (uint32_t)wave * 1024u + (uint32_t)lane * 16u, vb1 = vb0 + 4096u;
+    const bool has_next = dn.rows > 0;
+    // fragment addresses within a stage.  A fragment iu: rows of unit 2 iu + wm = block 2 iu + wm of the A tile; B fragment
+    // c (16 MFMA columns): block (c / 4) * 8 + wn * 4 + c % 4 of the B tile, i.e. columns wn * 64 + 16 (c % 4) of the W1 half
+    // (c < 4) or of the W3 half, so that acc[.][c] and acc[.][c + 4] are h1 and h3 of the same elements.  Lane l supplies
+    // row l % 16, chunk l / 16; the chunk swizzle depends on the row through l % 16 and the block's parity.
+    const uint32_t pa = (uint32_t)(wm * 16 + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | (wm << 4))) << 4);
+    uint32_t pb[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+        pb[h] = TILE_BYTES + (uint32_t)(wn * 64 + 16 * h + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | (h << 4))) << 4);
+    int cur = __builtin_amdgcn_readfirstlane(st.cur);
+    const unsigned char *lA = uniform_ptr(st.lA), *lB0 = uniform_ptr(st.lB0), *lB1 = uniform_ptr(st.lB1);
+
+    // GATHER: the tokens of the next item's rows are asked for now and used when the loads turn to that item, several
+    // steps later: every step waits until at most 24 younger loads are in flight, so they have landed by then (the
+    // compiler does not see these loads and must not be left to wait for them: its wait would drain the load ring)
+    Up4Tok ntk = {{0, 0, 0, 0}};
+    if (GATHER && has_next && dn.xrow0 < 0) {
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+            const int r = 16 * (wave + 4 * n) + (lane >> 2);
+            const uint32_t o = (uint32_t)(dn.row0 + (r < dn.rows ? r : 0)) * 4u;
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(ntk.t[n]) : "v"(o), "s"(tokp) : "memory");
+        }
+    }
+    if (!GATHER && has_next) nxt_it = up4_item<false>(dn, Axg, Ax, W1, W3, N, Kd, wave, lane, Up4Tok{});
+
+#define U4_READ(FA, FB, stage, r)                                                                                       \
+    do {                                                                                                                \
+        const unsigned char *sp = smem + (stage) * STAGE_BYTES;                                                         \
+        if ((r) < 8) FB[(r) & 7] = *(const bf16x8_t *)(sp + pb[(r) & 1] + (((r) & 3) >> 1) * 2048u + (((r) & 7) >> 2) * 8192u); \
+        else FA[((r) - 8) & 7] = *(const bf16x8_t *)(sp + pa + (((r) - 8) & 7) * 2048u);                                \
+    } while (0)
+// the wave's direct load l (0..7) of a k step into the stage at LDS address sb: A blocks wave + 4 n, then the B blocks
+#define U4_LOAD(l, sb)                                                                                                  \
+    do {                                                                                                                \
+        if ((l) < 4) dma16<((l) & 3) * 4096>(lA, st.va[(l) & 3], sb);                                                   \
+        else if (WNT) dma16_nt<TILE_BYTES + (((l) - 4) >> 1) * 8192 + ((l) & 1) * 4096>((l) < 6 ? lB0 : lB1, (l) & 1 ? vb1 : vb0, sb); \
+        else dma16<TILE_BYTES + (((l) - 4) >> 1) * 8192 + ((l) & 1) * 4096>((l) < 6 ? lB0 : lB1, (l) & 1 ? vb1 : vb0, sb); \
+    } while (0)
+// One k step on the fragments PA / PB (taken from stage `cur` during the step before): group g of 4 MFMAs = unit g / 2,
+// B fragments 4 (g % 2) ..; with the first 8 groups two fragment reads of the next step (stage cur + 1, into QA / QB), with
+// every other group one direct load of the step five ahead into stage `cur`, which every wave has left.  At the barrier
+// that ends the step the loads of the step after next must have landed: three younger steps (24 loads) may be in flight.
+// Z: the accumulators start from zero operands (an item's first step).
+// (the group index is spelled out: the LDS offsets of the loads are immediate operands)
+#define U4_MFMA(PA, PB, Z, iu, c)                                                                                       \
+    do {                                                                                                                \
+        if ((iu) < NU)                                                                                                  \
+            acc[(iu) % NA][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PB[c], PA[iu], (Z) ? zero4 : acc[(iu) % NA][c], 0, 0, 0); \
+    } while (0)
+// A wave issues one instruction every four cycles and an MFMA of this shape occupies the matrix core for sixteen: up
+// to three other instructions fit behind each MFMA without delaying the next one.  The order is pinned so: an MFMA,
+// then the two fragment reads or the direct load (three instructions with its m0 set-up) that go with it.
+#define U4_GROUP(PA, PB, QA, QB, Z, g)                                                                                  \
+    do {                                                                                                                \
+        U4_MFMA(PA, PB, Z, (g) >> 1, 4 * ((g) & 1));                                                                    \
+        if ((g) < 8) {                                                                                                  \
+            U4_READ(QA, QB, nxt, 2 * (g));                                                                              \
+            U4_READ(QA, QB, nxt, 2 * (g) + 1);                                                                          \
+        }                                                                                                               \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+        U4_MFMA(PA, PB, Z, (g) >> 1, 4 * ((g) & 1) + 1);                                                                \
+        if ((g) & 1) U4_LOAD((g) >> 1, sb);                                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+        U4_MFMA(PA, PB, Z, (g) >> 1, 4 * ((g) & 1) + 2);                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+        U4_MFMA(PA, PB, Z, (g) >> 1, 4 * ((g) & 1) + 3);                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+    } while (0)
+#define U4_STEP(PA, PB, QA, QB, Z)                                                                                      \
+    do {                                                                                                                \
+        const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;                                                                \
+        const uint32_t sb = lds_wave + cur * STAGE_BYTES;                                                               \
+        U4_GROUP(PA, PB, QA, QB, Z, 0); U4_GROUP(PA, PB, QA, QB, Z, 1); U4_GROUP(PA, PB, QA, QB, Z, 2);                 \
+        U4_GROUP(PA, PB, QA, QB, Z, 3); U4_GROUP(PA, PB, QA, QB, Z, 4); U4_GROUP(PA, PB, QA, QB, Z, 5);                 \
+        U4_GROUP(PA, PB, QA, QB, Z, 6); U4_GROUP(PA, PB, QA, QB, Z, 7); U4_GROUP(PA, PB, QA, QB, Z, 8);                 \
+        U4_GROUP(PA, PB, QA, QB, Z, 9); U4_GROUP(PA, PB, QA, QB, Z, 10); U4_GROUP(PA, PB, QA, QB, Z, 11);               \
+        U4_GROUP(PA, PB, QA, QB, Z, 12); U4_GROUP(PA, PB, QA, QB, Z, 13); U4_GROUP(PA, PB, QA, QB, Z, 14);              \
+        U4_GROUP(PA, PB, QA, QB, Z, 15);                                                                                \
+        lA += A_STEP;                                                                                                   \
+        lB0 += 8192;                                                                                                    \
+        lB1 += 8192;                                                                                                    \
+        asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");                                                    \
+        __syncthreads();                                                                                                \
+        cur = nxt;                                                                                                      \
+    } while (0)
+
+    f32x4_t acc[NA][8];  // acc[iu][c]: 16 x 16 piece (rows of unit 2 iu + wm, columns of B fragment c), weights as first operand
+    const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    // KT steps (even, at least 8), two at a time.  The loads issued during steps 0 .. KT - 6 are the item's own (its steps
+    // 5 .. KT - 1), those of the last five steps the next item's first five (behind the last item of a queue this item's
+    // once more: nobody reads them).
+    U4_STEP(st.fa0, st.fb0, st.fa1, st.fb1, true);
+    U4_STEP(st.fa1, st.fb1, st.fa0, st.fb0, false);
+    for (int k = 2; k < KT - 6; k += 2) {
+        U4_STEP(st.fa0, st.fb0, st.fa1, st.fb1, false);
+        U4_STEP(st.fa1, st.fb1, st.fa0, st.fb0, false);
+    }
+    U4_STEP(st.fa0, st.fb0, st.fa1, st.fb1, false);
+    if (GATHER && has_next) {
+        // three steps or more have passed since the token loads were issued: they have landed
+        asm volatile("; token loads done" : "+v"(ntk.t[0]), "+v"(ntk.t[1]), "+v"(ntk.t[2]), "+v"(ntk.t[3])::"memory");
+        if (dn.xrow0 >= 0) ntk = up4_tokens(dn, tokp, wave, lane);
+        nxt_it = up4_item<true>(dn, Axg, Ax, W1, W3, N, Kd, wave, lane, ntk);
+    }
+    lA = uniform_ptr(nxt_it.A);
+    lB0 = uniform_ptr(nxt_it.B0);
+    lB1 = uniform_ptr(nxt_it.B1);
+#pragma unroll
+    for (int n = 0; n < 4; ++n) st.va[n] = nxt_it.va[n];
+    U4_STEP(st.fa1, st.fb1, st.fa0, st.fb0, false);
+    for (int k = 0; k < 2; ++k) {
+        U4_STEP(st.fa0, st.fb0, st.fa1, st.fb1, false);
+        U4_STEP(st.fa1, st.fb1, st.fa0, st.fb0, false);
+    }
+#undef U4_STEP
+#undef U4_GROUP
+#undef U4_LOAD
+#undef U4_READ
+    st.cur = cur;
+    st.lA = lA;
+    st.lB0 = lB0;
+    st.lB1 = lB1;
+
+    // ---- epilogue: a = silu(h1) * h3 as packed bf16 ----
+    // lane: row l16 of unit 2 iu + wm; registers r of acc[iu][c] and acc[iu][c + 4]: h1 and h3 of column
+    // wn * 64 + 16 c + 4 lq + r of the tile's 128, i.e. k step n0 / 32 + 2 wn + c / 2 of the packed a, chunk 2 (c % 2) + lq / 2
+    const int KTa = N / BK;
+#pragma unroll
+    for (int iu = 0; iu < NU; ++iu) {
+        const int row = 16 * (2 * iu + wm) + l16;
+        if (row < it.rows) {
+            const int prow = it.row0 + row;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float h1 = acc[iu][c][r], h3 = acc[iu][c + 4][r];
+                    v[r] = h1 * __builtin_amdgcn_rcpf(1.0f + __expf(-h1)) * h3;  // v_exp_f32, v_rcp_f32: 1 ulp each
+                }
+                const uint2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+                *(uint2 *)((unsigned char *)Cout + pk_chunk_off(prow, (it.n0 >> 5) + 2 * wn + (c >> 1), 2 * (c & 1) + (lq >> 1), KTa) +
+                           (lq & 1) * 8) = o;
+            }
+        }
+    }
+}
+
+template <bool WNT, bool GATHER>
+__global__ __launch_bounds__(U4_WAVES * 64) void experts_up4_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
+                                                                    const bf16_t *__restrict__ W1, const bf16_t *__restrict__ W3,
+                                                                    void *__restrict__ Cout, const omega_tile_desc *__restrict__ wq,
+                                                                    int N, int Kd, const int32_t *__restrict__ tokp)
+{
+    constexpr int A_STEP = GATHER ? BK * 2 : 8192;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int n_wg = gridDim.x, wg = blockIdx.x;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    const uint32_t lds_wave = lds0 + wave * 1024;
+    const uint32_t vb0 = (uint32_t)wave * 1024u + (uint32_t)lane * 16u, vb1 = vb0 + 4096u;
+
+    omega_tile_desc d = wq[wg];
+    if (d.rows <= 0) return;
+    Up4Item it = up4_item<GATHER>(d, Axg, Ax, W1, W3, N, Kd, wave, lane, GATHER ? up4_tokens(d, tokp, wave, lane) : Up4Tok{});
+    Up4State st;
+    st.lA = it.A;
+    st.lB0 = it.B0;
+    st.lB1 = it.B1;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) st.va[n] = it.va[n];
+    // first item: k steps 0..4 into stages 0..4
+    for (int s5 = 0; s5 < NSTAGE; ++s5) {
+        const uint32_t sb = lds_wave + s5 * STAGE_BYTES;
+        dma16<0>(st.lA, st.va[0], sb);
+        dma16<4096>(st.lA, st.va[1], sb);
+        dma16<8192>(st.lA, st.va[2], sb);
+        dma16<12288>(st.lA, st.va[3], sb);
+        if (WNT) {
+            dma16_nt<TILE_BYTES>(st.lB0, vb0, sb);
+            dma16_nt<TILE_BYTES + 4096>(st.lB0, vb1, sb);
+            dma16_nt<TILE_BYTES + 8192>(st.lB1, vb0, sb);
+            dma16_nt<TILE_BYTES + 12288>(st.lB1, vb1, sb);
+        } else {
+            dma16<TILE_BYTES>(st.lB0, vb0, sb);
+            dma16<TILE_BYTES + 4096>(st.lB0, vb1, sb);
+            dma16<TILE_BYTES + 8192>(st.lB1, vb0, sb);
+            dma16<TILE_BYTES + 12288>(st.lB1, vb1, sb);
+        }
+        st.lA += A_STEP;
+        st.lB0 += 8192;
+        st.lB1 += 8192;
+    }
+    asm volatile("s_waitcnt vmcnt(32)" ::: "memory");  // step 0 has landed: U4_LOADS * (NSTAGE - 1) younger loads
+    __syncthreads();
+    {
+        const uint32_t pa = (uint32_t)(wm * 16 + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | (wm << 4))) << 4);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const uint32_t pbr = TILE_BYTES + (uint32_t)(wn * 64 + 16 * (r & 1) + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | ((r & 1) << 4))) << 4);
+            st.fb0[r] = *(const bf16x8_t *)(smem + pbr + ((r & 3) >> 1) * 2048u + (r >> 2) * 8192u);
+            st.fa0[r] = *(const bf16x8_t *)(smem + pa + r * 2048u);
+        }
+    }
+    // every wave has taken step 0 out of stage 0 before anyone refills it
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    st.cur = 0;
+
+    for (int q = 1;; ++q) {
+        const omega_tile_desc dn = wq[(size_t)q * n_wg + wg];
+        // units of this wave that hold valid rows: unit u = 2 iu + wm is valid if 16 u < rows
+        const int units = (it.rows + 15) >> 4;
+        const int nu = __builtin_amdgcn_readfirstlane(max(0, min(8, (units + 1 - wm) >> 1)));
+        Up4Item nxt_it = it;
+#define U4_RUN(NU) up4_run_item<NU, WNT, GATHER>(smem, st, it, nxt_it, dn, Axg, Ax, W1, W3, Cout, N, Kd, wave, lane, tokp)
+        switch (nu) {
+            case 8: U4_RUN(8); break;
+            case 7: U4_RUN(7); break;
+            case 6: U4_RUN(6); break;
+            case 5: U4_RUN(5); break;
+            case 4: U4_RUN(4); break;
+            case 3: U4_RUN(3); break;
+            case 2: U4_RUN(2); break;
+            case 1: U4_RUN(1); break;
+            default: U4_RUN(0); break;
+        }
+#undef U4_RUN
+        if (dn.rows <= 0) break;
+        it = nxt_it;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the loads behind the last item land in LDS that nobody reads)
 }
@@ -748,7 +1013,8 @@ hipError_t experts_bf16_init(void)
                          (const void *)experts_bf16_kernel<MODE_UPRAW>, (const void *)experts_bf16_kernel<MODE_DA>,
                          (const void *)experts_bf16_kernel<MODE_WGRAD>, (const void *)experts_bf16_kernel<MODE_UPREC>,
                          (const void *)experts_bf16_kernel<MODE_UP, true>, (const void *)experts_bf16_kernel<MODE_DOWN, true>,
-                         (const void *)experts_bf16_kernel<MODE_UP, false, true>, (const void *)experts_bf16_kernel<MODE_UP, true, true>};
+                         (const void *)experts_up4_kernel<false, false>, (const void *)experts_up4_kernel<true, false>,
+                         (const void *)experts_up4_kernel<false, true>, (const void *)experts_up4_kernel<true, true>};
     for (const void *f : fns) {
         hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
         if (e != hipSuccess) return e;
@@ -771,25 +1037,20 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
         hipLaunchKernelGGL(experts_bf16_kernel<MODE_UPREC>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s,
                            (const bf16_t *)m->xg, (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a,
                            (void *)m->bw_h1, (void *)m->bw_h3, m->wq_up, c.H, c.d);
-    } else if (which == 0 && m->gather_on_load) {
-        // the loads of the product fetch the rows of x themselves: no gathered copy (and no packed copy for the shared experts)
-        if (wnt)
-            hipLaunchKernelGGL((experts_bf16_kernel<MODE_UP, true, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)x,
-                               (const bf16_t *)x, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
-                               (void *)nullptr, m->wq_up, c.H, c.d, m->tokp);
-        else
-            hipLaunchKernelGGL((experts_bf16_kernel<MODE_UP, false, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)x,
-                               (const bf16_t *)x, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
-                               (void *)nullptr, m->wq_up, c.H, c.d, m->tokp);
     } else if (which == 0) {
-        if (wnt)
-            hipLaunchKernelGGL((experts_bf16_kernel<MODE_UP, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
-                               (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
-                               (void *)nullptr, m->wq_up, c.H, c.d);
-        else
-            hipLaunchKernelGGL(experts_bf16_kernel<MODE_UP>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->xg,
-                               (const bf16_t *)m->xs, (const bf16_t *)m->W1, (const bf16_t *)m->W3, m->a, (void *)nullptr,
-                               (void *)nullptr, m->wq_up, c.H, c.d);
+        // the forward pass outside training: one wave per SIMD (experts_up4_kernel)
+        const bf16_t *A = (const bf16_t *)(m->gather_on_load ? x : m->xg), *As = (const bf16_t *)(m->gather_on_load ? x : m->xs);
+#define UP4_LAUNCH(WNTV, GV)                                                                                            \
+    hipLaunchKernelGGL((experts_up4_kernel<WNTV, GV>), dim3(m->n_wg), dim3(U4_WAVES * 64), SMEM_BYTES, s, A, As, (const bf16_t *)m->W1, \
+                       (const bf16_t *)m->W3, m->a, m->wq_up, c.H, c.d, m->tokp)
+        if (m->gather_on_load) {
+            if (wnt) UP4_LAUNCH(true, true);
+            else UP4_LAUNCH(false, true);
+        } else {
+            if (wnt) UP4_LAUNCH(true, false);
+            else UP4_LAUNCH(false, false);
+        }
+#undef UP4_LAUNCH
     } else {
         // the table may hold k slices (every tile of a small batch, or the last tiles of a large one): their partial
         // results go to y_slabs and are added into y right behind the product
