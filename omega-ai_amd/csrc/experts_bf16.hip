@@ -637,6 +637,8 @@ struct Up4Item {                // uniform over the wave unless said otherwise
     const unsigned char *B0, *B1;  // k step 0 of the 128 rows of W1 / of W3
     uint32_t va[4];             // per lane: what the lane adds to A for the wave's A loads (16-row blocks wave + 4 n)
     int row0, rows, n0;
+    int kt;                     // k steps of the item (even, at least 8)
+    int slab;                   // down product: 0 = the item writes the output, > 0 = partial result `slab`
 };
 
 // GATHER: token of tile row 16 * (wave + 4 n) + lane / 4, or 0 behind the item's rows
@@ -644,9 +646,11 @@ struct Up4Tok {
     int t[4];
 };
 
-template <bool GATHER>
+// DOWN: the plain product y = a . W2^T: 256 columns of W2 (W1 = W2, W3 unused), A = the packed a; an item may be a k
+// slice of a tile (a_rg slices, slice kt0, partial result xrow0: see make_ctx) - slices start on even k steps here
+template <bool GATHER, bool DOWN = false>
 __device__ __forceinline__ Up4Item up4_item(const omega_tile_desc &d, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *W1,
-                                            const bf16_t *W3, int N, int Kd, int wave, int lane, const Up4Tok &tk)
+                                            const bf16_t *W3, int N, int Kd, int wave, int lane, const Up4Tok &tk, bool slices = false)
 {
     Up4Item c;
     const int KT = Kd / BK;
@@ -654,7 +658,34 @@ __device__ __forceinline__ Up4Item up4_item(const omega_tile_desc &d, const bf16
     c.row0 = d.row0;
     c.rows = d.rows;
     c.n0 = d.n0;
+    c.kt = KT;
+    c.slab = 0;
     const size_t wrg = (size_t)d.g * (N >> 7) + (d.n0 >> 7);
+    if (DOWN) {
+        size_t k0 = 0;
+        if (d.a_rg > 1) {
+            if (slices) {
+                const int first = ((d.kt0 * KT) / d.a_rg) & ~1;
+                c.kt = (d.kt0 + 1 == d.a_rg ? KT : (((d.kt0 + 1) * KT) / d.a_rg) & ~1) - first;
+                c.slab = d.kt0 > 0 ? d.xrow0 : 0;
+                k0 = (size_t)first * 8192;
+            } else if (d.kt0 > 0) {
+                c.rows = 0;  // a launch without room for partial results: slice 0 computes the whole range
+            }
+        }
+        c.B0 = uniform_ptr((const unsigned char *)W1 + wrg * rg_bytes + k0);
+        c.B1 = uniform_ptr(c.B0 + rg_bytes);
+        c.A = uniform_ptr((const unsigned char *)Axg + (size_t)(d.row0 / BM * 2) * rg_bytes + k0);
+        const int blk0 = (d.row0 & (BM - 1)) >> 4;
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+            const int q = wave + 4 * n;
+            const bool valid = 16 * q < c.rows;
+            const int qa = blk0 + (valid ? q : 0);
+            c.va[n] = (uint32_t)(qa >> 3) * (uint32_t)rg_bytes + (uint32_t)(qa & 7) * 1024u + (valid ? (uint32_t)lane * 16u : 0u);
+        }
+        return c;
+    }
     c.B0 = uniform_ptr((const unsigned char *)W1 + wrg * rg_bytes);
     c.B1 = uniform_ptr((const unsigned char *)W3 + wrg * rg_bytes);
     if (GATHER) {
@@ -702,16 +733,16 @@ struct Up4State {
 
 // One work item for a wave with NU units of valid rows (units beyond them issue no MFMAs; the accumulators live for
 // one item, so every NU is its own straight-line code with NU * 32 accumulator registers).
-template <int NU, bool WNT, bool GATHER>
+template <int NU, bool WNT, bool GATHER, bool DOWN>
 __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, const Up4Item &it, Up4Item &nxt_it,
                                              const omega_tile_desc &dn, const bf16_t *Axg, const bf16_t *Ax, const bf16_t *W1,
-                                             const bf16_t *W3, void *Cout, int N, int Kd, int wave, int lane,
+                                             const bf16_t *W3, void *Cout, void *slabs, int N, int Kd, int wave, int lane,
                                              const int32_t *__restrict__ tokp)
 {
     constexpr int A_STEP = GATHER ? BK * 2 : 8192;
     constexpr int NA = NU > 0 ? NU : 1;
     const int wm = wave >> 1, wn = wave & 1;
-    const int KT = Kd / BK;
+    const int KT = DOWN ? __builtin_amdgcn_readfirstlane(it.kt) : Kd / BK;
     const int l16 = lane & 15, lq = lane >> 4;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     const uint32_t lds_wave = lds0 + wave * 1024;
@@ -719,13 +750,14 @@ __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, 
     const bool has_next = dn.rows > 0;
     // fragment addresses within a stage.  A fragment iu: rows of unit 2 iu + wm = block 2 iu + wm of the A tile; B fragment
     // c (16 MFMA columns): block (c / 4) * 8 + wn * 4 + c % 4 of the B tile, i.e. columns wn * 64 + 16 (c % 4) of the W1 half
-    // (c < 4) or of the W3 half, so that acc[.][c] and acc[.][c + 4] are h1 and h3 of the same elements.  Lane l supplies
-    // row l % 16, chunk l / 16; the chunk swizzle depends on the row through l % 16 and the block's parity.
+    // (c < 4) or of the W3 half, so that acc[.][c] and acc[.][c + 4] are h1 and h3 of the same elements (DOWN: block
+    // wn * 8 + c, columns wn * 128 + 16 c of the tile's 256).  Lane l supplies row l % 16, chunk l / 16; the chunk swizzle
+    // depends on the row through l % 16 and the block's parity.
     const uint32_t pa = (uint32_t)(wm * 16 + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | (wm << 4))) << 4);
     uint32_t pb[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h)
-        pb[h] = TILE_BYTES + (uint32_t)(wn * 64 + 16 * h + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | (h << 4))) << 4);
+        pb[h] = TILE_BYTES + (uint32_t)(wn * (DOWN ? 128 : 64) + 16 * h + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | (h << 4))) << 4);
     int cur = __builtin_amdgcn_readfirstlane(st.cur);
     const unsigned char *lA = uniform_ptr(st.lA), *lB0 = uniform_ptr(st.lB0), *lB1 = uniform_ptr(st.lB1);
 
@@ -741,13 +773,13 @@ __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, 
             asm volatile("global_load_dword %0, %1, %2" : "=&v"(ntk.t[n]) : "v"(o), "s"(tokp) : "memory");
         }
     }
-    if (!GATHER && has_next) nxt_it = up4_item<false>(dn, Axg, Ax, W1, W3, N, Kd, wave, lane, Up4Tok{});
+    if (!GATHER && has_next) nxt_it = up4_item<false, DOWN>(dn, Axg, Ax, W1, W3, N, Kd, wave, lane, Up4Tok{}, slabs != nullptr);
 
-#define U4_READ(FA, FB, stage, r)                                                                                       \
+// fragment read r (0..7: B fragment r, 8..15: A fragment r - 8) of the stage whose read addresses are ra / rb0 / rb1
+#define U4_READ(FA, FB, r)                                                                                              \
     do {                                                                                                                \
-        const unsigned char *sp = smem + (stage) * STAGE_BYTES;                                                         \
-        if ((r) < 8) FB[(r) & 7] = *(const bf16x8_t *)(sp + pb[(r) & 1] + (((r) & 3) >> 1) * 2048u + (((r) & 7) >> 2) * 8192u); \
-        else FA[((r) - 8) & 7] = *(const bf16x8_t *)(sp + pa + (((r) - 8) & 7) * 2048u);                                \
+        if ((r) < 8) FB[(r) & 7] = *(const bf16x8_t *)(((r) & 1 ? rb1 : rb0) + (DOWN ? (((r) & 7) >> 1) * 2048u : (((r) & 3) >> 1) * 2048u + (((r) & 7) >> 2) * 8192u)); \
+        else FA[((r) - 8) & 7] = *(const bf16x8_t *)(ra + (((r) - 8) & 7) * 2048u);                                     \
     } while (0)
 // the wave's direct load l (0..7) of a k step into the stage at LDS address sb: A blocks wave + 4 n, then the B blocks
 #define U4_LOAD(l, sb)                                                                                                  \
@@ -765,7 +797,8 @@ __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, 
 #define U4_MFMA(PA, PB, Z, iu, c)                                                                                       \
     do {                                                                                                                \
         if ((iu) < NU)                                                                                                  \
-            acc[(iu) % NA][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PB[c], PA[iu], (Z) ? zero4 : acc[(iu) % NA][c], 0, 0, 0); \
+            acc[(iu) % NA][c] = DOWN ? __builtin_amdgcn_mfma_f32_16x16x32_bf16(PA[iu], PB[c], (Z) ? zero4 : acc[(iu) % NA][c], 0, 0, 0) \
+                                     : __builtin_amdgcn_mfma_f32_16x16x32_bf16(PB[c], PA[iu], (Z) ? zero4 : acc[(iu) % NA][c], 0, 0, 0); \
     } while (0)
 // A wave issues one instruction every four cycles and an MFMA of this shape occupies the matrix core for sixteen: up
 // to three other instructions fit behind each MFMA without delaying the next one.  The order is pinned so: an MFMA,
@@ -774,8 +807,8 @@ __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, 
     do {                                                                                                                \
         U4_MFMA(PA, PB, Z, (g) >> 1, 4 * ((g) & 1));                                                                    \
         if ((g) < 8) {                                                                                                  \
-            U4_READ(QA, QB, nxt, 2 * (g));                                                                              \
-            U4_READ(QA, QB, nxt, 2 * (g) + 1);                                                                          \
+            U4_READ(QA, QB, 2 * (g));                                                                                   \
+            U4_READ(QA, QB, 2 * (g) + 1);                                                                               \
         }                                                                                                               \
         __builtin_amdgcn_sched_barrier(0);                                                                              \
         U4_MFMA(PA, PB, Z, (g) >> 1, 4 * ((g) & 1) + 1);                                                                \
@@ -786,24 +819,48 @@ __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, 
         U4_MFMA(PA, PB, Z, (g) >> 1, 4 * ((g) & 1) + 3);                                                                \
         __builtin_amdgcn_sched_barrier(0);                                                                              \
     } while (0)
+// (the last group of a step also moves the ring on - the stage the next step's loads go to, the addresses its
+//  fragment reads come from, the load pointers - behind its MFMAs, so that the step after the barrier starts with work)
 #define U4_STEP(PA, PB, QA, QB, Z)                                                                                      \
     do {                                                                                                                \
-        const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;                                                                \
-        const uint32_t sb = lds_wave + cur * STAGE_BYTES;                                                               \
         U4_GROUP(PA, PB, QA, QB, Z, 0); U4_GROUP(PA, PB, QA, QB, Z, 1); U4_GROUP(PA, PB, QA, QB, Z, 2);                 \
         U4_GROUP(PA, PB, QA, QB, Z, 3); U4_GROUP(PA, PB, QA, QB, Z, 4); U4_GROUP(PA, PB, QA, QB, Z, 5);                 \
         U4_GROUP(PA, PB, QA, QB, Z, 6); U4_GROUP(PA, PB, QA, QB, Z, 7); U4_GROUP(PA, PB, QA, QB, Z, 8);                 \
         U4_GROUP(PA, PB, QA, QB, Z, 9); U4_GROUP(PA, PB, QA, QB, Z, 10); U4_GROUP(PA, PB, QA, QB, Z, 11);               \
         U4_GROUP(PA, PB, QA, QB, Z, 12); U4_GROUP(PA, PB, QA, QB, Z, 13); U4_GROUP(PA, PB, QA, QB, Z, 14);              \
-        U4_GROUP(PA, PB, QA, QB, Z, 15);                                                                                \
+        U4_MFMA(PA, PB, Z, 7, 4);                                                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+        U4_MFMA(PA, PB, Z, 7, 5);                                                                                       \
+        U4_LOAD(7, sb);                                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+        U4_MFMA(PA, PB, Z, 7, 6);                                                                                       \
+        cur = cur + 1 == NSTAGE ? 0 : cur + 1;                                                                          \
+        sb = lds_wave + cur * STAGE_BYTES;                                                                              \
         lA += A_STEP;                                                                                                   \
         lB0 += 8192;                                                                                                    \
         lB1 += 8192;                                                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
+        U4_MFMA(PA, PB, Z, 7, 7);                                                                                       \
+        {                                                                                                               \
+            const unsigned char *sn = smem + (cur + 1 == NSTAGE ? 0 : cur + 1) * STAGE_BYTES;                           \
+            ra = sn + pa;                                                                                               \
+            rb0 = sn + pb[0];                                                                                           \
+            rb1 = sn + pb[1];                                                                                           \
+        }                                                                                                               \
+        __builtin_amdgcn_sched_barrier(0);                                                                              \
         asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");                                                    \
         __syncthreads();                                                                                                \
-        cur = nxt;                                                                                                      \
     } while (0)
 
+    // the stage this step's loads go to and the addresses the fragments of the next step are read from
+    uint32_t sb = lds_wave + cur * STAGE_BYTES;
+    const unsigned char *ra, *rb0, *rb1;
+    {
+        const unsigned char *sn = smem + (cur + 1 == NSTAGE ? 0 : cur + 1) * STAGE_BYTES;
+        ra = sn + pa;
+        rb0 = sn + pb[0];
+        rb1 = sn + pb[1];
+    }
     f32x4_t acc[NA][8];  // acc[iu][c]: 16 x 16 piece (rows of unit 2 iu + wm, columns of B fragment c), weights as first operand
     const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
     // KT steps (even, at least 8), two at a time.  The loads issued during steps 0 .. KT - 6 are the item's own (its steps
@@ -820,7 +877,7 @@ __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, 
         // three steps or more have passed since the token loads were issued: they have landed
         asm volatile("; token loads done" : "+v"(ntk.t[0]), "+v"(ntk.t[1]), "+v"(ntk.t[2]), "+v"(ntk.t[3])::"memory");
         if (dn.xrow0 >= 0) ntk = up4_tokens(dn, tokp, wave, lane);
-        nxt_it = up4_item<true>(dn, Axg, Ax, W1, W3, N, Kd, wave, lane, ntk);
+        nxt_it = up4_item<true, false>(dn, Axg, Ax, W1, W3, N, Kd, wave, lane, ntk);
     }
     lA = uniform_ptr(nxt_it.A);
     lB0 = uniform_ptr(nxt_it.B0);
@@ -841,6 +898,30 @@ __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, 
     st.lB0 = lB0;
     st.lB1 = lB1;
 
+    if (DOWN) {
+        // ---- epilogue of the plain product: fp32 rows (a k slice other than the first: partial result it.slab, a tile of
+        // BM x 256 of its own).  The rows were the MFMAs' first operand: lane l holds column l % 16 of the 16 of fragment c,
+        // register r row 4 (l / 16) + r of the unit, so 16 lanes store 64 consecutive bytes of a row
+        float *Cbase = (float *)Cout + (size_t)it.row0 * N + it.n0;
+        int ld = N;
+        if (it.slab > 0) {
+            Cbase = (float *)slabs + (size_t)it.slab * (BM * 256);
+            ld = 256;
+        }
+#pragma unroll
+        for (int iu = 0; iu < NU; ++iu) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = 16 * (2 * iu + wm) + 4 * lq + r;
+                if (row < it.rows) {
+                    float *out = Cbase + (size_t)row * ld + wn * 128 + l16;
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) out[16 * c] = acc[iu][c][r];
+                }
+            }
+        }
+        return;
+    }
     // ---- epilogue: a = silu(h1) * h3 as packed bf16 ----
     // lane: row l16 of unit 2 iu + wm; registers r of acc[iu][c] and acc[iu][c + 4]: h1 and h3 of column
     // wn * 64 + 16 c + 4 lq + r of the tile's 128, i.e. k step n0 / 32 + 2 wn + c / 2 of the packed a, chunk 2 (c % 2) + lq / 2
@@ -866,11 +947,13 @@ __device__ __forceinline__ void up4_run_item(unsigned char *smem, Up4State &st, 
     }
 }
 
-template <bool WNT, bool GATHER>
+// DOWN: the plain down product on the same kernel (W1 = W2, slabs = room for the partial results of k slices or null)
+template <bool WNT, bool GATHER, bool DOWN = false>
 __global__ __launch_bounds__(U4_WAVES * 64) void experts_up4_kernel(const bf16_t *__restrict__ Axg, const bf16_t *__restrict__ Ax,
                                                                     const bf16_t *__restrict__ W1, const bf16_t *__restrict__ W3,
                                                                     void *__restrict__ Cout, const omega_tile_desc *__restrict__ wq,
-                                                                    int N, int Kd, const int32_t *__restrict__ tokp)
+                                                                    int N, int Kd, const int32_t *__restrict__ tokp,
+                                                                    void *slabs = nullptr)
 {
     constexpr int A_STEP = GATHER ? BK * 2 : 8192;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -885,7 +968,8 @@ __global__ __launch_bounds__(U4_WAVES * 64) void experts_up4_kernel(const bf16_t
 
     omega_tile_desc d = wq[wg];
     if (d.rows <= 0) return;
-    Up4Item it = up4_item<GATHER>(d, Axg, Ax, W1, W3, N, Kd, wave, lane, GATHER ? up4_tokens(d, tokp, wave, lane) : Up4Tok{});
+    Up4Item it = up4_item<GATHER, DOWN>(d, Axg, Ax, W1, W3, N, Kd, wave, lane, GATHER ? up4_tokens(d, tokp, wave, lane) : Up4Tok{},
+                                        slabs != nullptr);
     Up4State st;
     st.lA = it.A;
     st.lB0 = it.B0;
@@ -920,8 +1004,8 @@ __global__ __launch_bounds__(U4_WAVES * 64) void experts_up4_kernel(const bf16_t
         const uint32_t pa = (uint32_t)(wm * 16 + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | (wm << 4))) << 4);
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-            const uint32_t pbr = TILE_BYTES + (uint32_t)(wn * 64 + 16 * (r & 1) + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | ((r & 1) << 4))) << 4);
-            st.fb0[r] = *(const bf16x8_t *)(smem + pbr + ((r & 3) >> 1) * 2048u + (r >> 2) * 8192u);
+            const uint32_t pbr = TILE_BYTES + (uint32_t)(wn * (DOWN ? 128 : 64) + 16 * (r & 1) + l16) * (BK * 2) + ((uint32_t)(lq ^ swz(l16 | ((r & 1) << 4))) << 4);
+            st.fb0[r] = *(const bf16x8_t *)(smem + pbr + (DOWN ? (r >> 1) * 2048u : ((r & 3) >> 1) * 2048u + (r >> 2) * 8192u));
             st.fa0[r] = *(const bf16x8_t *)(smem + pa + r * 2048u);
         }
     }
@@ -936,7 +1020,7 @@ __global__ __launch_bounds__(U4_WAVES * 64) void experts_up4_kernel(const bf16_t
         const int units = (it.rows + 15) >> 4;
         const int nu = __builtin_amdgcn_readfirstlane(max(0, min(8, (units + 1 - wm) >> 1)));
         Up4Item nxt_it = it;
-#define U4_RUN(NU) up4_run_item<NU, WNT, GATHER>(smem, st, it, nxt_it, dn, Axg, Ax, W1, W3, Cout, N, Kd, wave, lane, tokp)
+#define U4_RUN(NU) up4_run_item<NU, WNT, GATHER, DOWN>(smem, st, it, nxt_it, dn, Axg, Ax, W1, W3, Cout, slabs, N, Kd, wave, lane, tokp)
         switch (nu) {
             case 8: U4_RUN(8); break;
             case 7: U4_RUN(7); break;
@@ -1014,7 +1098,8 @@ hipError_t experts_bf16_init(void)
                          (const void *)experts_bf16_kernel<MODE_WGRAD>, (const void *)experts_bf16_kernel<MODE_UPREC>,
                          (const void *)experts_bf16_kernel<MODE_UP, true>, (const void *)experts_bf16_kernel<MODE_DOWN, true>,
                          (const void *)experts_up4_kernel<false, false>, (const void *)experts_up4_kernel<true, false>,
-                         (const void *)experts_up4_kernel<false, true>, (const void *)experts_up4_kernel<true, true>};
+                         (const void *)experts_up4_kernel<false, true>, (const void *)experts_up4_kernel<true, true>,
+                         (const void *)experts_up4_kernel<false, false, true>, (const void *)experts_up4_kernel<true, false, true>};
     for (const void *f : fns) {
         hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
         if (e != hipSuccess) return e;
@@ -1055,7 +1140,17 @@ hipError_t launch_experts_bf16(const omega_moe *m, const void *x, int T, int whi
         // the table may hold k slices (every tile of a small batch, or the last tiles of a large one): their partial
         // results go to y_slabs and are added into y right behind the product
         void *slabs = (m->down_ks_max > 1 || m->down_tail_ks > 1) ? (void *)m->y_slabs : nullptr;
-        if (wnt)
+        if (m->down_cols == 256) {
+            // full-width items: one wave per SIMD (experts_up4_kernel, DOWN)
+            if (wnt)
+                hipLaunchKernelGGL((experts_up4_kernel<true, false, true>), dim3(m->n_wg), dim3(U4_WAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
+                                   (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y, m->wq_down, c.d,
+                                   c.H, (const int32_t *)nullptr, slabs);
+            else
+                hipLaunchKernelGGL((experts_up4_kernel<false, false, true>), dim3(m->n_wg), dim3(U4_WAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
+                                   (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y, m->wq_down, c.d,
+                                   c.H, (const int32_t *)nullptr, slabs);
+        } else if (wnt)
             hipLaunchKernelGGL((experts_bf16_kernel<MODE_DOWN, true>), dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)m->a,
                                (const bf16_t *)nullptr, (const bf16_t *)m->W2, (const bf16_t *)nullptr, (void *)m->y,
                                slabs, (void *)nullptr, m->wq_down, c.d, c.H);
@@ -1077,6 +1172,13 @@ hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, cons
                                void *Cout, void *Aux1, void *Aux2, const omega_tile_desc *wq, int N, int Kd, hipStream_t s)
 {
     if (Kd < (NSTAGE + 1) * BK) return hipErrorInvalidValue;
+    if (mode == MODE_DOWN && m->down_cols == 256 && Kd % 64 == 0 && Kd >= 8 * BK) {
+        // plain full-width products (the input gradient of the experts): one wave per SIMD
+        hipLaunchKernelGGL((experts_up4_kernel<false, false, true>), dim3(m->n_wg), dim3(U4_WAVES * 64), SMEM_BYTES, s, (const bf16_t *)A,
+                           (const bf16_t *)nullptr, (const bf16_t *)Wa, (const bf16_t *)nullptr, Cout, wq, N, Kd, (const int32_t *)nullptr,
+                           Aux1);
+        return hipGetLastError();
+    }
 #define LAUNCH(MODE)                                                                                                   \
     hipLaunchKernelGGL(experts_bf16_kernel<MODE>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)A,      \
                        (const bf16_t *)Aalt, (const bf16_t *)Wa, (const bf16_t *)Wb, Cout, Aux1, Aux2, wq, N, Kd)
