@@ -146,11 +146,11 @@ hipError_t launch_combine(const omega_moe *m, int T, void *out, const void *resi
     const int vec = bf ? 8 : 4;
     if (c.d % vec == 0 && (((uintptr_t)out | (uintptr_t)resid) % 16) == 0 && c.K <= MAXK) {
         const bool nt = (size_t)T * (c.K + c.Es) * c.d * 4 > OMEGA_LLC_BYTES;
-        // few tokens for the compute units there are: several waves per token, each with a share of the columns, until
-        // the launch has 64 waves per compute unit (4096 tokens x 4096 columns: 36.3 -> 33.0 us with 4 waves per token,
-        // 64 tokens: 12.0 -> 6.9 us with 8)
+        // several waves per token, each with a share of the columns, until the launch has 256 waves per compute unit:
+        // more loads in flight (4096 tokens x 4096 columns: 36.3 -> 30.6 us with 8 waves per token; 64 tokens:
+        // 12.0 -> 6.9 us; 8192 tokens x 2048 columns x 8 rows: 122.6 -> 113.8 us with 4; 16384 tokens: 228 -> 210 us)
         int split = 1;
-        while (split < 8 && (long long)T * split < 64LL * m->ctx->num_cus && c.d % (64 * vec * split * 2) == 0) split *= 2;
+        while (split < 8 && (long long)T * split < 256LL * m->ctx->num_cus && c.d % (64 * vec * split * 2) == 0) split *= 2;
 #define COMBINE_LAUNCH2(KUV, NTV)                                                                                      \
     do {                                                                                                              \
         if (bf)                                                                                                       \
