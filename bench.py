@@ -198,7 +198,7 @@ def main():
         "config": {"workload": f"{cfg.name}: T={cfg.T} ({cfg.batch}x{cfg.seq}) d={cfg.d} E={cfg.E} K={cfg.K} H={cfg.H} "
                                f"Es={cfg.Es} renorm={int(cfg.renorm)} {cfg.dtype}, fp32 accumulate",
                    "router_mode": a.router, "seed": a.seed},
-        "roofline": {"bound": "mfma", "kernel": "experts_bf16_kernel<0> (up): a = silu(xg W1^T) * (xg W3^T)",
+        "roofline": {"bound": "mfma", "kernel": ("experts_up4_kernel" if cfg.dtype == "bf16" else "experts_f32_kernel<true>") + " (up product): a = silu(xg W1^T) * (xg W3^T)",
                      "achieved": up_tflops, "peak": peak, "unit": "TFLOP/s", "frac": up_tflops / peak,
                      "algorithmic_flops_per_launch": up_flops, "avg_launch_ms": stage_ms["experts_up"],
                      "traffic": traffic, "traffic_source": traffic_src,
