@@ -5,22 +5,26 @@
 // (J/engine/nn/layer/llama/LlamaMLPLayer.java:117-130; y = x W^T with W [out,in], J/engine/nn/layer/FullyLayer.java:181,235.)
 //
 // Both operands are K-contiguous ("NT" product), so a lane's 8 consecutive k values are one 16-byte LDS read.
-// Workgroup = 8 waves (2 row halves x 4 column quarters, two waves per SIMD so that one computes while the
-// other waits on LDS, on the address unit, at the barrier or through its item switch: four waves of 128 x 128, one
-// per SIMD, read a third fewer fragments and were 2-3 % faster on long full tiles, but lost twice as much per item
-// and more on ragged tiles and short items); tile = 256 rows x 256 MFMA columns, each wave
-// 4x2 MFMA blocks (the 32-row blocks of the tile alternate between the row halves, so a ragged tile splits evenly) with
-// 128 accumulator registers (of the 256 a wave has at two waves per SIMD).  For the up product the 256 MFMA columns are
-// 128 columns of W1 and the same 128 columns of W3, arranged so that a wave holds h1 and h3 of the same
-// output element and applies silu(h1)*h3 in registers.
+// Tile = 256 rows x 256 MFMA columns; for the up product the 256 MFMA columns are 128 columns of W1 and the same 128
+// columns of W3, arranged so that a wave holds h1 and h3 of the same output element and applies silu(h1)*h3 in
+// registers.  Two kernels share everything below except the shape of a workgroup:
+//   experts_up4_kernel   four waves of 128 x 128, one per SIMD, 256 accumulator registers each (AGPRs), 16 fragment
+//                        reads per 64 MFMAs, the instruction order of a k step pinned (a lone wave issues one instruction
+//                        every four cycles, an MFMA occupies the matrix core for sixteen).  The forward pass's up
+//                        product (it can fetch its rows from x through the row -> token table), the down product with
+//                        256-column items and the backward pass's input-gradient product: 2-3 % faster than eight waves.
+//   experts_bf16_kernel  eight waves (2 row halves x 4 column quarters, two per SIMD, 128 accumulator registers each;
+//                        the 32-row blocks of the tile alternate between the row halves, so a ragged tile splits
+//                        evenly): the products that keep or read h1 / h3 records, the weight gradients, and down
+//                        products with 128-column items.
 //
 // Data movement: global -> LDS directly (global_load_lds_dwordx4, no staging registers) into a ring of five
 // stages of (A 256x32 + B 256x32) bf16 = 160 KiB, i.e. all of a CU's LDS.  A wave-wide direct load fills 1 KiB
 // of LDS in lane order = 16 rows of four 16-byte chunks.  All three operands (weights, xg, a) are kept in
 // memory as that very image (pack.h: 1 KiB blocks of 16 rows x 32 k with the chunk index XOR-swizzled so the
 // MFMA operand reads are free of bank conflicts), so every direct load reads 1 KiB of contiguous memory.
-// The weights are packed once when they are set, xg by the gather kernel, a by the up product's epilogue.
-// Pipeline per 32-k step and wave: two phases of 16 MFMAs; the fragments of the next phase are read from LDS
+// The weights are packed once when they are set, xg by the dispatch launch, a by the up product's epilogue.
+// Pipeline per 32-k step and wave (eight waves): two phases of 16 MFMAs; the fragments of the next phase are read from LDS
 // while the current one computes; one barrier per step, after which the stage just read is refilled with the
 // step five ahead; four direct loads per wave and step.  Every step of every item is the same code (the addresses the
 // loads read from next sit in scalar registers and are switched to the next item when its turn comes), and the bulk of
