@@ -159,7 +159,7 @@ struct omega_moe {
     size_t prof_used = 0;
 };
 
-// Tokens per router workgroup = per row of tile_counts / tile_base and per workgroup of the rank kernel: 16 for layers
+// Tokens per router workgroup = per row of tile_counts and per workgroup of the dispatch kernel: 16 for layers
 // with at most 16 experts, else 32 (router.hip).
 int router_tok_tile(int E);
 #define ROUTER_TOK_TILE_MAX 32
