@@ -1097,10 +1097,11 @@ hipError_t launch_down_slab_reduce(const omega_moe *m, float *y, hipStream_t s)
 
 hipError_t experts_bf16_init(void)
 {
-    const void *fns[] = {(const void *)experts_bf16_kernel<MODE_UP>, (const void *)experts_bf16_kernel<MODE_DOWN>,
+    // (the plain up product runs on experts_up4_kernel only: the eight-wave kernel is not instantiated for it)
+    const void *fns[] = {(const void *)experts_bf16_kernel<MODE_DOWN>,
                          (const void *)experts_bf16_kernel<MODE_UPRAW>, (const void *)experts_bf16_kernel<MODE_DA>,
                          (const void *)experts_bf16_kernel<MODE_WGRAD>, (const void *)experts_bf16_kernel<MODE_UPREC>,
-                         (const void *)experts_bf16_kernel<MODE_UP, true>, (const void *)experts_bf16_kernel<MODE_DOWN, true>,
+                         (const void *)experts_bf16_kernel<MODE_DOWN, true>,
                          (const void *)experts_up4_kernel<false, false>, (const void *)experts_up4_kernel<true, false>,
                          (const void *)experts_up4_kernel<false, true>, (const void *)experts_up4_kernel<true, true>,
                          (const void *)experts_up4_kernel<false, false, true>, (const void *)experts_up4_kernel<true, false, true>};
@@ -1187,7 +1188,6 @@ hipError_t launch_product_bf16(const omega_moe *m, int mode, const void *A, cons
     hipLaunchKernelGGL(experts_bf16_kernel<MODE>, dim3(m->n_wg), dim3(NWAVES * 64), SMEM_BYTES, s, (const bf16_t *)A,      \
                        (const bf16_t *)Aalt, (const bf16_t *)Wa, (const bf16_t *)Wb, Cout, Aux1, Aux2, wq, N, Kd)
     switch (mode) {
-        case MODE_UP: LAUNCH(MODE_UP); break;
         case MODE_DOWN: LAUNCH(MODE_DOWN); break;
         case MODE_UPRAW: LAUNCH(MODE_UPRAW); break;
         case MODE_DA: LAUNCH(MODE_DA); break;
