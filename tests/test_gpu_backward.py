@@ -152,6 +152,33 @@ def test_backward_bf16_matches_oracle(name, kw):
     layer.close()
 
 
+@pytest.mark.parametrize("name,kw,block", [
+    ("c2_mixtral", dict(T=300, d=256, H=384), False),
+    ("c4_finegrained", dict(T=200, d=256, H=256, E=16, K=4, Es=2), True),     # shared experts, block form
+    ("c5_skewed", dict(T=257, d=512, H=256, E=32, K=4), False),               # experts without rows
+])
+def test_backward_bf16_same_bits_in_both_gather_modes(name, kw, block):
+    """A backward pass needs the gathered rows of x.  When the forward pass left them to the loads of the up product
+    (omega_moe_set_gather_mode ON_LOAD) the copy is made on demand: input gradient and every parameter gradient carry
+    the same bits as after a forward pass that wrote the copy itself, in the plain and in the block form."""
+    G, cfg, inp, dout, layer = _setup(name, kw, 53)
+    if block:
+        layer.set_norm((1.0 + 0.1 * O.fill_normal(cfg.d, 17, 901, 1.0)).astype(np.float32))
+    x = G.P.DeviceBuffer.from_numpy(G.ctx(), inp["x"], cfg.dtype)
+    g = G.P.DeviceBuffer.from_numpy(G.ctx(), dout, cfg.dtype)
+    got = {}
+    for mode in (1, 2):
+        layer.set_gather_mode(mode)
+        out = (layer.forward_block(x) if block else layer.forward(x)).to_numpy()
+        assert layer.gather_on_load() == (mode == 2)
+        dx = (layer.back_block(g) if block else layer.back(g)).to_numpy()
+        got[mode] = [out, dx] + _all_grads(layer, cfg, block)
+    assert len(got[1]) == len(got[2])
+    for a, b in zip(got[1], got[2]):
+        assert np.array_equal(a, b)
+    layer.close()
+
+
 def test_backward_full_size_mixtral():
     """C2 at full size.  Rows of a token depend on that token only: input gradient and dlogits of sampled tokens against
     the oracle (with the experts those tokens use).  Weight gradients of every expert through bilinear probes:
